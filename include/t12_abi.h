@@ -1,0 +1,143 @@
+/*
+ * t12_abi.h -- C ABI of libturbo12.so: split-12 fused decode + GEMV / GEMM,
+ * standalone decompress and the engine glue kernels, hand-written for gfx950.
+ *
+ * Conventions (the same as the reference's launch layer, engine/inference.cpp:7-41):
+ * extern "C", plain device pointers and sizes, the HIP stream passed as an
+ * opaque pointer, launches are asynchronous on that stream, no ownership is
+ * transferred.  Unlike the reference every entry point validates its operands
+ * on the host and checks the launch; the return value is 0 on success and a
+ * negative T12_E* code otherwise (t12_last_error() gives the text).
+ *
+ * Data layout (byte-exact with what split12_pack.c:47-128 emits):
+ *   sm   u8  [M*K]        (sign << 7) | mantissa7, row-major
+ *   gr   u8  [(M*K+1)/2]  4-bit group per element, flat index i -> byte i/2,
+ *                         low nibble for even i; group = exponent - base_exp in
+ *                         1..15, 0 = escape
+ *   CSR  row_off i32[M+1], cols i32[P] (ascending in a row), correct i16[P]
+ *        (exact bf16 bits), wrong i16[P] (what the plain rule yields for group 0)
+ *   activations  bf16 [B, K] row-major (row stride act_stride elements)
+ *   outputs      fp32 out[b * out_stride + m]
+ */
+#ifndef T12_ABI_H
+#define T12_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define T12_OK          0
+#define T12_EINVAL     (-1)   /* bad shape / null pointer / unsupported size */
+#define T12_ELAUNCH    (-2)   /* HIP reported a launch or runtime error      */
+#define T12_MAX_SEGMENTS 8
+
+/* One weight tensor of a fused launch.  Several tensors that consume the same
+ * activations (wq|wk|wv, gate|up, the experts of one token group) are passed as
+ * a segment table so that one launch fills the whole chip; each keeps its own
+ * base_exp (replaces the pair of base_exp arguments of
+ * launch_split12_v2_dual_async, decompress_v2.hip:549, and the
+ * PatchBatchDesc table of decompress_v2.hip:36-44).  All pointers are device
+ * pointers.  row_off == NULL means "no escape list": group-0 elements then
+ * decode to the wrong value, exactly like the reference's unpatched kernels. */
+typedef struct T12Segment {
+    const uint8_t* sm;
+    const uint8_t* gr;
+    const int32_t* row_off;
+    const int32_t* cols;
+    const int16_t* correct;
+    const int16_t* wrong;
+    float*         out;        /* this tensor's output base: out[b*out_stride + m] */
+    int32_t        M;
+    int32_t        base_exp;
+} T12Segment;
+
+/* ---- library ------------------------------------------------------------- */
+const char* t12_version(void);
+const char* t12_last_error(void);      /* text of the last failure on this thread */
+
+/* ---- calibration kernels (no counterpart in the reference) ------------------
+ * Plain streaming read / copy of `bytes` (a multiple of 16) with `blocks`
+ * workgroups of 256 lanes: the yardstick for achieved HBM bandwidth and for the
+ * profiler's FETCH_SIZE / WRITE_SIZE counters.  `sink` holds blocks x u32. */
+int t12_util_read(const void* src, size_t bytes, void* sink, int blocks, void* stream);
+int t12_util_copy(void* dst, const void* src, size_t bytes, int blocks, void* stream);
+/* Pins the B = 1 kernel variant (100*waves + 10*rows_per_wave + ring depth);
+ * 0 restores the choice by shape.  For benchmark sweeps. */
+int t12_tune_gemv(int variant);
+
+/* ---- (a) decode-GEMV, one activation vector ------------------------------
+ * out_s[m] = sum_k dec(W_s[m,k]) * x[k] for every segment s, escapes exact.
+ * Replaces launch_split12_v2_async (decompress_v2.hip:530) +
+ * launch_split12_v2_dual_async (:549) + launch_patches_v2_async (:113) +
+ * launch_patches_b1_batched_async (:129) with one launch.  `segs` is a HOST
+ * array (it travels as a kernel argument; no device copy is made). */
+int t12_gemv(const T12Segment* segs, int nseg, const void* act_bf16, int K, void* stream);
+
+/* ---- (a') small-batch decode-GEMV, 1 <= B <= 8 ----------------------------
+ * Same as t12_gemm but guaranteed to take the bandwidth-bound vector path.
+ * Replaces launch_split12_batch4_async / _batch8_async (decompress_v2.hip:860,877). */
+int t12_gemv_batch(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride,
+                   int out_stride, int K, int B, void* stream);
+
+/* ---- (b) decode+GEMM, any B >= 1 ------------------------------------------
+ * out_s[b*out_stride + m] = sum_k dec(W_s[m,k]) * X[b*act_stride + k], bf16 MFMA with
+ * fp32 accumulation for B > 8, escapes exact.  Replaces
+ * nv_launch_split12_fused_gemm_async (nvidia_kernels.cu:444) +
+ * nv_launch_patches_batch_async (:426) + nv_launch_split12_cublas_batch_async (:550). */
+int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride,
+             int out_stride, int K, int B, void* stream);
+
+/* ---- (c) standalone decompress --------------------------------------------
+ * out_bf16[m*K + k] = decoded weight bits.  patched != 0: escapes take
+ * `correct` (lossless, bit-exact with the tensor that was packed).
+ * patched == 0 (or row_off NULL): the reference's nv_decode_split12_to_bf16
+ * semantics (nvidia_kernels.cu:533-548): escapes keep the wrong value. */
+int t12_decompress(const void* sm, const void* gr, int base_exp, const void* row_off,
+                   const void* cols, const void* correct, void* out_bf16,
+                   int M, int K, int patched, void* stream);
+
+/* ---- reference-named launchers (same signatures and semantics) -------------
+ * For host code written against the reference's launch layer.
+ * decompress_v2.hip:530,549,113,129,860,877 */
+int launch_split12_v2_async(const void* sign_mantissa, const void* groups, int base_exp,
+                            const void* activations, void* output, int M, int K, void* stream);
+int launch_split12_v2_dual_async(const void* sm_a, const void* gr_a, int base_exp_a,
+                                 const void* sm_b, const void* gr_b, int base_exp_b,
+                                 const void* activations, void* output_a, void* output_b,
+                                 int M, int K, void* stream);
+int launch_patches_v2_async(const void* row_offsets, const void* patch_cols, const void* correct_vals,
+                            const void* wrong_vals, const void* activations, void* output, int M,
+                            void* stream);
+int launch_patches_v2(const void* row_offsets, const void* patch_cols, const void* correct_vals,
+                      const void* wrong_vals, const void* activations, void* output, int M);
+
+/* Must match the reference's PatchBatchDesc (decompress_v2.hip:36-44): 56 bytes. */
+typedef struct PatchBatchDesc {
+    const int32_t* row_offsets;
+    const int32_t* patch_cols;
+    const int16_t* patch_correct;
+    const int16_t* patch_wrong;
+    const int16_t* activations;
+    float*         output;
+    int            M;
+} PatchBatchDesc;
+int launch_patches_b1_batched_async(void* descs_gpu, const void* descs_cpu, int num_descs,
+                                    int max_M, void* stream);
+int launch_split12_batch4_async(const void* sm, const void* gr, int base_exp,
+                                const void* a0, const void* a1, const void* a2, const void* a3,
+                                const void* esc_row_base, const void* esc_counts, const void* esc_vals,
+                                void* o0, void* o1, void* o2, void* o3, int M, int K, void* stream);
+int launch_split12_batch8_async(const void* sm, const void* gr, int base_exp,
+                                const void* a0, const void* a1, const void* a2, const void* a3,
+                                const void* a4, const void* a5, const void* a6, const void* a7,
+                                const void* esc_row_base, const void* esc_counts, const void* esc_vals,
+                                void* o0, void* o1, void* o2, void* o3,
+                                void* o4, void* o5, void* o6, void* o7, int M, int K, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* T12_ABI_H */

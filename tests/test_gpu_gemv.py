@@ -1,0 +1,197 @@
+"""GPU parity: split-12 decode-GEMV (B = 1) through the C ABI vs the CPU oracle.
+
+Tolerance: BASELINE north star -- outputs within 1e-2 relative of the
+decode-then-fp32-accumulate reference.  The kernels accumulate in fp32 like the
+oracle, so the observed error is ~1e-6; the assertions use 1e-4 to catch a wrong
+pairing / dropped tile, which would show at 1e-2..1.
+"""
+import importlib
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import dev, rel_err, to_dev_bits
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def synth(t12):
+    return importlib.import_module("turbo_lossless_amd.synth")
+
+
+def run_gemv(t12, packs, x, patched=True):
+    dts = [t12.DeviceTensor12.from_packed(p, dev()) for p in packs]
+    outs = t12.gemv(dts, to_dev_bits(x), patched=patched)
+    torch.cuda.synchronize()
+    return [o.cpu().numpy() for o in outs]
+
+
+@pytest.mark.parametrize("M,K", [(4096, 4096), (1024, 4096), (256, 14336), (300, 1280), (77, 5120),
+                                 (1, 1024), (9, 16), (64, 1040), (5, 2064)])
+def test_gemv_llm_law(t12, oracle, synth, M, K):
+    w = synth.weights_llm(M, K, seed=1001 + M + K, p_outlier=3e-4 if M * K > 1e5 else 2e-2)
+    x = synth.activations(1, K, seed=1002)[0]
+    p = oracle.pack(w)
+    (got,) = run_gemv(t12, [p], x)
+    assert rel_err(got, oracle.gemv(p, x)) < TOL
+
+
+def test_gemv_config1_escape_statistics(t12, oracle, synth):
+    """BASELINE config 1: 4096x4096 N(0,.02) + 0.03 % N(0,8) outliers."""
+    w = synth.weights_llm(4096, 4096, seed=1001)
+    x = synth.activations(1, 4096, seed=1002)[0]
+    p = oracle.pack(w)
+    assert p.base_exp == 108 and 0.0003 < p.P / w.size < 0.0007
+    (got,) = run_gemv(t12, [p], x)
+    ref = oracle.gemv(p, x)
+    assert rel_err(got, ref) < TOL
+    # escapes matter: dropping the patch list must be visible
+    (un,) = run_gemv(t12, [p], x, patched=False)
+    assert rel_err(un, oracle.gemv(p, x, patched=False)) < TOL
+    assert rel_err(un, ref) > 1e-2
+
+
+def test_gemv_escape_heavy(t12, oracle, synth):
+    """BASELINE config 3 law: every row holds several escapes."""
+    for (M, K) in [(1280, 5120), (640, 1280)]:
+        w = synth.weights_diffusion(M, K, seed=3000 + M)
+        x = synth.activations(1, K, seed=3001)[0]
+        p = oracle.pack(w)
+        assert p.P > 2 * M and (K < 5120 or np.all(np.diff(p.row_off) > 0))
+        (got,) = run_gemv(t12, [p], x)
+        assert rel_err(got, oracle.gemv(p, x)) < TOL
+
+
+def test_gemv_fused_segments(t12, oracle, synth):
+    """wq|wk|wv in one launch: three tensors, three base_exp, one activation vector."""
+    K = 2048
+    ws = [synth.weights_llm(512, K, seed=1, sigma=0.02), synth.weights_llm(130, K, seed=2, sigma=0.3),
+          synth.weights_llm(128, K, seed=3, sigma=0.002)]
+    x = synth.activations(1, K, seed=4)[0]
+    ps = [oracle.pack(w) for w in ws]
+    assert len({p.base_exp for p in ps}) == 3
+    gots = run_gemv(t12, ps, x)
+    for g, p in zip(gots, ps):
+        assert rel_err(g, oracle.gemv(p, x)) < TOL
+
+
+def test_gemv_eight_segments(t12, oracle, synth):
+    K = 1024
+    ps = [oracle.pack(synth.weights_llm(8 + 3 * i, K, seed=10 + i, sigma=0.01 * (i + 1))) for i in range(8)]
+    x = synth.activations(1, K, seed=5)[0]
+    for g, p in zip(run_gemv(t12, ps, x), ps):
+        assert rel_err(g, oracle.gemv(p, x)) < TOL
+
+
+def test_gemv_general_path(t12, oracle, synth, golden):
+    """Odd K, K % 16 != 0, base_exp = -1 and the reference-packed golden cases."""
+    rng = np.random.default_rng(5)
+    for name, g in golden.items():
+        w = g["w"]
+        if name in ("special_4x64", "high_exp_2x32", "top_window_2x30"):
+            continue  # Inf/NaN weights: covered by test_gemv_nonfinite
+        M, K = w.shape
+        p = oracle.pack(w, int(g["base_exp"]))
+        x = oracle.f32_to_bf16_bits(rng.standard_normal(K).astype(np.float32))
+        (got,) = run_gemv(t12, [p], x)
+        ref = oracle.gemv(p, x)
+        assert rel_err(got, ref) < TOL, name
+    w = synth.weights_llm(33, 1001, seed=9, p_outlier=0.01)
+    x = synth.activations(1, 1001, seed=9)[0]
+    p = oracle.pack(w)
+    (got,) = run_gemv(t12, [p], x)
+    assert rel_err(got, oracle.gemv(p, x)) < TOL
+
+
+def test_gemv_nonfinite(t12, oracle, synth):
+    """An Inf weight (always an escape here) must surface as Inf in exactly its row."""
+    w = synth.weights_llm(32, 1024, seed=21, p_outlier=0)
+    w[5, 100] = 0x7F80
+    x = synth.activations(1, 1024, seed=22)[0]
+    x[100] = 0x3F80  # 1.0
+    p = oracle.pack(w)
+    (got,) = run_gemv(t12, [p], x)
+    ref = oracle.gemv(p, x)
+    assert np.isinf(got[5]) and np.isinf(ref[5])
+    mask = np.ones(32, bool); mask[5] = False
+    assert rel_err(got[mask], ref[mask]) < TOL
+
+
+def test_all_variants_agree(t12, oracle, synth):
+    M, K = 520, 4096
+    w = synth.weights_llm(M, K, seed=31, p_outlier=1e-3)
+    x = synth.activations(1, K, seed=32)[0]
+    p = oracle.pack(w)
+    ref = oracle.gemv(p, x)
+    try:
+        for v in [412, 414, 422, 424, 442, 444, 814, 822, 824, 224, 214, 114, 124, 99]:
+            t12.check(t12.lib.t12_tune_gemv(v))
+            (got,) = run_gemv(t12, [p], x)
+            assert rel_err(got, ref) < TOL, v
+    finally:
+        t12.lib.t12_tune_gemv(0)
+
+
+def test_reference_named_launchers(t12, oracle, synth):
+    """launch_split12_v2_async (+dual) give the UNPATCHED product; the patch launchers add
+    (correct - wrong) * x -- the call sequence of the reference's forward_b1."""
+    M, K = 256, 2048
+    pa = oracle.pack(synth.weights_llm(M, K, seed=41, p_outlier=2e-3))
+    pb = oracle.pack(synth.weights_llm(M, K, seed=42, sigma=0.2, p_outlier=2e-3))
+    x = synth.activations(1, K, seed=43)[0]
+    xd = to_dev_bits(x)
+    st = t12.current_stream()
+    da, db = (t12.DeviceTensor12.from_packed(p, dev()) for p in (pa, pb))
+    oa = torch.zeros(M, device=dev()); ob = torch.zeros(M, device=dev())
+    t12.check(t12.lib.launch_split12_v2_async(da.sm.data_ptr(), da.gr.data_ptr(), da.base_exp, xd.data_ptr(),
+                                              oa.data_ptr(), M, K, st))
+    torch.cuda.synchronize()
+    assert rel_err(oa.cpu().numpy(), oracle.gemv(pa, x, patched=False)) < TOL
+    t12.check(t12.lib.launch_patches_v2_async(da.row_off.data_ptr(), da.cols.data_ptr(), da.correct.data_ptr(),
+                                              da.wrong.data_ptr(), xd.data_ptr(), oa.data_ptr(), M, st))
+    torch.cuda.synchronize()
+    assert rel_err(oa.cpu().numpy(), oracle.gemv(pa, x)) < TOL
+    # dual + batched patches
+    oa.zero_()
+    t12.check(t12.lib.launch_split12_v2_dual_async(da.sm.data_ptr(), da.gr.data_ptr(), da.base_exp,
+                                                   db.sm.data_ptr(), db.gr.data_ptr(), db.base_exp, xd.data_ptr(),
+                                                   oa.data_ptr(), ob.data_ptr(), M, K, st))
+    descs = (t12.PatchBatchDesc * 2)(
+        t12.PatchBatchDesc(da.row_off.data_ptr(), da.cols.data_ptr(), da.correct.data_ptr(), da.wrong.data_ptr(),
+                           xd.data_ptr(), oa.data_ptr(), M),
+        t12.PatchBatchDesc(db.row_off.data_ptr(), db.cols.data_ptr(), db.correct.data_ptr(), db.wrong.data_ptr(),
+                           xd.data_ptr(), ob.data_ptr(), M))
+    scratch = torch.zeros(8 * 56, dtype=torch.uint8, device=dev())
+    t12.check(t12.lib.launch_patches_b1_batched_async(scratch.data_ptr(), descs, 2, M, st))
+    torch.cuda.synchronize()
+    assert rel_err(oa.cpu().numpy(), oracle.gemv(pa, x)) < TOL
+    assert rel_err(ob.cpu().numpy(), oracle.gemv(pb, x)) < TOL
+
+
+def test_gemv_rejects_bad_operands(t12):
+    segs = (t12.Segment * 1)(t12.Segment(None, None, None, None, None, None, None, 4, 100))
+    x = torch.zeros(16, dtype=torch.int16, device=dev())
+    assert t12.lib.t12_gemv(segs, 1, x.data_ptr(), 16, None) == -1
+    assert b"null" in t12.lib.t12_last_error()
+    assert t12.lib.t12_gemv(segs, 0, x.data_ptr(), 16, None) == -1
+    assert t12.lib.t12_gemv(segs, 9, x.data_ptr(), 16, None) == -1
+
+
+def test_full_size_linearity(t12, oracle, synth):
+    """Size-independent property at a full Llama layer shape (down: 4096 x 14336):
+    W.(x1 + x2) == W.x1 + W.x2 when x1, x2 have disjoint support (so the bf16 sum is exact)."""
+    M, K = 4096, 14336
+    w = synth.weights_llm(M, K, seed=2003)
+    p = oracle.pack(w)
+    x = synth.activations(1, K, seed=2004)[0]
+    x1 = x.copy(); x1[K // 2:] = 0
+    x2 = x.copy(); x2[:K // 2] = 0
+    dt = t12.DeviceTensor12.from_packed(p, dev())
+    o, o1, o2 = (t12.gemv(dt, to_dev_bits(v))[0].clone() for v in (x, x1, x2))
+    torch.cuda.synchronize()
+    assert rel_err((o1 + o2).cpu().numpy(), o.cpu().numpy()) < 1e-5
+    ref = oracle.gemv(p, x)
+    assert rel_err(o.cpu().numpy(), ref) < TOL

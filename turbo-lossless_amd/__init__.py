@@ -1,0 +1,141 @@
+"""turbo12 for MI355X: ctypes face of libturbo12.so (the C ABI in include/t12_abi.h).
+
+The library is the product; this module only marshals pointers.  torch is used
+for device memory and streams.  There is no CPU fallback: if the HIP library is
+missing, importing this module fails.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libturbo12.so")
+MAX_SEGMENTS = 8
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        "libturbo12.so is not built: run `python turbo-lossless_amd/build.py` "
+        "(hipcc --offload-arch=gfx950). There is no CPU fallback.")
+
+lib = C.CDLL(LIB_PATH)
+
+
+class Segment(C.Structure):
+    """Mirror of T12Segment (include/t12_abi.h)."""
+    _fields_ = [("sm", C.c_void_p), ("gr", C.c_void_p), ("row_off", C.c_void_p), ("cols", C.c_void_p),
+                ("correct", C.c_void_p), ("wrong", C.c_void_p), ("out", C.c_void_p),
+                ("M", C.c_int32), ("base_exp", C.c_int32)]
+
+
+class PatchBatchDesc(C.Structure):
+    _fields_ = [("row_offsets", C.c_void_p), ("patch_cols", C.c_void_p), ("patch_correct", C.c_void_p),
+                ("patch_wrong", C.c_void_p), ("activations", C.c_void_p), ("output", C.c_void_p), ("M", C.c_int)]
+
+
+_vp, _i = C.c_void_p, C.c_int
+_SIGS = {
+    "t12_version": (C.c_char_p, []),
+    "t12_last_error": (C.c_char_p, []),
+    "t12_tune_gemv": (_i, [_i]),
+    "t12_util_read": (_i, [_vp, C.c_size_t, _vp, _i, _vp]),
+    "t12_util_copy": (_i, [_vp, _vp, C.c_size_t, _i, _vp]),
+    "t12_gemv": (_i, [C.POINTER(Segment), _i, _vp, _i, _vp]),
+    "t12_decompress": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "launch_split12_v2_async": (_i, [_vp, _vp, _i, _vp, _vp, _i, _i, _vp]),
+    "launch_split12_v2_dual_async": (_i, [_vp, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _vp]),
+    "launch_patches_v2_async": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
+    "launch_patches_v2": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i]),
+    "launch_patches_b1_batched_async": (_i, [_vp, C.POINTER(PatchBatchDesc), _i, _i, _vp]),
+}
+_OPTIONAL = {}
+for _name, (_res, _args) in _SIGS.items():
+    _fn = getattr(lib, _name)
+    _fn.restype, _fn.argtypes = _res, _args
+
+
+class T12Error(RuntimeError):
+    pass
+
+
+def check(rc: int, what: str = "") -> None:
+    if rc != 0:
+        raise T12Error("%s failed (%d): %s" % (what, rc, lib.t12_last_error().decode()))
+
+
+def _torch():
+    import torch
+    return torch
+
+
+def current_stream() -> int:
+    return _torch().cuda.current_stream().cuda_stream
+
+
+def _dp(t):
+    return None if t is None else t.data_ptr()
+
+
+class DeviceTensor12:
+    """A split-12 tensor resident in HBM: the planes and the CSR escape list."""
+
+    def __init__(self, M, K, base_exp, sm, gr, row_off=None, cols=None, correct=None, wrong=None):
+        self.M, self.K, self.base_exp = int(M), int(K), int(base_exp)
+        self.sm, self.gr = sm, gr
+        self.row_off, self.cols, self.correct, self.wrong = row_off, cols, correct, wrong
+
+    @classmethod
+    def from_packed(cls, p, device="cuda"):
+        """Upload the arrays a packer produced (anything with .sm .gr .row_off .cols .correct .wrong)."""
+        torch = _torch()
+
+        def up(a):
+            a = np.ascontiguousarray(a)
+            if a.size == 0:
+                return torch.zeros(1, dtype=getattr(torch, str(a.dtype)), device=device)[:0]
+            return torch.from_numpy(a).to(device)
+
+        return cls(p.M, p.K, p.base_exp, up(p.sm), up(p.gr), up(p.row_off), up(p.cols), up(p.correct), up(p.wrong))
+
+    @property
+    def P(self):
+        return 0 if self.cols is None else int(self.cols.numel())
+
+    def segment(self, out, patched=True) -> Segment:
+        use = patched and self.row_off is not None and self.P > 0   # no escapes: no list
+        return Segment(_dp(self.sm), _dp(self.gr), _dp(self.row_off) if use else None,
+                       _dp(self.cols) if use else None, _dp(self.correct) if use else None,
+                       _dp(self.wrong) if use else None, _dp(out), self.M, self.base_exp)
+
+
+def _seg_array(segs):
+    arr = (Segment * len(segs))(*segs)
+    return arr
+
+
+def gemv(tensors, act, outs=None, patched=True, stream=None):
+    """Fused decode-GEMV (B = 1) over one or more tensors sharing `act` (bf16 [K])."""
+    torch = _torch()
+    if isinstance(tensors, DeviceTensor12):
+        tensors = [tensors]
+    K = tensors[0].K
+    if outs is None:
+        outs = [torch.empty(t.M, dtype=torch.float32, device=act.device) for t in tensors]
+    segs = _seg_array([t.segment(o, patched) for t, o in zip(tensors, outs)])
+    st = current_stream() if stream is None else stream
+    check(lib.t12_gemv(segs, len(tensors), act.data_ptr(), K, st), "t12_gemv")
+    return outs
+
+
+def decompress(t: DeviceTensor12, patched=True, out=None, stream=None):
+    torch = _torch()
+    if out is None:
+        out = torch.empty((t.M, t.K), dtype=torch.int16, device=t.sm.device)
+    st = current_stream() if stream is None else stream
+    has = t.row_off is not None and t.P > 0
+    check(lib.t12_decompress(_dp(t.sm), _dp(t.gr), t.base_exp, _dp(t.row_off) if has else None,
+                             _dp(t.cols) if has else None, _dp(t.correct) if has else None,
+                             out.data_ptr(), t.M, t.K, int(patched), st), "t12_decompress")
+    return out

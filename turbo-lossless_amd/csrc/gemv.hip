@@ -1,0 +1,411 @@
+// Split-12 fused decode-GEMV for one activation vector (B = 1), gfx950.
+//
+// Computes, for every segment s of a fused launch,
+//     out_s[m] = sum_k dec(W_s[m,k]) * x[k]
+// the function of the reference's split12_matvec_v2 / _multirow / _dual
+// (decompress_v2.hip:148-227, 234-380, 387-523) followed by apply_patches_v2
+// (:78-99), in ONE launch and with a different mapping:
+//   * a lane streams 16 consecutive weights per step with one 128-bit load of
+//     the sign/mantissa plane and one 64-bit load of the nibble plane (a wave
+//     covers 1024 consecutive K of a row), instead of byte loads;
+//   * two weights are rebuilt per 32-bit register (t12_decode8) and multiplied
+//     with v_dot2_f32_bf16 against activations that were paired to match when
+//     they were staged into LDS, once per workgroup;
+//   * escapes: the streamed value of a group-0 weight is the "wrong" value; the
+//     wave that owns the row adds (correct - wrong) * x[col] from the CSR list
+//     before its reduction (wave-level patch, no second launch).
+// Bandwidth bound: 1.5 B per weight from HBM, everything else is L2/LDS.
+
+#include "t12_device.h"
+#include "t12_host.h"
+
+namespace {
+
+struct GemvParams {
+    T12Segment seg[T12_MAX_SEGMENTS];
+    int blk_start[T12_MAX_SEGMENTS + 1];   // first workgroup of each segment
+    int nseg;
+    int K;
+    const uint16_t* act;
+};
+
+__device__ __forceinline__ int find_segment(const GemvParams& p, int blk)
+{
+    int s = 0;
+#pragma unroll
+    for (int i = 1; i < T12_MAX_SEGMENTS; i++)
+        if (i < p.nseg && blk >= p.blk_start[i]) s = i;
+    return s;
+}
+
+// This lane's share of the row's escape corrections.
+// DELTA: the streamed sum already holds wrong * x for every escape, so the
+// correction is (correct - wrong) * x (wrong is finite whenever base_exp >= 0).
+// !DELTA: the streamed sum skipped the escapes, the correction is correct * x.
+template <bool DELTA>
+__device__ __forceinline__ float patch_partial(const T12Segment& sg, int row, int lane,
+                                               const uint16_t* __restrict__ act)
+{
+    float c = 0.0f;
+    if (sg.row_off) {
+        const int beg = sg.row_off[row], end = sg.row_off[row + 1];
+        for (int q = beg + lane; q < end; q += T12_WAVE) {
+            float w = t12_bf16_to_f32((uint16_t)sg.correct[q]);
+            if (DELTA) w -= t12_bf16_to_f32((uint16_t)sg.wrong[q]);
+            c += w * t12_bf16_to_f32(act[sg.cols[q]]);
+        }
+    }
+    return c;
+}
+
+// ---------------------------------------------------------------------------
+// Fast path: K % 16 == 0, 0 <= base_exp <= 240.
+// Workgroup = NW waves; a wave owns R consecutive rows and walks their full K
+// in 1024-column tiles, software pipelined D tiles deep through a register
+// ring: every lane keeps D*R 128-bit + D*R 64-bit loads in flight.
+// Order inside a wave: (1) first D tiles of weight loads go out, (2) the rows'
+// escape corrections are gathered (they become the initial accumulators, so the
+// dependent CSR loads overlap the weight latency instead of draining the
+// stream at the row end), (3) the workgroup stages the activations, (4) steady
+// state: consume a tile, refill its ring slot.
+// LDS: activations, paired (t12_pair_acts), laid out per 1024-column chunk as
+// [half j = 0,1][lane 0..63] x 16 B so that both ds_read_b128 of a lane are
+// conflict free.  Columns >= K are stored as zeros.
+// ---------------------------------------------------------------------------
+template <int NW, int R, int D>
+__global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(const GemvParams p)
+{
+    extern __shared__ uint4 lds_act[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = p.K;
+    const int T = K >> 10;                     // whole 1024-column tiles
+    const int nchunk = (K + 1023) >> 10;
+
+    const int blk = blockIdx.x;
+    const int s = find_segment(p, blk);
+    const T12Segment& sg = p.seg[s];
+    const int M = sg.M;
+    const int row0 = (blk - p.blk_start[s]) * (NW * R) + wave * R;
+    const bool live = row0 < M;                // wave-uniform
+    const uint32_t be2 = ((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23);
+
+    const uint8_t* smp[R];
+    const uint8_t* grp[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const size_t e = (size_t)min(row0 + r, M - 1) * K;      // clamp: loads stay in bounds
+        smp[r] = sg.sm + e + lane * 16;
+        grp[r] = sg.gr + (e >> 1) + lane * 8;
+    }
+
+    constexpr int DR = D > 0 ? D : 1;          // the K tail borrows slot 0
+    uint4 ringS[DR][R];
+    uint2 ringG[DR][R];
+#define T12_FETCH(slot, tile)                                                   \
+    _Pragma("unroll") for (int r = 0; r < R; r++) {                             \
+        ringS[slot][r] = t12_ldg_stream16(smp[r] + (size_t)(tile) * 1024);      \
+        ringG[slot][r] = t12_ldg_stream8(grp[r] + (size_t)(tile) * 512);        \
+    }
+#define T12_CONSUME(slot, tile)                                                                        \
+    {                                                                                                  \
+        const uint4 a0 = lds_act[(tile) * 128 + lane];                                                 \
+        const uint4 a1 = lds_act[(tile) * 128 + 64 + lane];                                            \
+        _Pragma("unroll") for (int r = 0; r < R; r++) {                                                \
+            acc[r] = t12_decode_dot8(ringS[slot][r].x, ringS[slot][r].y, ringG[slot][r].x, be2, a0, acc[r]); \
+            acc[r] = t12_decode_dot8(ringS[slot][r].z, ringS[slot][r].w, ringG[slot][r].y, be2, a1, acc[r]); \
+        }                                                                                              \
+    }
+
+    // the host picks D <= T, so the first D tiles always exist (rows are clamped)
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+        T12_FETCH(d, d)
+        __builtin_amdgcn_sched_barrier(0);   // issue in ring order: waits can then be partial
+    }
+
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+        acc[r] = (live && row0 + r < M) ? patch_partial<true>(sg, row0 + r, lane, p.act) : 0.0f;
+
+    for (int q = tid; q < nchunk * 128; q += NW * 64) {
+        const int k = q * 8;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (k < K) v = *(const uint4*)(p.act + k);
+        lds_act[(q >> 7) * 128 + (q & 1) * 64 + ((q & 127) >> 1)] = t12_pair_acts(v);
+    }
+    __syncthreads();
+    if (!live) return;
+
+    int t = 0;
+    // steady state: whole ring rotations in which every slot is refilled
+    for (; D > 0 && t + 2 * D <= T; t += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            T12_CONSUME(d, t + d)
+            T12_FETCH(d, t + d + D)
+            __builtin_amdgcn_sched_barrier(0);   // keep the refill right behind its consumer
+        }
+    }
+    // drain: the last (up to 2D - 1) tiles
+    for (; D > 0 && t < T; t += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            if (t + d < T) {
+                T12_CONSUME(d, t + d)
+                if (t + d + D < T) { T12_FETCH(d, t + d + D) }
+            }
+        }
+    }
+    if (T < nchunk && T * 1024 + lane * 16 < K) {   // K tail: whole 16-column pieces
+        T12_FETCH(0, T)
+        T12_CONSUME(0, T)
+    }
+#undef T12_FETCH
+#undef T12_CONSUME
+
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        if (row0 + r < M) {                              // wave-uniform
+            const float v = t12_wave_sum_lane63(acc[r]);
+            if (lane == 63) sg.out[row0 + r] = v;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// General path: any K (odd included: nibble parity follows the flat element
+// index), any base_exp (-1 included, where the "wrong" value of an escape is a
+// NaN/Inf pattern).  One wave per row, scalar decode rule.  With an escape list
+// the group-0 elements are skipped in the stream and taken exactly from the
+// list; without one they decode to the wrong value like the reference's
+// unpatched kernels.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void gemv_general_kernel(const GemvParams p)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int blk = blockIdx.x;
+    const int s = find_segment(p, blk);
+    const T12Segment& sg = p.seg[s];
+    const int row = (blk - p.blk_start[s]) * 4 + wave;
+    if (row >= sg.M) return;
+    const int K = p.K;
+    const size_t base = (size_t)row * K;
+    float acc = 0.0f;
+    for (int k = lane; k < K; k += T12_WAVE) {
+        const size_t i = base + k;
+        const uint32_t g = (sg.gr[i >> 1] >> (4 * (i & 1))) & 0xFu;
+        const uint16_t w = t12_decode_scalar(sg.sm[i], g, sg.base_exp);
+        if (g != 0 || !sg.row_off) acc += t12_bf16_to_f32(w) * t12_bf16_to_f32(p.act[k]);
+    }
+    acc += patch_partial<false>(sg, row, lane, p.act);
+    acc = t12_wave_sum(acc);
+    if (lane == 0) sg.out[row] = acc;
+}
+
+// Only the escape corrections (the reference's separate patch kernels).
+__global__ __launch_bounds__(256) void patches_kernel(const GemvParams p)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int blk = blockIdx.x;
+    const int s = find_segment(p, blk);
+    const T12Segment& sg = p.seg[s];
+    const int row = (blk - p.blk_start[s]) * 4 + wave;
+    if (row >= sg.M) return;
+    float c = t12_wave_sum(patch_partial<true>(sg, row, lane, p.act));
+    if (lane == 0 && c != 0.0f) sg.out[row] += c;
+}
+
+int g_gemv_variant = 0;   // 0 = choose by shape; see t12_tune_gemv
+
+template <int NW, int R, int D>
+int launch_stream(GemvParams& p, const T12Segment* segs, int nseg, hipStream_t st)
+{
+    int total = 0;
+    for (int i = 0; i < nseg; i++) {
+        p.blk_start[i] = total;
+        total += (segs[i].M + NW * R - 1) / (NW * R);
+    }
+    p.blk_start[nseg] = total;
+    const size_t lds = (size_t)((p.K + 1023) / 1024) * 2048;
+    hipLaunchKernelGGL((gemv_stream_kernel<NW, R, D>), dim3(total), dim3(NW * 64), lds, st, p);
+    T12_CHECK_LAUNCH("t12_gemv");
+    return T12_OK;
+}
+
+int validate(const T12Segment* segs, int nseg, const void* act, int K, bool need_out)
+{
+    T12_REQUIRE(segs && nseg >= 1 && nseg <= T12_MAX_SEGMENTS, "nseg must be 1..%d (got %d)", T12_MAX_SEGMENTS, nseg);
+    T12_REQUIRE(act && K >= 1, "activations null or K < 1 (K=%d)", K);
+    for (int i = 0; i < nseg; i++) {
+        const T12Segment& g = segs[i];
+        T12_REQUIRE(g.M >= 1, "segment %d: M must be >= 1 (got %d)", i, g.M);
+        T12_REQUIRE(g.sm && g.gr, "segment %d: sm/gr plane is null", i);
+        T12_REQUIRE(!need_out || g.out, "segment %d: output is null", i);
+        T12_REQUIRE(!g.row_off || (g.cols && g.correct && g.wrong),
+                    "segment %d: row_off given without cols/correct/wrong", i);
+        T12_REQUIRE(g.base_exp >= -1 && g.base_exp <= 254, "segment %d: base_exp %d out of range", i, g.base_exp);
+    }
+    return T12_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+// Selects the B = 1 kernel variant (benchmark sweeps): 0 = by shape.
+int t12_tune_gemv(int variant)
+{
+    g_gemv_variant = variant;
+    return T12_OK;
+}
+
+int t12_gemv(const T12Segment* segs, int nseg, const void* act_bf16, int K, void* stream)
+{
+    int rc = validate(segs, nseg, act_bf16, K, true);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    GemvParams p;
+    p.nseg = nseg;
+    p.K = K;
+    p.act = (const uint16_t*)act_bf16;
+    bool fast = (K % 16 == 0) && ((K + 1023) / 1024 * 2048 <= 160 * 1024);
+    for (int i = 0; i < nseg; i++) {
+        p.seg[i] = segs[i];
+        if (segs[i].base_exp < 0 || segs[i].base_exp > 240) fast = false;
+    }
+    if (!fast || g_gemv_variant == 99) {
+        int total = 0;
+        for (int i = 0; i < nseg; i++) {
+            p.blk_start[i] = total;
+            total += (segs[i].M + 3) / 4;
+        }
+        p.blk_start[nseg] = total;
+        hipLaunchKernelGGL(gemv_general_kernel, dim3(total), dim3(256), 0, st, p);
+        T12_CHECK_LAUNCH("t12_gemv(general)");
+        return T12_OK;
+    }
+    // variant = 100*NW + 10*R + D ; 0 = by shape.  The ring depth may not exceed
+    // the number of whole 1024-column tiles.
+    const int T = K / 1024;
+    int v = g_gemv_variant;
+    if (v == 0) v = T >= 4 ? 424 : (T >= 2 ? 422 : 421);
+    if (v % 10 > T) v = v - v % 10 + (T >= 4 ? 4 : (T >= 2 ? 2 : (T >= 1 ? 1 : 0)));
+    switch (v) {
+        case 420: return launch_stream<4, 2, 0>(p, segs, nseg, st);
+        case 421: return launch_stream<4, 2, 1>(p, segs, nseg, st);
+        case 410: return launch_stream<4, 1, 0>(p, segs, nseg, st);
+        case 411: return launch_stream<4, 1, 1>(p, segs, nseg, st);
+        case 412: return launch_stream<4, 1, 2>(p, segs, nseg, st);
+        case 414: return launch_stream<4, 1, 4>(p, segs, nseg, st);
+        case 417: return launch_stream<4, 1, 7>(p, segs, nseg, st);
+        case 422: return launch_stream<4, 2, 2>(p, segs, nseg, st);
+        case 424: return launch_stream<4, 2, 4>(p, segs, nseg, st);
+        case 427: return launch_stream<4, 2, 7>(p, segs, nseg, st);
+        case 442: return launch_stream<4, 4, 2>(p, segs, nseg, st);
+        case 444: return launch_stream<4, 4, 4>(p, segs, nseg, st);
+        case 814: return launch_stream<8, 1, 4>(p, segs, nseg, st);
+        case 822: return launch_stream<8, 2, 2>(p, segs, nseg, st);
+        case 824: return launch_stream<8, 2, 4>(p, segs, nseg, st);
+        case 224: return launch_stream<2, 2, 4>(p, segs, nseg, st);
+        case 214: return launch_stream<2, 1, 4>(p, segs, nseg, st);
+        case 114: return launch_stream<1, 1, 4>(p, segs, nseg, st);
+        case 124: return launch_stream<1, 2, 4>(p, segs, nseg, st);
+        default:
+            if (T >= 4) return launch_stream<4, 2, 4>(p, segs, nseg, st);
+            if (T >= 2) return launch_stream<4, 2, 2>(p, segs, nseg, st);
+            if (T >= 1) return launch_stream<4, 2, 1>(p, segs, nseg, st);
+            return launch_stream<4, 2, 0>(p, segs, nseg, st);
+    }
+}
+
+// ---- reference-named launchers ---------------------------------------------
+int launch_split12_v2_async(const void* sign_mantissa, const void* groups, int base_exp,
+                            const void* activations, void* output, int M, int K, void* stream)
+{
+    T12Segment g = {(const uint8_t*)sign_mantissa, (const uint8_t*)groups, nullptr, nullptr, nullptr, nullptr,
+                    (float*)output, M, base_exp};
+    return t12_gemv(&g, 1, activations, K, stream);
+}
+
+int launch_split12_v2_dual_async(const void* sm_a, const void* gr_a, int base_exp_a,
+                                 const void* sm_b, const void* gr_b, int base_exp_b,
+                                 const void* activations, void* output_a, void* output_b,
+                                 int M, int K, void* stream)
+{
+    T12Segment g[2] = {
+        {(const uint8_t*)sm_a, (const uint8_t*)gr_a, nullptr, nullptr, nullptr, nullptr, (float*)output_a, M, base_exp_a},
+        {(const uint8_t*)sm_b, (const uint8_t*)gr_b, nullptr, nullptr, nullptr, nullptr, (float*)output_b, M, base_exp_b}};
+    return t12_gemv(g, 2, activations, K, stream);
+}
+
+static int launch_patch_descs(const PatchBatchDesc* d, int n, hipStream_t st)
+{
+    // all descriptors of one call read the same activation vector in the reference's
+    // call sites (inference.cpp:263-269, 318-322); different vectors get one launch each
+    int i = 0;
+    while (i < n) {
+        GemvParams p;
+        int cnt = 0, total = 0;
+        p.act = (const uint16_t*)d[i].activations;
+        while (i < n && cnt < T12_MAX_SEGMENTS && (const uint16_t*)d[i].activations == p.act) {
+            T12Segment& g = p.seg[cnt];
+            g.sm = g.gr = nullptr;
+            g.row_off = d[i].row_offsets;
+            g.cols = d[i].patch_cols;
+            g.correct = d[i].patch_correct;
+            g.wrong = d[i].patch_wrong;
+            g.out = d[i].output;
+            g.M = d[i].M;
+            g.base_exp = 0;
+            p.blk_start[cnt] = total;
+            total += (d[i].M + 3) / 4;
+            cnt++;
+            i++;
+        }
+        p.blk_start[cnt] = total;
+        p.nseg = cnt;
+        p.K = 0;
+        if (total > 0) {
+            hipLaunchKernelGGL(patches_kernel, dim3(total), dim3(256), 0, st, p);
+            T12_CHECK_LAUNCH("launch_patches");
+        }
+    }
+    return T12_OK;
+}
+
+int launch_patches_v2_async(const void* row_offsets, const void* patch_cols, const void* correct_vals,
+                            const void* wrong_vals, const void* activations, void* output, int M, void* stream)
+{
+    if (M == 0) return 0;
+    T12_REQUIRE(row_offsets && patch_cols && correct_vals && wrong_vals && activations && output && M > 0,
+                "launch_patches_v2_async: null operand or M < 0");
+    PatchBatchDesc d = {(const int32_t*)row_offsets, (const int32_t*)patch_cols, (const int16_t*)correct_vals,
+                        (const int16_t*)wrong_vals, (const int16_t*)activations, (float*)output, M};
+    return launch_patch_descs(&d, 1, (hipStream_t)stream);
+}
+
+int launch_patches_v2(const void* row_offsets, const void* patch_cols, const void* correct_vals,
+                      const void* wrong_vals, const void* activations, void* output, int M)
+{
+    int rc = launch_patches_v2_async(row_offsets, patch_cols, correct_vals, wrong_vals, activations, output, M, nullptr);
+    if (rc) return -1;
+    return hipDeviceSynchronize() == hipSuccess ? 0 : -1;
+}
+
+// descs_gpu is accepted for signature compatibility and left untouched: the
+// descriptors travel as kernel arguments, so no host-to-device copy is needed.
+int launch_patches_b1_batched_async(void* descs_gpu, const void* descs_cpu, int num_descs, int max_M, void* stream)
+{
+    (void)descs_gpu;
+    if (num_descs == 0 || max_M == 0) return 0;
+    T12_REQUIRE(descs_cpu && num_descs > 0 && num_descs <= 8, "launch_patches_b1_batched_async: 1..8 descriptors");
+    const PatchBatchDesc* d = (const PatchBatchDesc*)descs_cpu;
+    for (int i = 0; i < num_descs; i++)
+        T12_REQUIRE(d[i].row_offsets && d[i].patch_cols && d[i].patch_correct && d[i].patch_wrong &&
+                        d[i].activations && d[i].output && d[i].M > 0,
+                    "launch_patches_b1_batched_async: descriptor %d has a null field", i);
+    return launch_patch_descs(d, num_descs, (hipStream_t)stream);
+}
+
+}  // extern "C"
