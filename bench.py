@@ -1,0 +1,201 @@
+#!/usr/bin/env python3
+"""Benchmark of the split-12 hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+Workloads (synthetic, seeded, random-init weights of the Llama-3.1-8B shape:
+32 layers, hidden 4096, FFN 14336, 32/8 heads, vocab 128256; N(0, 0.02) with
+3e-4 of the entries replaced by N(0, 8) outliers so that ~0.045 % escape):
+
+  gemv_stack_b1   one step = every linear layer of one decode step at B = 1 through
+                  the fused split-12 decode-GEMV: per layer QKV (3 segments, one
+                  launch), O, gate+up (2 segments, one launch), down; then lm_head.
+                  7 504 658 432 weights = 11.257 GB of compressed planes per step.
+
+Prints ONE JSON line.  `value` is tokens per second of the step (inputs resident
+in HBM), `roofline` prices the decode-GEMV kernel against the 8 TB/s HBM peak in
+algorithmic bytes (1.5 B per weight + escape list + activations + outputs), and
+`cpu_baseline` is the CPU oracle (fused decode + fp32 GEMV, OpenMP over the host
+cores) timed on one decoder layer of the same weights and scaled to the model.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+LLAMA8B = dict(n_layer=32, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=8, n_vocab=128256)
+HBM_PEAK_GBS = 8000.0
+
+
+def synth_weight(torch, M, K, seed, dev, sigma=0.02, p_out=3e-4, sigma_out=8.0):
+    """bf16 [M, K] on the GPU: N(0, sigma) with outliers N(0, sigma_out) at rate p_out."""
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    w = torch.randn((M, K), generator=g, device=dev, dtype=torch.float32) * sigma
+    m = torch.rand((M, K), generator=g, device=dev) < p_out
+    o = torch.randn((M, K), generator=g, device=dev, dtype=torch.float32) * sigma_out
+    w = torch.where(m, o, w).to(torch.bfloat16)
+    return w
+
+
+def algorithmic_bytes(t, B=1):
+    """1.5*M*K + 8*P + 4*(M+1) + 2*K*B + 4*M*B  (the figure the roofline is priced in)."""
+    return 1.5 * t.M * t.K + 8 * t.P + 4 * (t.M + 1) + 2 * t.K * B + 4 * t.M * B
+
+
+def build_stack(t12, torch, dev, cfg, base_seed=4000):
+    """Packs the model's linear layers on the GPU.  Returns the list of launches:
+    each is (tensors, act_key) with act_key in {'h', 'ff'}."""
+    n, ff, hd = cfg["n_embd"], cfg["n_ff"], cfg["n_embd"] // cfg["n_head"]
+    kv = cfg["n_head_kv"] * hd
+    launches = []
+    seed = base_seed
+    for _ in range(cfg["n_layer"]):
+        def mk(M, K):
+            nonlocal seed
+            seed += 1
+            return t12.pack_device(synth_weight(torch, M, K, seed, dev))
+        launches.append(([mk(n, n), mk(kv, n), mk(kv, n)], "h"))      # wq | wk | wv
+        launches.append(([mk(n, n)], "h"))                             # wo
+        launches.append(([mk(ff, n), mk(ff, n)], "h"))                 # w_gate | w_up
+        launches.append(([mk(n, ff)], "ff"))                           # w_down
+    # lm_head: built in 8 row slabs to bound the fp32 staging memory, then joined
+    slabs = []
+    rows = cfg["n_vocab"] // 8
+    for i in range(8):
+        seed += 1
+        slabs.append(synth_weight(torch, rows, n, seed, dev))
+    w = torch.cat(slabs)
+    del slabs
+    launches.append(([t12.pack_device(w)], "h"))
+    del w
+    torch.cuda.empty_cache()
+    return launches
+
+
+def cpu_baseline(torch, launches, cfg, runs=3):
+    """Times the CPU oracle on the first decoder layer (7 tensors, 218 M weights) and scales
+    the per-weight rate to the whole model."""
+    import numpy as np
+    from oracle import oracle
+
+    class P:  # the oracle's Packed duck type, filled from device arrays
+        pass
+
+    packs = []
+    for tensors, key in launches[:4]:
+        for t in tensors:
+            p = oracle.Packed(t.M, t.K, t.base_exp, t.sm.cpu().numpy(), t.gr.cpu().numpy(),
+                              t.row_off.cpu().numpy(), t.cols.cpu().numpy(), t.correct.cpu().numpy(),
+                              t.wrong.cpu().numpy())
+            packs.append(p)
+    rng = np.random.default_rng(7)
+    xs = {K: oracle.f32_to_bf16_bits(rng.standard_normal(K).astype(np.float32)) for K in {p.K for p in packs}}
+    times = []
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        for p in packs:
+            oracle.gemv(p, xs[p.K])
+        times.append(time.perf_counter() - t0)
+    t_layer = sorted(times)[len(times) // 2]
+    w_layer = sum(p.M * p.K for p in packs)
+    w_model = sum(t.M * t.K for tensors, _ in launches for t in tensors)
+    t_model = t_layer * w_model / w_layer
+    return {
+        "value": 1.0 / t_model, "unit": "tok/s", "cores": oracle.num_threads(), "kind": "port",
+        "sample": "decoder layer 0 (wq,wk,wv,wo,gate,up,down = %d weights) x%d runs, median %.3f s, scaled by weight "
+                  "count to the %d-weight model; %.2f GB/s compressed" % (w_layer, runs, t_layer, w_model,
+                                                                          1.5 * w_layer / t_layer / 1e9),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="gemv_stack_b1")
+    ap.add_argument("--layers", type=int, default=LLAMA8B["n_layer"], help="debug: fewer layers (invalid as a result)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path has no collective); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import __graft_entry__ as ge
+    t12 = ge.load_package()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = dict(LLAMA8B, n_layer=args.layers)
+
+    t0 = time.time()
+    launches = build_stack(t12, torch, dev, cfg)
+    torch.cuda.synchronize()
+    t_build = time.time() - t0
+
+    g = torch.Generator(device=dev)
+    g.manual_seed(99)
+    acts = {"h": torch.randn(cfg["n_embd"], generator=g, device=dev).to(torch.bfloat16),
+            "ff": torch.randn(cfg["n_ff"], generator=g, device=dev).to(torch.bfloat16)}
+    outs = [[torch.empty(t.M, dtype=torch.float32, device=dev) for t in tensors] for tensors, _ in launches]
+    stream = t12.current_stream()
+    # segment tables are built once; a step is pure launches
+    seg_tabs = [(t12._seg_array([t.segment(o) for t, o in zip(tensors, out)]), len(tensors), acts[key].data_ptr(),
+                 tensors[0].K) for (tensors, key), out in zip(launches, outs)]
+
+    def step():
+        for segs, n, act, K in seg_tabs:
+            rc = t12.lib.t12_gemv(segs, n, act, K, stream)
+            if rc:
+                t12.check(rc, "t12_gemv")
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    w0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - w0) * 1e3 / args.steps
+    ms = e0.elapsed_time(e1) / args.steps          # HIP events on the launch stream
+    ms_step = max(ms, wall_ms)
+
+    n_launch = len(launches)
+    alg_bytes = sum(algorithmic_bytes(t) for tensors, _ in launches for t in tensors)
+    plane_bytes = sum(1.5 * t.M * t.K for tensors, _ in launches for t in tensors)
+    n_weights = sum(t.M * t.K for tensors, _ in launches for t in tensors)
+    achieved = alg_bytes / (ms * 1e-3) / 1e9       # GB/s, per-launch bytes / per-launch duration
+    result = {
+        "metric": "tok/s at B=1 (Llama-3.1-8B shape), split-12 decode-GEMV over every linear layer of a decode step",
+        "value": 1e3 / ms_step, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "shape": "Llama-3.1-8B", "batch": 1, "n_layer": cfg["n_layer"],
+                   "weights": n_weights, "launches_per_step": n_launch,
+                   "compressed_GB_per_step": plane_bytes / 1e9, "escape_fraction":
+                       sum(t.P for tensors, _ in launches for t in tensors) / n_weights},
+        "gemv_compressed_GBps": plane_bytes / (ms * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "gemv_stream_kernel", "bytes_per_launch": alg_bytes / n_launch,
+                     "us_per_launch": ms * 1e3 / n_launch},
+        "setup_s": t_build,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(torch, launches, cfg)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

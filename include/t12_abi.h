@@ -99,6 +99,26 @@ int t12_decompress(const void* sm, const void* gr, int base_exp, const void* row
                    const void* cols, const void* correct, void* out_bf16,
                    int M, int K, int patched, void* stream);
 
+/* ---- GPU-side packer ---------------------------------------------------------
+ * The reference packs on one CPU thread (split12_pack.c); these entry points
+ * produce byte-identical arrays from a bf16 matrix resident in HBM.
+ *   t12_pack_histogram : 256-bin histogram of the exponent byte (u64 counters,
+ *                        zeroed by the call)                  split12_pack.c:20-24
+ *   t12_pack_base_exp  : HOST function, window rule on a host copy of the
+ *                        histogram                            split12_pack.c:26-36
+ *   t12_pack_planes    : sm, gr and per-row escape counts (i32[M], zeroed by
+ *                        the call)                            split12_pack.c:76-97
+ *   t12_pack_row_offsets: exclusive scan -> row_off[M+1]      split12_pack.c:99-101
+ *   t12_pack_escapes   : cols / correct / wrong in CSR order  split12_pack.c:103-124
+ * The caller reads row_off[M] (= P) back to size the three escape arrays. */
+int t12_pack_histogram(const void* w_bf16, size_t n, void* hist_u64x256, void* stream);
+int t12_pack_base_exp(const uint64_t* hist_host);
+int t12_pack_planes(const void* w_bf16, int M, int K, int base_exp, void* sm, void* gr, void* row_cnt,
+                    void* stream);
+int t12_pack_row_offsets(const void* row_cnt, int M, void* row_off, void* stream);
+int t12_pack_escapes(const void* w_bf16, int M, int K, int base_exp, const void* row_off, void* cols,
+                     void* correct, void* wrong, void* stream);
+
 /* ---- reference-named launchers (same signatures and semantics) -------------
  * For host code written against the reference's launch layer.
  * decompress_v2.hip:530,549,113,129,860,877 */

@@ -127,7 +127,7 @@ def test_all_variants_agree(t12, oracle, synth):
     p = oracle.pack(w)
     ref = oracle.gemv(p, x)
     try:
-        for v in [412, 414, 422, 424, 442, 444, 814, 822, 824, 224, 214, 114, 124, 99]:
+        for v in [810, 811, 812, 814, 411, 412, 414, 421, 422, 424, 442, 99]:
             t12.check(t12.lib.t12_tune_gemv(v))
             (got,) = run_gemv(t12, [p], x)
             assert rel_err(got, ref) < TOL, v

@@ -42,6 +42,11 @@ _SIGS = {
     "t12_tune_gemv": (_i, [_i]),
     "t12_util_read": (_i, [_vp, C.c_size_t, _vp, _i, _vp]),
     "t12_util_copy": (_i, [_vp, _vp, C.c_size_t, _i, _vp]),
+    "t12_pack_histogram": (_i, [_vp, C.c_size_t, _vp, _vp]),
+    "t12_pack_base_exp": (_i, [C.POINTER(C.c_uint64)]),
+    "t12_pack_planes": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
+    "t12_pack_row_offsets": (_i, [_vp, _i, _vp, _vp]),
+    "t12_pack_escapes": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "t12_gemv": (_i, [C.POINTER(Segment), _i, _vp, _i, _vp]),
     "t12_decompress": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "launch_split12_v2_async": (_i, [_vp, _vp, _i, _vp, _vp, _i, _i, _vp]),
@@ -139,3 +144,40 @@ def decompress(t: DeviceTensor12, patched=True, out=None, stream=None):
                              _dp(t.cols) if has else None, _dp(t.correct) if has else None,
                              out.data_ptr(), t.M, t.K, int(patched), st), "t12_decompress")
     return out
+
+
+def find_base_exp_device(w, stream=None) -> int:
+    """split12_find_base_exp on a bf16 matrix resident in HBM."""
+    torch = _torch()
+    st = current_stream() if stream is None else stream
+    hist = torch.empty(256, dtype=torch.int64, device=w.device)
+    check(lib.t12_pack_histogram(w.data_ptr(), w.numel(), hist.data_ptr(), st), "t12_pack_histogram")
+    h = hist.cpu().numpy().astype(np.uint64)       # synchronises
+    return int(lib.t12_pack_base_exp(h.ctypes.data_as(C.POINTER(C.c_uint64))))
+
+
+def pack_device(w, base_exp=None, stream=None) -> DeviceTensor12:
+    """Pack a bf16 matrix [M, K] (torch.bfloat16 or int16 bits, on the GPU) into split-12 on the GPU."""
+    torch = _torch()
+    assert w.dim() == 2 and w.is_contiguous() and w.element_size() == 2
+    M, K = w.shape
+    st = current_stream() if stream is None else stream
+    if base_exp is None:
+        base_exp = find_base_exp_device(w, st)
+    n = M * K
+    dev = w.device
+    sm = torch.empty(n, dtype=torch.uint8, device=dev)
+    gr = torch.empty((n + 1) // 2, dtype=torch.uint8, device=dev)
+    cnt = torch.empty(M, dtype=torch.int32, device=dev)
+    row_off = torch.empty(M + 1, dtype=torch.int32, device=dev)
+    check(lib.t12_pack_planes(w.data_ptr(), M, K, base_exp, sm.data_ptr(), gr.data_ptr(), cnt.data_ptr(), st),
+          "t12_pack_planes")
+    check(lib.t12_pack_row_offsets(cnt.data_ptr(), M, row_off.data_ptr(), st), "t12_pack_row_offsets")
+    P = int(row_off[M].item())                      # synchronises
+    cols = torch.empty(P, dtype=torch.int32, device=dev)
+    correct = torch.empty(P, dtype=torch.int16, device=dev)
+    wrong = torch.empty(P, dtype=torch.int16, device=dev)
+    if P:
+        check(lib.t12_pack_escapes(w.data_ptr(), M, K, base_exp, row_off.data_ptr(), cols.data_ptr(),
+                                   correct.data_ptr(), wrong.data_ptr(), st), "t12_pack_escapes")
+    return DeviceTensor12(M, K, base_exp, sm, gr, row_off, cols, correct, wrong)

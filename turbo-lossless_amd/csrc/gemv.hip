@@ -63,17 +63,30 @@ __device__ __forceinline__ float patch_partial(const T12Segment& sg, int row, in
 // Workgroup = NW waves; a wave owns R consecutive rows and walks their full K
 // in 1024-column tiles, software pipelined D tiles deep through a register
 // ring: every lane keeps D*R 128-bit + D*R 64-bit loads in flight.
-// Order inside a wave: (1) first D tiles of weight loads go out, (2) the rows'
-// escape corrections are gathered (they become the initial accumulators, so the
-// dependent CSR loads overlap the weight latency instead of draining the
-// stream at the row end), (3) the workgroup stages the activations, (4) steady
-// state: consume a tile, refill its ring slot.
+// Order inside a wave, arranged so that no dependent load chain is exposed:
+//   (1) CSR row pointers of the R rows (one vector load, lanes 0..R),
+//   (2) the first D tiles of weight loads,
+//   (3) the workgroup stages the activations into LDS, barrier,
+//   (4) the rows' first 64 escape entries each (cols / correct / wrong) are
+//       requested; they arrive while
+//   (5) the tile stream is consumed and refilled,
+//   (6) escape corrections: (correct - wrong) * x[col], x read back from LDS,
+//   (7) DPP wave reduction, lane 63 stores.
 // LDS: activations, paired (t12_pair_acts), laid out per 1024-column chunk as
 // [half j = 0,1][lane 0..63] x 16 B so that both ds_read_b128 of a lane are
 // conflict free.  Columns >= K are stored as zeros.
 // ---------------------------------------------------------------------------
-template <int NW, int R, int D>
-__global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(const GemvParams p)
+__device__ __forceinline__ float lds_act_at(const uint4* lds_act, int k)
+{
+    // inverse of the staging layout: column k -> its bf16 inside the paired tiles
+    const int q = k >> 3, i = k & 7;
+    const int slot = (q >> 7) * 128 + (q & 1) * 64 + ((q & 127) >> 1);
+    const uint16_t* h = (const uint16_t*)(lds_act + slot);
+    return t12_bf16_to_f32(h[(i & 3) * 2 + (i >> 2)]);
+}
+
+template <int NW, int R, int D, int MINB>
+__global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvParams p)
 {
     extern __shared__ uint4 lds_act[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -88,6 +101,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(const GemvParams p
     const int row0 = (blk - p.blk_start[s]) * (NW * R) + wave * R;
     const bool live = row0 < M;                // wave-uniform
     const uint32_t be2 = ((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23);
+    const bool patched = sg.row_off != nullptr;
+
+    int ro = 0;                                // lane l <= R: row_off[row0 + l]
+    if (patched && live && lane <= R) ro = sg.row_off[min(row0 + lane, M)];
 
     const uint8_t* smp[R];
     const uint8_t* grp[R];
@@ -123,11 +140,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(const GemvParams p
         __builtin_amdgcn_sched_barrier(0);   // issue in ring order: waits can then be partial
     }
 
-    float acc[R];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-        acc[r] = (live && row0 + r < M) ? patch_partial<true>(sg, row0 + r, lane, p.act) : 0.0f;
-
     for (int q = tid; q < nchunk * 128; q += NW * 64) {
         const int k = q * 8;
         uint4 v = make_uint4(0, 0, 0, 0);
@@ -136,6 +148,28 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(const GemvParams p
     }
     __syncthreads();
     if (!live) return;
+
+    // escape entries: lane l takes entry beg + l of each row
+    int pcol[R];
+    float pdelta[R];
+    int pend[R], pnext[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int beg = __builtin_amdgcn_readlane(ro, r), end = __builtin_amdgcn_readlane(ro, r + 1);
+        pend[r] = end;
+        pnext[r] = beg + T12_WAVE;
+        pcol[r] = -1;
+        pdelta[r] = 0.0f;
+        if (beg + lane < end) {
+            pcol[r] = sg.cols[beg + lane];
+            pdelta[r] = t12_bf16_to_f32((uint16_t)sg.correct[beg + lane]) -
+                        t12_bf16_to_f32((uint16_t)sg.wrong[beg + lane]);
+        }
+    }
+
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.0f;
 
     int t = 0;
     // steady state: whole ring rotations in which every slot is refilled
@@ -167,7 +201,12 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(const GemvParams p
 #pragma unroll
     for (int r = 0; r < R; r++) {
         if (row0 + r < M) {                              // wave-uniform
-            const float v = t12_wave_sum_lane63(acc[r]);
+            float v = acc[r];
+            if (pcol[r] >= 0) v += pdelta[r] * lds_act_at(lds_act, pcol[r]);
+            for (int q = pnext[r] + lane; q < pend[r]; q += T12_WAVE)     // rows with > 64 escapes
+                v += (t12_bf16_to_f32((uint16_t)sg.correct[q]) - t12_bf16_to_f32((uint16_t)sg.wrong[q])) *
+                     lds_act_at(lds_act, sg.cols[q]);
+            v = t12_wave_sum_lane63(v);
             if (lane == 63) sg.out[row0 + r] = v;
         }
     }
@@ -218,7 +257,7 @@ __global__ __launch_bounds__(256) void patches_kernel(const GemvParams p)
 
 int g_gemv_variant = 0;   // 0 = choose by shape; see t12_tune_gemv
 
-template <int NW, int R, int D>
+template <int NW, int R, int D, int MINB = 1>
 int launch_stream(GemvParams& p, const T12Segment* segs, int nseg, hipStream_t st)
 {
     int total = 0;
@@ -228,7 +267,7 @@ int launch_stream(GemvParams& p, const T12Segment* segs, int nseg, hipStream_t s
     }
     p.blk_start[nseg] = total;
     const size_t lds = (size_t)((p.K + 1023) / 1024) * 2048;
-    hipLaunchKernelGGL((gemv_stream_kernel<NW, R, D>), dim3(total), dim3(NW * 64), lds, st, p);
+    hipLaunchKernelGGL((gemv_stream_kernel<NW, R, D, MINB>), dim3(total), dim3(NW * 64), lds, st, p);
     T12_CHECK_LAUNCH("t12_gemv");
     return T12_OK;
 }
@@ -285,37 +324,33 @@ int t12_gemv(const T12Segment* segs, int nseg, const void* act_bf16, int K, void
         T12_CHECK_LAUNCH("t12_gemv(general)");
         return T12_OK;
     }
-    // variant = 100*NW + 10*R + D ; 0 = by shape.  The ring depth may not exceed
-    // the number of whole 1024-column tiles.
+    // variant = 100*NW + 10*R + D ; 0 = by shape.  The ring depth may not exceed the
+    // number of whole 1024-column tiles.  Measured on MI355X (Llama-3.1-8B layer
+    // shapes): 8 waves x 1 row x depth 2 is the fastest everywhere -- the chip
+    // hides HBM latency better with many light waves (62 VGPRs, 8 waves/SIMD)
+    // than with deep per-wave rings.
     const int T = K / 1024;
-    int v = g_gemv_variant;
-    if (v == 0) v = T >= 4 ? 424 : (T >= 2 ? 422 : 421);
-    if (v % 10 > T) v = v - v % 10 + (T >= 4 ? 4 : (T >= 2 ? 2 : (T >= 1 ? 1 : 0)));
+    int v = g_gemv_variant ? g_gemv_variant : 812;
+    const int dmax = T >= 4 ? 4 : (T >= 2 ? 2 : T);
+    if (v % 10 > dmax) v = v - v % 10 + dmax;
+    if (v % 10 == 0 && T > 0) v += 1;               // depth 0 only exists for K < 1024
     switch (v) {
-        case 420: return launch_stream<4, 2, 0>(p, segs, nseg, st);
-        case 421: return launch_stream<4, 2, 1>(p, segs, nseg, st);
+        case 810: return launch_stream<8, 1, 0>(p, segs, nseg, st);
+        case 811: return launch_stream<8, 1, 1>(p, segs, nseg, st);
+        case 812: return launch_stream<8, 1, 2>(p, segs, nseg, st);
+        case 814: return launch_stream<8, 1, 4>(p, segs, nseg, st);
         case 410: return launch_stream<4, 1, 0>(p, segs, nseg, st);
         case 411: return launch_stream<4, 1, 1>(p, segs, nseg, st);
         case 412: return launch_stream<4, 1, 2>(p, segs, nseg, st);
         case 414: return launch_stream<4, 1, 4>(p, segs, nseg, st);
-        case 417: return launch_stream<4, 1, 7>(p, segs, nseg, st);
+        case 420: return launch_stream<4, 2, 0>(p, segs, nseg, st);
+        case 421: return launch_stream<4, 2, 1>(p, segs, nseg, st);
         case 422: return launch_stream<4, 2, 2>(p, segs, nseg, st);
         case 424: return launch_stream<4, 2, 4>(p, segs, nseg, st);
-        case 427: return launch_stream<4, 2, 7>(p, segs, nseg, st);
         case 442: return launch_stream<4, 4, 2>(p, segs, nseg, st);
-        case 444: return launch_stream<4, 4, 4>(p, segs, nseg, st);
-        case 814: return launch_stream<8, 1, 4>(p, segs, nseg, st);
-        case 822: return launch_stream<8, 2, 2>(p, segs, nseg, st);
-        case 824: return launch_stream<8, 2, 4>(p, segs, nseg, st);
-        case 224: return launch_stream<2, 2, 4>(p, segs, nseg, st);
-        case 214: return launch_stream<2, 1, 4>(p, segs, nseg, st);
-        case 114: return launch_stream<1, 1, 4>(p, segs, nseg, st);
-        case 124: return launch_stream<1, 2, 4>(p, segs, nseg, st);
         default:
-            if (T >= 4) return launch_stream<4, 2, 4>(p, segs, nseg, st);
-            if (T >= 2) return launch_stream<4, 2, 2>(p, segs, nseg, st);
-            if (T >= 1) return launch_stream<4, 2, 1>(p, segs, nseg, st);
-            return launch_stream<4, 2, 0>(p, segs, nseg, st);
+            t12_set_error("t12_gemv: unknown kernel variant %d", v);
+            return T12_EINVAL;
     }
 }
 
