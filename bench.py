@@ -31,6 +31,10 @@ sys.path.insert(0, ROOT)
 
 LLAMA8B = dict(n_layer=32, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=8, n_vocab=128256)
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per gemv launch of the gemv_stack_b1 workload, from two rocprofv3 --pmc runs of this file
+# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from the --calibrate copy kernel; the summary is
+# profiles/gemv_stream_kernel_llama8b_stack_b1.md).  Valid for the full 32-layer stack only.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"gemv_stack_b1": 88.48e6}
 
 
 def synth_weight(torch, M, K, seed, dev, sigma=0.02, p_out=3e-4, sigma_out=8.0):
@@ -123,6 +127,9 @@ def main():
     ap.add_argument("--workload", default="gemv_stack_b1")
     ap.add_argument("--layers", type=int, default=LLAMA8B["n_layer"], help="debug: fewer layers (invalid as a result)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch one plain 1 GiB copy kernel (t12_util_copy) before the steps: the known-size "
+                         "yardstick for the profiler's FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no collective); run with --gpus 1",
@@ -157,6 +164,13 @@ def main():
             if rc:
                 t12.check(rc, "t12_gemv")
 
+    if args.calibrate:
+        src = torch.empty(2**30, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        t12.check(t12.lib.t12_util_copy(dst.data_ptr(), src.data_ptr(), src.numel(), 8192, stream), "t12_util_copy")
+        torch.cuda.synchronize()
+        del src, dst
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -187,7 +201,9 @@ def main():
                        sum(t.P for tensors, _ in launches for t in tensors) / n_weights},
         "gemv_compressed_GBps": plane_bytes / (ms * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload)
+                     if cfg["n_layer"] == LLAMA8B["n_layer"] else None,
                      "kernel": "gemv_stream_kernel", "bytes_per_launch": alg_bytes / n_launch,
                      "us_per_launch": ms * 1e3 / n_launch},
         "setup_s": t_build,
