@@ -90,6 +90,9 @@ int t12_gemv_batch(const T12Segment* segs, int nseg, const void* act_bf16, int a
 int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride,
              int out_stride, int K, int B, void* stream);
 
+/* Pins the number of K splits of the MFMA path; 0 restores the choice by shape. */
+int t12_tune_gemm(int ksplit);
+
 /* ---- (c) standalone decompress --------------------------------------------
  * out_bf16[m*K + k] = decoded weight bits.  patched != 0: escapes take
  * `correct` (lossless, bit-exact with the tensor that was packed).

@@ -1,0 +1,131 @@
+"""GPU parity: split-12 decode+GEMM (bf16 MFMA, fp32 accumulate) through the C ABI vs the
+CPU oracle's decode-then-fp32-accumulate GEMM.
+
+Tolerance: north star 1e-2 relative; both sides multiply bf16 x bf16 exactly and accumulate
+in fp32, so the observed error is ~1e-6 and the assertions use 1e-4.
+"""
+import importlib
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import dev, rel_err, to_dev_bits
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def synth(t12):
+    return importlib.import_module("turbo_lossless_amd.synth")
+
+
+def run_gemm(t12, packs, X, patched=True):
+    dts = [t12.DeviceTensor12.from_packed(p, dev()) for p in packs]
+    Xd = to_dev_bits(X).reshape(X.shape)
+    outs = t12.gemm(dts, Xd, patched=patched)
+    torch.cuda.synchronize()
+    return [o.cpu().numpy() for o in outs]
+
+
+@pytest.mark.parametrize("B", [1, 7, 16, 32, 33, 64, 100, 128, 129, 200, 256, 300, 512])
+def test_gemm_batches(t12, oracle, synth, B):
+    M, K = 300, 1024
+    p = oracle.pack(synth.weights_llm(M, K, seed=B, p_outlier=2e-3))
+    X = synth.activations(B, K, seed=100 + B)
+    (got,) = run_gemm(t12, [p], X)
+    assert got.shape == (B, M)
+    assert rel_err(got, oracle.gemm(p, X)) < TOL
+
+
+@pytest.mark.parametrize("M,K,B", [(4096, 4096, 16), (1024, 4096, 64), (512, 14336, 256), (1280, 5120, 64),
+                                   (5120, 1280, 64), (129, 64, 5), (1, 128, 256)])
+def test_gemm_shapes(t12, oracle, synth, M, K, B):
+    gen = synth.weights_diffusion if K in (5120, 1280) else synth.weights_llm
+    p = oracle.pack(gen(M, K, seed=M + K))
+    X = synth.activations(B, K, seed=B)
+    (got,) = run_gemm(t12, [p], X)
+    assert rel_err(got, oracle.gemm(p, X)) < TOL
+    (un,) = run_gemm(t12, [p], X, patched=False)
+    assert rel_err(un, oracle.gemm(p, X, patched=False)) < TOL
+
+
+def test_gemm_ksplit_values_agree(t12, oracle, synth):
+    M, K, B = 256, 4096, 96
+    p = oracle.pack(synth.weights_llm(M, K, seed=5, p_outlier=1e-3))
+    X = synth.activations(B, K, seed=6)
+    ref = oracle.gemm(p, X)
+    try:
+        for ks in (1, 2, 3, 4, 8, 16):
+            t12.check(t12.lib.t12_tune_gemm(ks))
+            (got,) = run_gemm(t12, [p], X)
+            assert rel_err(got, ref) < TOL, ks
+    finally:
+        t12.lib.t12_tune_gemm(0)
+
+
+def test_gemm_fused_segments_and_strides(t12, oracle, synth):
+    """Three tensors with three base_exp in one launch; activations with a padded row stride;
+    outputs written into column slices of one [B, sum M] buffer (out_stride > M)."""
+    K, B = 2048, 48
+    ps = [oracle.pack(synth.weights_llm(512, K, seed=1, sigma=0.02)),
+          oracle.pack(synth.weights_llm(130, K, seed=2, sigma=0.3)),
+          oracle.pack(synth.weights_llm(128, K, seed=3, sigma=0.002))]
+    X = synth.activations(B, K, seed=4)
+    Xpad = torch.zeros((B, K + 64), dtype=torch.int16, device=dev())
+    Xpad[:, :K] = to_dev_bits(X).reshape(B, K)
+    dts = [t12.DeviceTensor12.from_packed(p, dev()) for p in ps]
+    total = sum(p.M for p in ps)
+    big = torch.full((B, total), float("nan"), device=dev())
+    outs, c = [], 0
+    for p in ps:
+        outs.append(big[:, c:c + p.M]); c += p.M
+    t12.gemm(dts, Xpad[:, :K], outs=outs)
+    torch.cuda.synchronize()
+    c = 0
+    for p in ps:
+        assert rel_err(big[:, c:c + p.M].cpu().numpy(), oracle.gemm(p, X)) < TOL
+        c += p.M
+
+
+def test_gemm_general_path(t12, oracle, synth, golden):
+    rng = np.random.default_rng(8)
+    for name in ("oddK_3x5", "zeros_4x32", "low_exp_3x32", "tie_2x30", "outliers_16x256", "llm_64x512"):
+        g = golden[name]
+        p = oracle.pack(g["w"], int(g["base_exp"]))
+        X = oracle.f32_to_bf16_bits(rng.standard_normal((11, p.K)).astype(np.float32)).reshape(11, p.K)
+        (got,) = run_gemm(t12, [p], X)
+        assert rel_err(got, oracle.gemm(p, X)) < TOL, name
+
+
+def test_gemm_matches_gemv_at_b1(t12, oracle, synth):
+    M, K = 700, 4096
+    p = oracle.pack(synth.weights_llm(M, K, seed=77))
+    x = synth.activations(1, K, seed=78)
+    (g,) = run_gemm(t12, [p], x)
+    dt = t12.DeviceTensor12.from_packed(p, dev())
+    (v,) = t12.gemv(dt, to_dev_bits(x[0]))
+    torch.cuda.synchronize()
+    assert rel_err(g[0], v.cpu().numpy()) < 1e-5
+
+
+def test_full_size_linearity_b256(t12, oracle, synth):
+    """Full Llama O-projection shape at B=256: rows of X that are copies of one another must give
+    identical output rows, and X with disjoint halves must add up (size-independent properties)."""
+    M, K, B = 4096, 4096, 256
+    w = synth.weights_llm(M, K, seed=2003)
+    p = oracle.pack(w)
+    x = synth.activations(2, K, seed=9)
+    X = np.repeat(x, B // 2, axis=0)
+    (got,) = run_gemm(t12, [p], X)
+    assert np.array_equal(got[0], got[B // 2 - 1]) and np.array_equal(got[B // 2], got[B - 1])
+    ref = oracle.gemm(p, x)
+    assert rel_err(got[[0, B - 1]], ref) < TOL
+
+
+def test_gemm_rejects_bad_operands(t12):
+    segs = (t12.Segment * 1)(t12.Segment(None, None, None, None, None, None, None, 4, 100))
+    x = torch.zeros(64, dtype=torch.int16, device=dev())
+    assert t12.lib.t12_gemm(segs, 1, x.data_ptr(), 64, 4, 64, 1, None) == -1
+    assert t12.lib.t12_gemm(segs, 1, x.data_ptr(), 32, 4, 64, 1, None) == -1

@@ -48,6 +48,8 @@ _SIGS = {
     "t12_pack_row_offsets": (_i, [_vp, _i, _vp, _vp]),
     "t12_pack_escapes": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "t12_gemv": (_i, [C.POINTER(Segment), _i, _vp, _i, _vp]),
+    "t12_gemm": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
+    "t12_tune_gemm": (_i, [_i]),
     "t12_decompress": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "launch_split12_v2_async": (_i, [_vp, _vp, _i, _vp, _vp, _i, _i, _vp]),
     "launch_split12_v2_dual_async": (_i, [_vp, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _vp]),
@@ -131,6 +133,23 @@ def gemv(tensors, act, outs=None, patched=True, stream=None):
     segs = _seg_array([t.segment(o, patched) for t, o in zip(tensors, outs)])
     st = current_stream() if stream is None else stream
     check(lib.t12_gemv(segs, len(tensors), act.data_ptr(), K, st), "t12_gemv")
+    return outs
+
+
+def gemm(tensors, X, outs=None, patched=True, stream=None):
+    """Fused decode+GEMM: X is bf16 [B, K] (row stride = X.stride(0)); returns fp32 [B, M] per tensor."""
+    torch = _torch()
+    if isinstance(tensors, DeviceTensor12):
+        tensors = [tensors]
+    B, K = X.shape
+    assert K == tensors[0].K and X.stride(1) == 1
+    if outs is None:
+        outs = [torch.empty((B, t.M), dtype=torch.float32, device=X.device) for t in tensors]
+    stride = outs[0].stride(0)
+    assert all(o.stride(0) == stride for o in outs)
+    segs = _seg_array([t.segment(o, patched) for t, o in zip(tensors, outs)])
+    st = current_stream() if stream is None else stream
+    check(lib.t12_gemm(segs, len(tensors), X.data_ptr(), X.stride(0), stride, K, B, st), "t12_gemm")
     return outs
 
 

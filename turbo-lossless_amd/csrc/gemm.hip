@@ -1,0 +1,459 @@
+// Split-12 fused decode + GEMM on CDNA4 matrix cores (gfx950).
+//
+//   out_s[b*out_stride + m] = sum_k dec(W_s[m,k]) * X[b*act_stride + k]
+//
+// the function of the reference's split12_fused_gemm V1/V2/V3
+// (split12_gemm.cuh:99-288, split12_gemm_v2.cuh:86-240, split12_gemm_v3.cuh:111-253)
+// plus nv_apply_patches_batch (nvidia_kernels.cu:295-319), re-designed for
+// wave64 MFMA instead of warp-level mma.sync:
+//
+//   * v_mfma_f32_32x32x16_bf16, activations as the A operand (rows = batch),
+//     weights as the B operand (columns = output features), so that an
+//     accumulator register holds 32 consecutive m of one batch row and the
+//     stores to out[b, m] coalesce without a transpose through LDS.
+//   * The whole batch tile (up to 256 rows) lives in one workgroup: every
+//     weight byte is fetched once per launch (the reference re-decodes per
+//     batch tile, nvidia_kernels.cu:456).
+//   * The compressed planes are staged global -> LDS as they are (1.5 B per
+//     weight) and rebuilt to bf16 in registers, two weights per VGPR
+//     (t12_decode8), straight into the MFMA B operand: no bf16 copy of W ever
+//     exists in LDS or HBM.  The activations are staged already paired the way
+//     t12_decode8 orders its outputs, so no operand shuffling is needed.
+//   * Waves are laid out WB x WM; a wave owns FB x FM 32x32 accumulator tiles.
+//     B <= 128 uses 1 x 4 waves (each weight decoded once per workgroup);
+//     B <= 256 uses 2 x 2 waves with 4 x 2 tiles (128 accumulator VGPRs).
+//   * Few row tiles (small M) are split along K across workgroups; the partial
+//     sums go to a workspace and a second kernel adds them in a fixed order
+//     (deterministic) together with the escape corrections.
+//   * Escapes: the streamed value of a group-0 weight is the "wrong" value; the
+//     epilogue kernel adds (correct - wrong) * X[b, col] for every batch row.
+//
+// Fast path requirements: K % 64 == 0, 0 <= base_exp <= 240, 16-byte aligned
+// activation rows.  Everything else goes to the general kernel below.
+
+#include "t12_device.h"
+#include "t12_host.h"
+
+namespace {
+
+constexpr int KC = 64;          // K columns staged per pipeline stage
+constexpr int TM = 128;         // weight rows per workgroup
+
+struct GemmParams {
+    T12Segment seg[T12_MAX_SEGMENTS];
+    int blk_start[T12_MAX_SEGMENTS + 1];   // first row-tile of each segment
+    int seg_row0[T12_MAX_SEGMENTS];        // first row of each segment in the workspace
+    int nseg;
+    int K, B;
+    int act_stride, out_stride;
+    int ksplit;                            // workgroups along K
+    int kslice;                            // columns per K split (multiple of KC)
+    int m_total;                           // sum of M over segments (workspace row length)
+    const uint16_t* act;
+    float* ws;                             // [ksplit][B][m_total] partial sums when ksplit > 1
+};
+
+__device__ __forceinline__ int find_segment(const GemmParams& p, int tile)
+{
+    int s = 0;
+#pragma unroll
+    for (int i = 1; i < T12_MAX_SEGMENTS; i++)
+        if (i < p.nseg && tile >= p.blk_start[i]) s = i;
+    return s;
+}
+
+// ---------------------------------------------------------------------------
+// LDS stage layout (one of two buffers):
+//   act  [8 units][TB rows] x 16 B   unit u = (k % 64) / 8, eight bf16 paired by
+//                                     t12_pair_acts
+//   sm   [4 units][TM rows] x 16 B   unit c = (k % 64) / 16
+//   gr   [4 units][TM rows] x  8 B
+// Consecutive lanes read consecutive rows of one unit: conflict free.
+// One 32-column block q of a stage feeds two MFMA k-steps s = 0, 1; MFMA slot
+// (half h of the wave, element j) stands for column 32q + 16h + 8s + j.
+// ---------------------------------------------------------------------------
+template <int WB, int WM, int FB, int FM>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
+{
+    constexpr int TB = WB * FB * 32;                  // batch rows per workgroup
+    static_assert(WB * WM == 4, "four waves per workgroup");
+    static_assert(WM * FM * 32 == TM, "row tile is 128");
+    constexpr int ACT_UNITS = TB * 8;                 // 16-byte units per stage
+    constexpr int ACT_LD = ACT_UNITS / 256;           // per thread
+    constexpr int STAGE_BYTES = ACT_UNITS * 16 + TM * 64 + TM * 32;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wb = wave / WM, wm = wave % WM;
+    const int ln = lane & 31, lh = lane >> 5;
+
+    const int tile = blockIdx.x;
+    const int s = find_segment(p, tile);
+    const T12Segment& sg = p.seg[s];
+    const int M = sg.M, K = p.K, B = p.B;
+    const int m0 = (tile - p.blk_start[s]) * TM;
+    const int b0 = blockIdx.y * TB;
+    const int k_begin = blockIdx.z * p.kslice;
+    const int k_end = min(K, k_begin + p.kslice);
+    const int nstage = (k_end - k_begin) / KC;
+    const uint32_t be2 = ((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23);
+
+    // ---- this thread's share of the global -> LDS staging
+    //  acts: unit idx = tid + 256*i -> row idx / 8, unit idx % 8 (8 lanes = 128 contiguous bytes)
+    //  sm / gr: unit idx = tid + 256*i (i < 2) -> row idx / 4, unit idx % 4
+    const uint16_t* a_src[ACT_LD];
+    int a_dst[ACT_LD];
+    bool a_ok[ACT_LD];
+#pragma unroll
+    for (int i = 0; i < ACT_LD; i++) {
+        const int idx = tid + 256 * i;
+        const int r = idx >> 3, u = idx & 7;
+        a_ok[i] = b0 + r < B;
+        a_src[i] = p.act + (size_t)min(b0 + r, B - 1) * p.act_stride + k_begin + u * 8;
+        a_dst[i] = (u * TB + r) * 16;
+    }
+    const uint8_t* s_src[2];
+    const uint8_t* g_src[2];
+    int s_dst[2], g_dst[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int idx = tid + 256 * i;
+        const int r = idx >> 2, c = idx & 3;
+        const size_t e = (size_t)min(m0 + r, M - 1) * K + k_begin;      // clamp: loads stay in bounds
+        s_src[i] = sg.sm + e + c * 16;
+        g_src[i] = sg.gr + (e >> 1) + c * 8;
+        s_dst[i] = ACT_UNITS * 16 + (c * TM + r) * 16;
+        g_dst[i] = ACT_UNITS * 16 + TM * 64 + (c * TM + r) * 8;
+    }
+
+    uint4 ra[ACT_LD];
+    uint4 rs[2];
+    uint2 rg[2];
+    auto load_stage = [&](int st) {
+#pragma unroll
+        for (int i = 0; i < ACT_LD; i++) {
+            ra[i] = make_uint4(0, 0, 0, 0);
+            if (a_ok[i]) ra[i] = *(const uint4*)(a_src[i] + (size_t)st * KC);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            rs[i] = t12_ldg_stream16(s_src[i] + (size_t)st * KC);
+            rg[i] = t12_ldg_stream8(g_src[i] + (size_t)st * (KC / 2));
+        }
+    };
+    auto store_stage = [&](int buf) {
+        uint8_t* base = lds + buf * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < ACT_LD; i++) *(uint4*)(base + a_dst[i]) = t12_pair_acts(ra[i]);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            *(uint4*)(base + s_dst[i]) = rs[i];
+            *(uint2*)(base + g_dst[i]) = rg[i];
+        }
+    };
+
+    t12_f32x16 acc[FB][FM];
+#pragma unroll
+    for (int i = 0; i < FB; i++)
+#pragma unroll
+        for (int j = 0; j < FM; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    if (nstage > 0) {
+        load_stage(0);
+        store_stage(0);
+    }
+    __syncthreads();
+
+    for (int st = 0; st < nstage; st++) {
+        const int buf = st & 1;
+        if (st + 1 < nstage) load_stage(st + 1);          // global loads fly under the MFMAs
+
+        const uint8_t* base = lds + buf * STAGE_BYTES;
+        const uint4* lact = (const uint4*)base;
+        const uint4* lsm = (const uint4*)(base + ACT_UNITS * 16);
+        const uint2* lgr = (const uint2*)(base + ACT_UNITS * 16 + TM * 64);
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            uint32_t wf[FM][2][4];
+#pragma unroll
+            for (int j = 0; j < FM; j++) {
+                const int row = (wm * FM + j) * 32 + ln;
+                const uint4 S = lsm[(2 * q + lh) * TM + row];
+                const uint2 G = lgr[(2 * q + lh) * TM + row];
+                t12_decode8(S.x, S.y, G.x, be2, wf[j][0]);
+                t12_decode8(S.z, S.w, G.y, be2, wf[j][1]);
+            }
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+                for (int i = 0; i < FB; i++) {
+                    const int brow = (wb * FB + i) * 32 + ln;
+                    const uint4 A = lact[(4 * q + 2 * lh + ks) * TB + brow];
+                    const t12_bf16x8 av = __builtin_bit_cast(t12_bf16x8, A);
+#pragma unroll
+                    for (int j = 0; j < FM; j++) {
+                        const uint4 Wv = make_uint4(wf[j][ks][0], wf[j][ks][1], wf[j][ks][2], wf[j][ks][3]);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            av, __builtin_bit_cast(t12_bf16x8, Wv), acc[i][j], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        if (st + 1 < nstage) store_stage(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: accumulator register r of lane (ln, lh) is
+    //      D[row = 8*(r/4) + 4*lh + r%4][col = ln]   (row = batch, col = m)
+    float* dst;
+    size_t ld;
+    int col_off;
+    if (p.ksplit > 1) {
+        dst = p.ws + (size_t)blockIdx.z * B * p.m_total;
+        ld = p.m_total;
+        col_off = p.seg_row0[s];
+    } else {
+        dst = sg.out;
+        ld = p.out_stride;
+        col_off = 0;
+    }
+#pragma unroll
+    for (int i = 0; i < FB; i++)
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            const int m = m0 + (wm * FM + j) * 32 + ln;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int b = b0 + (wb * FB + i) * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                if (m < M && b < B) dst[(size_t)b * ld + col_off + m] = acc[i][j][r];
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------
+// Epilogue kernel: out[b, m] = sum over K splits of the partials (fixed order)
+// + escape corrections.  One workgroup per (row block of 64 m, batch row b).
+// With ksplit == 1 only the corrections are added (rows without escapes are
+// left untouched).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void gemm_epilogue_kernel(const GemmParams p)
+{
+    const int tile = blockIdx.x;            // 64-row blocks; blk_start here counts 64-row blocks
+    const int s = find_segment(p, tile);
+    const T12Segment& sg = p.seg[s];
+    const int m = (tile - p.blk_start[s]) * 64 + threadIdx.x;
+    const int b = blockIdx.y;
+    if (m >= sg.M) return;
+    float v;
+    bool dirty = false;
+    if (p.ksplit > 1) {
+        v = 0.0f;
+        for (int z = 0; z < p.ksplit; z++)
+            v += p.ws[((size_t)z * p.B + b) * p.m_total + p.seg_row0[s] + m];
+        dirty = true;
+    } else {
+        v = 0.0f;
+    }
+    if (sg.row_off) {
+        const int beg = sg.row_off[m], end = sg.row_off[m + 1];
+        if (end > beg) {
+            if (!dirty) v = sg.out[(size_t)b * p.out_stride + m];
+            const uint16_t* x = p.act + (size_t)b * p.act_stride;
+            for (int q = beg; q < end; q++)
+                v += (t12_bf16_to_f32((uint16_t)sg.correct[q]) - t12_bf16_to_f32((uint16_t)sg.wrong[q])) *
+                     t12_bf16_to_f32(x[sg.cols[q]]);
+            dirty = true;
+        }
+    }
+    if (dirty) sg.out[(size_t)b * p.out_stride + m] = v;
+}
+
+// ---------------------------------------------------------------------------
+// General path: any K, any base_exp, any alignment.  One wave per (row, 8
+// batch rows); scalar decode rule; escapes exact from the CSR list.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void gemm_general_kernel(const GemmParams p)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int tile = blockIdx.x;            // blk_start counts 4-row blocks
+    const int s = find_segment(p, tile);
+    const T12Segment& sg = p.seg[s];
+    const int row = (tile - p.blk_start[s]) * 4 + wave;
+    if (row >= sg.M) return;
+    const int b0 = blockIdx.y * 8;
+    const int nb = min(8, p.B - b0);
+    const int K = p.K;
+    const size_t base = (size_t)row * K;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int k = lane; k < K; k += T12_WAVE) {
+        const size_t i = base + k;
+        const uint32_t g = (sg.gr[i >> 1] >> (4 * (i & 1))) & 0xFu;
+        if (g == 0 && sg.row_off) continue;            // taken from the list below
+        const float w = t12_bf16_to_f32(t12_decode_scalar(sg.sm[i], g, sg.base_exp));
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (j < nb) acc[j] += w * t12_bf16_to_f32(p.act[(size_t)(b0 + j) * p.act_stride + k]);
+    }
+    if (sg.row_off) {
+        const int beg = sg.row_off[row], end = sg.row_off[row + 1];
+        for (int q = beg + lane; q < end; q += T12_WAVE) {
+            const float w = t12_bf16_to_f32((uint16_t)sg.correct[q]);
+            const int k = sg.cols[q];
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                if (j < nb) acc[j] += w * t12_bf16_to_f32(p.act[(size_t)(b0 + j) * p.act_stride + k]);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float v = t12_wave_sum(acc[j]);
+        if (lane == 0 && j < nb) sg.out[(size_t)(b0 + j) * p.out_stride + row] = v;
+    }
+}
+
+// ---- workspace for the K-split partial sums (grown on demand, per device) ----
+float* g_ws[16] = {};
+size_t g_ws_bytes[16] = {};
+
+float* workspace(size_t bytes)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
+    if (g_ws_bytes[dev] < bytes) {
+        if (g_ws[dev]) (void)hipFree(g_ws[dev]);
+        g_ws[dev] = nullptr;
+        g_ws_bytes[dev] = 0;
+        if (hipMalloc((void**)&g_ws[dev], bytes) != hipSuccess) return nullptr;
+        g_ws_bytes[dev] = bytes;
+    }
+    return g_ws[dev];
+}
+
+int g_gemm_ksplit = 0;   // 0 = choose by shape
+
+template <int WB, int WM, int FB, int FM>
+int launch_mfma(GemmParams& p, int tiles, hipStream_t st)
+{
+    constexpr int TB = WB * FB * 32;
+    constexpr int STAGE_BYTES = TB * 8 * 16 + TM * 64 + TM * 32;
+    const dim3 grid(tiles, (p.B + TB - 1) / TB, p.ksplit);
+    auto kfn = gemm_mfma_kernel<WB, WM, FB, FM>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE_BYTES) !=
+            hipSuccess) {
+            t12_set_error("t12_gemm: cannot reserve %d bytes of LDS", 2 * STAGE_BYTES);
+            return T12_ELAUNCH;
+        }
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kfn, grid, dim3(256), 2 * STAGE_BYTES, st, p);
+    T12_CHECK_LAUNCH("t12_gemm");
+    return T12_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+// Pins the number of K splits of the MFMA path (benchmark sweeps); 0 = by shape.
+int t12_tune_gemm(int ksplit)
+{
+    g_gemm_ksplit = ksplit;
+    return T12_OK;
+}
+
+int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride, int out_stride, int K, int B,
+             void* stream)
+{
+    T12_REQUIRE(segs && nseg >= 1 && nseg <= T12_MAX_SEGMENTS, "t12_gemm: nseg must be 1..%d (got %d)",
+                T12_MAX_SEGMENTS, nseg);
+    T12_REQUIRE(act_bf16 && K >= 1 && B >= 1, "t12_gemm: activations null or K/B < 1 (K=%d B=%d)", K, B);
+    T12_REQUIRE(act_stride >= K, "t12_gemm: act_stride %d < K %d", act_stride, K);
+    hipStream_t st = (hipStream_t)stream;
+    GemmParams p;
+    p.nseg = nseg;
+    p.K = K;
+    p.B = B;
+    p.act_stride = act_stride;
+    p.out_stride = out_stride;
+    p.act = (const uint16_t*)act_bf16;
+    p.ws = nullptr;
+    bool fast = (K % KC == 0) && (act_stride % 8 == 0) && ((uintptr_t)act_bf16 % 16 == 0);
+    int m_total = 0, any_patch = 0;
+    for (int i = 0; i < nseg; i++) {
+        const T12Segment& g = segs[i];
+        T12_REQUIRE(g.M >= 1 && g.sm && g.gr && g.out, "t12_gemm: segment %d has M < 1 or a null pointer", i);
+        T12_REQUIRE(out_stride >= g.M, "t12_gemm: out_stride %d < M %d of segment %d", out_stride, g.M, i);
+        T12_REQUIRE(!g.row_off || (g.cols && g.correct && g.wrong), "t12_gemm: segment %d: row_off without lists", i);
+        T12_REQUIRE(g.base_exp >= -1 && g.base_exp <= 254, "t12_gemm: segment %d: base_exp %d out of range", i,
+                    g.base_exp);
+        if (g.base_exp < 0 || g.base_exp > 240) fast = false;
+        if (g.row_off) any_patch = 1;
+        p.seg[i] = g;
+        p.seg_row0[i] = m_total;
+        m_total += g.M;
+    }
+    p.m_total = m_total;
+
+    if (!fast) {
+        int tiles = 0;
+        for (int i = 0; i < nseg; i++) {
+            p.blk_start[i] = tiles;
+            tiles += (segs[i].M + 3) / 4;
+        }
+        p.blk_start[nseg] = tiles;
+        p.ksplit = 1;
+        p.kslice = K;
+        hipLaunchKernelGGL(gemm_general_kernel, dim3(tiles, (B + 7) / 8), dim3(256), 0, st, p);
+        T12_CHECK_LAUNCH("t12_gemm(general)");
+        return T12_OK;
+    }
+
+    int tiles = 0;
+    for (int i = 0; i < nseg; i++) {
+        p.blk_start[i] = tiles;
+        tiles += (segs[i].M + TM - 1) / TM;
+    }
+    p.blk_start[nseg] = tiles;
+    // K split: aim at >= 256 workgroups (one per CU) while every split keeps >= 8 stages
+    const int btiles = (B + 255) / 256;
+    int ks = 1;
+    if (g_gemm_ksplit > 0) ks = g_gemm_ksplit;
+    else
+        while (tiles * btiles * ks < 192 && K / (ks * 2) >= 8 * KC && ks < 16) ks *= 2;
+    int kslice = ((K / KC + ks - 1) / ks) * KC;
+    ks = (K + kslice - 1) / kslice;
+    p.ksplit = ks;
+    p.kslice = kslice;
+    if (ks > 1) {
+        p.ws = workspace((size_t)ks * B * m_total * sizeof(float));
+        if (!p.ws) {
+            t12_set_error("t12_gemm: cannot allocate %zu bytes of K-split workspace",
+                          (size_t)ks * B * m_total * sizeof(float));
+            return T12_ELAUNCH;
+        }
+    }
+    int rc;
+    if (B <= 32) rc = launch_mfma<1, 4, 1, 1>(p, tiles, st);
+    else if (B <= 64) rc = launch_mfma<1, 4, 2, 1>(p, tiles, st);
+    else if (B <= 128) rc = launch_mfma<1, 4, 4, 1>(p, tiles, st);
+    else rc = launch_mfma<2, 2, 4, 2>(p, tiles, st);
+    if (rc) return rc;
+
+    if (ks > 1 || any_patch) {
+        int t64 = 0;
+        for (int i = 0; i < nseg; i++) {
+            p.blk_start[i] = t64;
+            t64 += (segs[i].M + 63) / 64;
+        }
+        p.blk_start[nseg] = t64;
+        hipLaunchKernelGGL(gemm_epilogue_kernel, dim3(t64, B), dim3(64), 0, st, p);
+        T12_CHECK_LAUNCH("t12_gemm(epilogue)");
+    }
+    return T12_OK;
+}
+
+}  // extern "C"
