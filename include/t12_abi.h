@@ -52,6 +52,8 @@ typedef struct T12Segment {
     float*         out;        /* this tensor's output base: out[b*out_stride + m] */
     int32_t        M;
     int32_t        base_exp;
+    int32_t        out_stride; /* row stride of `out` for B > 1; 0 = the call's out_stride */
+    int32_t        reserved;   /* must be 0 */
 } T12Segment;
 
 /* ---- library ------------------------------------------------------------- */

@@ -259,3 +259,65 @@ def argmax_first(logits: np.ndarray) -> int:
     """Index of the maximum logit; lowest index among exact ties (kernels.hip:90-122
     resolves ties by thread id; the rewrite fixes the rule to lowest index)."""
     return int(np.argmax(logits))
+
+
+# ------------------------------------------------------------ whole decode step
+class RefModel:
+    """CPU restatement of one decode step at B = 1: the layer wiring of the reference's forward_b1
+    (engine/inference.cpp:198-366) over the oracle's decode-then-fp32 GEMV and glue formulas.
+    For small models only (pure numpy between the C GEMVs)."""
+
+    def __init__(self, cfg, embd_bits, output_norm, output_proj, layers, max_seq):
+        self.cfg = dict(cfg)
+        self.embd = np.asarray(embd_bits, np.uint16).reshape(cfg["n_vocab"], cfg["n_embd"])
+        self.output_norm = np.asarray(output_norm, np.float32)
+        self.output_proj = output_proj
+        self.layers = layers
+        self.hd = cfg["n_embd"] // cfg["n_head"]
+        nl, nkv = cfg["n_layer"], cfg["n_head_kv"]
+        self.kc = np.zeros((nl, max_seq, nkv, self.hd), np.int8)
+        self.vc = np.zeros((nl, max_seq, nkv, self.hd), np.int8)
+        self.ks = np.zeros((nl, max_seq, nkv), np.float32)
+        self.vs = np.zeros((nl, max_seq, nkv), np.float32)
+
+    def step(self, token: int, pos: int) -> np.ndarray:
+        c = self.cfg
+        nh, nkv, hd, eps, theta = c["n_head"], c["n_head_kv"], self.hd, c["rms_norm_eps"], c["rope_theta"]
+        cur = embed_lookup(self.embd, [token], c["n_vocab"])[0]
+        a = None
+        for li, L in enumerate(self.layers):
+            if li == 0:
+                a = rms_norm_bf16(cur, L["attn_norm"], eps)
+            q = gemv(L["wq"], a)
+            k = gemv(L["wk"], a)
+            v = gemv(L["wv"], a)
+            q = rope(q, pos, nh, hd, theta)
+            k = rope(k, pos, nkv, hd, theta)
+            self.kc[li, pos], self.ks[li, pos] = quant_kv_int8(k, nkv, hd)
+            self.vc[li, pos], self.vs[li, pos] = quant_kv_int8(v, nkv, hd)
+            att = attention_int8(q, self.kc[li], self.vc[li], self.ks[li], self.vs[li], pos + 1, nh, nkv, hd)
+            res = gemv(L["wo"], att)
+            res, a = add_rms_norm_bf16(res, cur, L["ffn_norm"], eps)
+            b = silu_mul_bf16(gemv(L["w_gate"], a), gemv(L["w_up"], a))
+            cur = gemv(L["w_down"], b)
+            nxt = self.layers[li + 1]["attn_norm"] if li + 1 < len(self.layers) else self.output_norm
+            cur, a = add_rms_norm_bf16(cur, res, nxt, eps)
+        if not self.layers:
+            a = rms_norm_bf16(cur, self.output_norm, eps)
+        return gemv(self.output_proj, a)
+
+    def generate(self, prompt, max_tokens, eos=2):
+        """generate() of engine/inference.cpp:716-730 (greedy, stops at token id 2)."""
+        logits = None
+        for i, t in enumerate(prompt):
+            logits = self.step(int(t), i)
+        pos = len(prompt)
+        out = []
+        for _ in range(max_tokens):
+            nxt = argmax_first(logits)
+            if nxt == eos:
+                break
+            out.append(nxt)
+            logits = self.step(nxt, pos)
+            pos += 1
+        return out

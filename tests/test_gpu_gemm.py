@@ -125,7 +125,7 @@ def test_full_size_linearity_b256(t12, oracle, synth):
 
 
 def test_gemm_rejects_bad_operands(t12):
-    segs = (t12.Segment * 1)(t12.Segment(None, None, None, None, None, None, None, 4, 100))
+    segs = (t12.Segment * 1)(t12.Segment(None, None, None, None, None, None, None, 4, 100, 0, 0))
     x = torch.zeros(64, dtype=torch.int16, device=dev())
     assert t12.lib.t12_gemm(segs, 1, x.data_ptr(), 64, 4, 64, 1, None) == -1
     assert t12.lib.t12_gemm(segs, 1, x.data_ptr(), 32, 4, 64, 1, None) == -1

@@ -172,7 +172,7 @@ def test_reference_named_launchers(t12, oracle, synth):
 
 
 def test_gemv_rejects_bad_operands(t12):
-    segs = (t12.Segment * 1)(t12.Segment(None, None, None, None, None, None, None, 4, 100))
+    segs = (t12.Segment * 1)(t12.Segment(None, None, None, None, None, None, None, 4, 100, 0, 0))
     x = torch.zeros(16, dtype=torch.int16, device=dev())
     assert t12.lib.t12_gemv(segs, 1, x.data_ptr(), 16, None) == -1
     assert b"null" in t12.lib.t12_last_error()

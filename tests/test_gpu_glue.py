@@ -1,0 +1,196 @@
+"""GPU parity: engine glue launchers (reference names/signatures) vs the oracle's closed forms.
+
+bf16 outputs: the kernels round fp32 results to bf16; the oracle computes the same formulas in
+float64/float32, so an output may differ by one bf16 ulp where the fp32 value sits next to a rounding
+boundary.  Assertions: every element within 1 bf16 ulp and >= 99 % bit-identical."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import dev
+
+pytestmark = pytest.mark.gpu
+
+
+def st(t12):
+    return t12.current_stream()
+
+
+def bf16_close(got_bits, ref_bits, frac=0.99):
+    g = got_bits.astype(np.uint16).view(np.int16).astype(np.int32)
+    r = ref_bits.astype(np.uint16).view(np.int16).astype(np.int32)
+    # bf16 bit patterns are monotone in magnitude per sign; compare as sign-magnitude integers
+    gi = np.where(g < 0, -(g & 0x7FFF), g)
+    ri = np.where(r < 0, -(r & 0x7FFF), r)
+    assert np.abs(gi - ri).max() <= 1
+    assert (g == r).mean() >= frac
+
+
+def test_embed_lookup(t12, oracle):
+    rng = np.random.default_rng(0)
+    V, n = 50, 96
+    embd = oracle.f32_to_bf16_bits(rng.standard_normal((V, n)).astype(np.float32)).reshape(V, n)
+    toks = [3, 49, 0, -1, 50]
+    e = torch.from_numpy(embd.view(np.int16)).to(dev())
+    t = torch.tensor(toks, dtype=torch.int32, device=dev())
+    out = torch.full((len(toks), n), 7.0, device=dev())
+    t12.lib.launch_embed_lookup(e.data_ptr(), t.data_ptr(), out.data_ptr(), n, len(toks), V, st(t12))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), oracle.embed_lookup(embd, toks, V))
+
+
+@pytest.mark.parametrize("n,B", [(4096, 1), (4096, 5), (256, 3), (14336, 2), (100, 1)])
+def test_rms_norm_and_add(t12, oracle, n, B):
+    rng = np.random.default_rng(n + B)
+    x = rng.standard_normal((B, n)).astype(np.float32) * 3
+    r = rng.standard_normal((B, n)).astype(np.float32)
+    w = (1 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    xd, rd, wd = (torch.from_numpy(a).to(dev()) for a in (x, r, w))
+    y = torch.zeros((B, n), dtype=torch.int16, device=dev())
+    t12.lib.launch_rms_norm_bf16_batch(xd.data_ptr(), wd.data_ptr(), y.data_ptr(), n, 1e-5, B, st(t12))
+    torch.cuda.synchronize()
+    bf16_close(y.cpu().numpy().view(np.uint16), oracle.rms_norm_bf16(x, w, 1e-5).reshape(B, n))
+    assert np.array_equal(xd.cpu().numpy(), x)
+    t12.lib.launch_add_rms_norm_bf16_batch(xd.data_ptr(), rd.data_ptr(), wd.data_ptr(), y.data_ptr(), n, 1e-5, B, st(t12))
+    torch.cuda.synchronize()
+    s, yb = oracle.add_rms_norm_bf16(x, r, w, 1e-5)
+    assert np.array_equal(xd.cpu().numpy(), s)          # x += residual, exact in fp32
+    bf16_close(y.cpu().numpy().view(np.uint16), yb.reshape(B, n))
+
+
+def test_silu_mul_and_add(t12, oracle):
+    rng = np.random.default_rng(2)
+    for (n, B) in [(14336, 2), (1001, 3)]:
+        g = rng.standard_normal((B, n)).astype(np.float32) * 4
+        u = rng.standard_normal((B, n)).astype(np.float32)
+        gd, ud = torch.from_numpy(g).to(dev()), torch.from_numpy(u).to(dev())
+        o = torch.zeros((B, n), dtype=torch.int16, device=dev())
+        t12.lib.launch_silu_mul_bf16_batch(gd.data_ptr(), ud.data_ptr(), o.data_ptr(), n, B, st(t12))
+        t12.lib.launch_add_batch(gd.data_ptr(), ud.data_ptr(), n, B, st(t12))
+        torch.cuda.synchronize()
+        bf16_close(o.cpu().numpy().view(np.uint16), oracle.silu_mul_bf16(g, u).reshape(B, n), frac=0.98)
+        assert np.array_equal(gd.cpu().numpy(), g + u)
+
+
+def make_qkv(rng, B, nh, nkv, hd):
+    q = rng.standard_normal((B, nh * hd)).astype(np.float32)
+    k = rng.standard_normal((B, nkv * hd)).astype(np.float32)
+    v = rng.standard_normal((B, nkv * hd)).astype(np.float32) * 2
+    return q, k, v
+
+
+@pytest.mark.parametrize("nh,nkv,hd", [(32, 8, 128), (4, 4, 64), (8, 2, 32)])
+def test_rope_store_kv_b1(t12, oracle, nh, nkv, hd):
+    rng = np.random.default_rng(nh)
+    theta, pos, max_seq = 500000.0, 37, 64
+    q, k, v = make_qkv(rng, 1, nh, nkv, hd)
+    qd, kd, vd = (torch.from_numpy(a.copy()).to(dev()) for a in (q, k, v))
+    ck = torch.zeros((max_seq, nkv, hd), dtype=torch.int8, device=dev()); cv = torch.zeros_like(ck)
+    sk = torch.zeros((max_seq, nkv), device=dev()); sv = torch.zeros_like(sk)
+    t12.lib.launch_rope_store_kv(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), ck.data_ptr(), cv.data_ptr(),
+                                 sk.data_ptr(), sv.data_ptr(), hd, nh, nkv, pos, max_seq, theta, st(t12))
+    torch.cuda.synchronize()
+    qr = oracle.rope(q[0], pos, nh, hd, theta); kr = oracle.rope(k[0], pos, nkv, hd, theta)
+    assert np.allclose(qd.cpu().numpy()[0], qr, rtol=1e-5, atol=1e-5)
+    assert np.allclose(kd.cpu().numpy()[0], kr, rtol=1e-5, atol=1e-5)
+    # quantisation is checked on the GPU's own rotated K (rounding boundaries are discontinuous)
+    k8, ks = oracle.quant_kv_int8(kd.cpu().numpy()[0], nkv, hd)
+    v8, vs = oracle.quant_kv_int8(v[0], nkv, hd)
+    assert np.array_equal(ck.cpu().numpy()[pos], k8) and np.array_equal(cv.cpu().numpy()[pos], v8)
+    assert np.allclose(sk.cpu().numpy()[pos], ks, rtol=1e-6) and np.allclose(sv.cpu().numpy()[pos], vs, rtol=1e-6)
+    assert not ck.cpu().numpy()[:pos].any() and not ck.cpu().numpy()[pos + 1:].any()
+
+
+def test_rope_and_store_batch_launchers(t12, oracle):
+    rng = np.random.default_rng(5)
+    nh, nkv, hd, B, theta, max_seq = 8, 2, 64, 3, 10000.0, 40
+    q, k, v = make_qkv(rng, B, nh, nkv, hd)
+    positions = [0, 7, 39]
+    pd = torch.tensor(positions, dtype=torch.int32, device=dev())
+    qd, kd, vd = (torch.from_numpy(a.copy()).to(dev()) for a in (q, k, v))
+    t12.lib.launch_rope_batch(qd.data_ptr(), kd.data_ptr(), pd.data_ptr(), hd, nh, nkv, nh * hd, nkv * hd, theta, B, st(t12))
+    ck = torch.zeros((max_seq, nkv, hd), dtype=torch.int8, device=dev()); cv = torch.zeros_like(ck)
+    sk = torch.zeros((max_seq, nkv), device=dev()); sv = torch.zeros_like(sk)
+    t12.lib.launch_store_kv_batch(kd.data_ptr(), vd.data_ptr(), ck.data_ptr(), cv.data_ptr(), sk.data_ptr(), sv.data_ptr(),
+                                  pd.data_ptr(), nkv * hd, max_seq, nkv, hd, B, st(t12))
+    torch.cuda.synchronize()
+    for b, pos in enumerate(positions):
+        assert np.allclose(qd.cpu().numpy()[b], oracle.rope(q[b], pos, nh, hd, theta), rtol=1e-5, atol=1e-5)
+        k8, ks = oracle.quant_kv_int8(kd.cpu().numpy()[b], nkv, hd)
+        v8, vs = oracle.quant_kv_int8(v[b], nkv, hd)
+        assert np.array_equal(ck.cpu().numpy()[pos], k8) and np.array_equal(cv.cpu().numpy()[pos], v8)
+        assert np.allclose(sv.cpu().numpy()[pos], vs, rtol=1e-6)
+    # the fused batch launcher gives the same cache
+    q2, k2, v2 = (torch.from_numpy(a.copy()).to(dev()) for a in (q, k, v))
+    ck2 = torch.zeros_like(ck); cv2 = torch.zeros_like(cv); sk2 = torch.zeros_like(sk); sv2 = torch.zeros_like(sv)
+    t12.lib.launch_rope_store_kv_batch(q2.data_ptr(), k2.data_ptr(), v2.data_ptr(), ck2.data_ptr(), cv2.data_ptr(),
+                                       sk2.data_ptr(), sv2.data_ptr(), pd.data_ptr(), hd, nh, nkv, nh * hd, nkv * hd,
+                                       theta, B, st(t12))
+    torch.cuda.synchronize()
+    assert torch.equal(ck, ck2) and torch.equal(cv, cv2) and torch.equal(sk, sk2) and torch.equal(q2, qd)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,seq", [(32, 8, 128, 1), (32, 8, 128, 300), (32, 8, 128, 1500), (4, 4, 64, 77),
+                                            (16, 1, 32, 513)])
+def test_attention_b1_both_names(t12, oracle, nh, nkv, hd, seq):
+    rng = np.random.default_rng(seq)
+    max_seq = seq + 3
+    q = rng.standard_normal(nh * hd).astype(np.float32)
+    kc = rng.integers(-127, 128, size=(max_seq, nkv, hd)).astype(np.int8)
+    vc = rng.integers(-127, 128, size=(max_seq, nkv, hd)).astype(np.int8)
+    ks = (rng.random((max_seq, nkv)).astype(np.float32) + 0.5) / 127
+    vs = (rng.random((max_seq, nkv)).astype(np.float32) + 0.5) / 127
+    ref = oracle.attention_int8(q, kc, vc, ks, vs, seq, nh, nkv, hd)
+    d = [torch.from_numpy(a).to(dev()) for a in (q, kc, vc, ks, vs)]
+    for fn in (t12.lib.launch_attention_all_heads, t12.lib.launch_flash_attention):
+        out = torch.zeros(nh * hd, dtype=torch.int16, device=dev())
+        fn(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), d[4].data_ptr(), out.data_ptr(),
+           nh, nkv, hd, seq, max_seq, 1.0 / np.sqrt(hd), st(t12))
+        torch.cuda.synchronize()
+        got = oracle.bf16_bits_to_f32(out.cpu().numpy().view(np.uint16))
+        want = oracle.bf16_bits_to_f32(ref)
+        assert np.abs(got - want).max() <= 2e-2 * np.abs(want).max()   # bf16 output: 2^-8 relative steps
+
+
+def test_attention_batch_shared_and_strided_cache(t12, oracle):
+    rng = np.random.default_rng(9)
+    nh, nkv, hd, B, max_seq = 8, 2, 64, 3, 50
+    positions = [4, 30, 49]
+    q = rng.standard_normal((B, nh * hd)).astype(np.float32)
+    kc = rng.integers(-127, 128, size=(B, max_seq, nkv, hd)).astype(np.int8)
+    vc = rng.integers(-127, 128, size=(B, max_seq, nkv, hd)).astype(np.int8)
+    ks = (rng.random((B, max_seq, nkv)).astype(np.float32) + 0.5) / 127
+    vs = (rng.random((B, max_seq, nkv)).astype(np.float32) + 0.5) / 127
+    d = [torch.from_numpy(a).to(dev()) for a in (q, kc, vc, ks, vs)]
+    pd = torch.tensor(positions, dtype=torch.int32, device=dev())
+    for stride, sel in ((0, lambda b: 0), (max_seq * nkv * hd, lambda b: b)):
+        out = torch.zeros((B, nh * hd), dtype=torch.int16, device=dev())
+        t12.lib.launch_attention_all_heads_batch(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(),
+                                                 d[4].data_ptr(), out.data_ptr(), pd.data_ptr(), nh, nkv, hd,
+                                                 max(positions) + 1, 1.0 / np.sqrt(hd), B, stride, st(t12))
+        torch.cuda.synchronize()
+        for b in range(B):
+            s = sel(b)
+            ref = oracle.attention_int8(q[b], kc[s], vc[s], ks[s], vs[s], positions[b] + 1, nh, nkv, hd)
+            got = oracle.bf16_bits_to_f32(out.cpu().numpy()[b].view(np.uint16))
+            want = oracle.bf16_bits_to_f32(ref)
+            assert np.abs(got - want).max() <= 2e-2 * np.abs(want).max()
+
+
+def test_argmax(t12, oracle):
+    rng = np.random.default_rng(4)
+    for (B, n) in [(1, 128256), (7, 1000), (256, 4099), (1, 5)]:
+        x = rng.standard_normal((B, n)).astype(np.float32)
+        x[0, n // 2] = x[0, n - 1] = 50.0        # exact tie: lowest index wins
+        xd = torch.from_numpy(x).to(dev())
+        r = torch.full((B,), -1, dtype=torch.int32, device=dev())
+        if B == 1:
+            t12.lib.launch_argmax(xd.data_ptr(), r.data_ptr(), n, st(t12))
+        else:
+            t12.lib.launch_argmax_batch(xd.data_ptr(), r.data_ptr(), n, B, st(t12))
+        torch.cuda.synchronize()
+        assert r.cpu().tolist() == [oracle.argmax_first(row) for row in x]
+    nanrow = np.full((1, 300), np.nan, np.float32); nanrow[0, 17] = -3.0
+    xd = torch.from_numpy(nanrow).to(dev()); r = torch.zeros(1, dtype=torch.int32, device=dev())
+    t12.lib.launch_argmax(xd.data_ptr(), r.data_ptr(), 300, st(t12)); torch.cuda.synchronize()
+    assert r.item() == 17

@@ -27,7 +27,7 @@ class Segment(C.Structure):
     """Mirror of T12Segment (include/t12_abi.h)."""
     _fields_ = [("sm", C.c_void_p), ("gr", C.c_void_p), ("row_off", C.c_void_p), ("cols", C.c_void_p),
                 ("correct", C.c_void_p), ("wrong", C.c_void_p), ("out", C.c_void_p),
-                ("M", C.c_int32), ("base_exp", C.c_int32)]
+                ("M", C.c_int32), ("base_exp", C.c_int32), ("out_stride", C.c_int32), ("reserved", C.c_int32)]
 
 
 class PatchBatchDesc(C.Structure):
@@ -48,6 +48,42 @@ _SIGS = {
     "t12_pack_row_offsets": (_i, [_vp, _i, _vp, _vp]),
     "t12_pack_escapes": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "t12_gemv": (_i, [C.POINTER(Segment), _i, _vp, _i, _vp]),
+    "t12_synth_normal_bf16": (_i, [_vp, C.c_size_t, C.c_uint64, C.c_float, C.c_float, C.c_float, _vp]),
+    "t12_fill_f32": (_i, [_vp, C.c_size_t, C.c_float, _vp]),
+    # glue launchers (reference names; void return)
+    "launch_rope_init": (None, [_i, C.c_float]),
+    "launch_embed_lookup": (None, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "launch_rms_norm_bf16_batch": (None, [_vp, _vp, _vp, _i, C.c_float, _i, _vp]),
+    "launch_add_rms_norm_bf16_batch": (None, [_vp, _vp, _vp, _vp, _i, C.c_float, _i, _vp]),
+    "launch_silu_mul_bf16_batch": (None, [_vp, _vp, _vp, _i, _i, _vp]),
+    "launch_add_batch": (None, [_vp, _vp, _i, _i, _vp]),
+    "launch_rope_batch": (None, [_vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _i, _vp]),
+    "launch_store_kv_batch": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "launch_rope_store_kv": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _vp]),
+    "launch_rope_store_kv_batch": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _i, _vp]),
+    "launch_attention_all_heads": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _vp]),
+    "launch_flash_attention": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _vp]),
+    "launch_attention_all_heads_batch": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, C.c_float, _i, _i, _vp]),
+    "launch_flash_attention_batch": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, C.c_float, _i, _i, _vp]),
+    "launch_argmax": (None, [_vp, _vp, _i, _vp]),
+    "launch_argmax_batch": (None, [_vp, _vp, _i, _i, _vp]),
+    # engine (C face of model.h / inference.h / sampler.h)
+    "t12_engine_load": (_vp, [C.c_char_p, _i]),
+    "t12_engine_create_synthetic": (_vp, [_i, _i, _i, _i, _i, _i, _i, C.c_float, C.c_float, C.c_uint64, _i, C.c_float]),
+    "t12_engine_save": (_i, [_vp, C.c_char_p]),
+    "t12_engine_free_model": (None, [_vp]),
+    "t12_engine_create_state": (_vp, [_vp, _i, _i]),
+    "t12_engine_free_state": (None, [_vp]),
+    "t12_engine_forward": (_i, [_vp, C.POINTER(C.c_int)]),
+    "t12_engine_logits": (_vp, [_vp]),
+    "t12_engine_stream": (_vp, [_vp]),
+    "t12_engine_max_seq": (_i, [_vp]),
+    "t12_engine_set_positions": (None, [_vp, C.POINTER(C.c_int)]),
+    "t12_engine_get_positions": (None, [_vp, C.POINTER(C.c_int)]),
+    "t12_engine_sample": (_i, [_vp, C.POINTER(C.c_int)]),
+    "t12_engine_generate": (_i, [_vp, C.POINTER(C.c_int), _i, _i, C.POINTER(C.c_int)]),
+    "t12_engine_sync": (_i, [_vp]),
+    "t12_engine_weight": (_i, [_vp, _i, _i, C.POINTER(Segment), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "t12_gemm": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_tune_gemm": (_i, [_i]),
     "t12_decompress": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
@@ -114,7 +150,8 @@ class DeviceTensor12:
         use = patched and self.row_off is not None and self.P > 0   # no escapes: no list
         return Segment(_dp(self.sm), _dp(self.gr), _dp(self.row_off) if use else None,
                        _dp(self.cols) if use else None, _dp(self.correct) if use else None,
-                       _dp(self.wrong) if use else None, _dp(out), self.M, self.base_exp)
+                       _dp(self.wrong) if use else None, _dp(out), self.M, self.base_exp,
+                       int(out.stride(0)) if (out is not None and out.dim() == 2) else 0, 0)
 
 
 def _seg_array(segs):
@@ -145,8 +182,7 @@ def gemm(tensors, X, outs=None, patched=True, stream=None):
     assert K == tensors[0].K and X.stride(1) == 1
     if outs is None:
         outs = [torch.empty((B, t.M), dtype=torch.float32, device=X.device) for t in tensors]
-    stride = outs[0].stride(0)
-    assert all(o.stride(0) == stride for o in outs)
+    stride = outs[0].stride(0)      # every segment carries its own stride; this is the default
     segs = _seg_array([t.segment(o, patched) for t, o in zip(tensors, outs)])
     st = current_stream() if stream is None else stream
     check(lib.t12_gemm(segs, len(tensors), X.data_ptr(), X.stride(0), stride, K, B, st), "t12_gemm")
@@ -200,3 +236,102 @@ def pack_device(w, base_exp=None, stream=None) -> DeviceTensor12:
         check(lib.t12_pack_escapes(w.data_ptr(), M, K, base_exp, row_off.data_ptr(), cols.data_ptr(),
                                    correct.data_ptr(), wrong.data_ptr(), st), "t12_pack_escapes")
     return DeviceTensor12(M, K, base_exp, sm, gr, row_off, cols, correct, wrong)
+
+
+# ------------------------------------------------------------------ engine
+class Engine:
+    """The engine's load / forward / sample / generate API (include/turbo/*.h) through its C face."""
+
+    def __init__(self, model_handle, batch=1):
+        if not model_handle:
+            raise T12Error("model could not be loaded/created")
+        self.model = model_handle
+        self.batch = batch
+        self.state = lib.t12_engine_create_state(self.model, batch, 0)
+
+    @classmethod
+    def load(cls, path, batch=1, device=0):
+        return cls(lib.t12_engine_load(os.fsencode(path), device), batch)
+
+    @classmethod
+    def synthetic(cls, cfg, seed=4000, max_seq=2048, batch=1, p_outlier=3e-4):
+        h = lib.t12_engine_create_synthetic(cfg["n_vocab"], cfg["n_embd"], cfg["n_head"], cfg["n_head_kv"],
+                                            cfg["n_layer"], cfg["n_ff"], cfg.get("n_ctx", max_seq),
+                                            cfg.get("rope_theta", 500000.0), cfg.get("rms_norm_eps", 1e-5), seed,
+                                            max_seq, p_outlier)
+        return cls(h, batch)
+
+    def new_state(self, batch):
+        """A second InferenceState on the same model (they share the model's KV cache)."""
+        e = Engine.__new__(Engine)
+        e.model, e.batch = self.model, batch
+        e.state = lib.t12_engine_create_state(self.model, batch, 0)
+        e._borrowed = True
+        return e
+
+    def save(self, path):
+        check(lib.t12_engine_save(self.model, os.fsencode(path)), "save_model")
+
+    def set_positions(self, pos):
+        arr = (C.c_int * self.batch)(*[int(p) for p in pos])
+        lib.t12_engine_set_positions(self.state, arr)
+
+    def positions(self):
+        arr = (C.c_int * self.batch)()
+        lib.t12_engine_get_positions(self.state, arr)
+        return list(arr)
+
+    def forward(self, tokens):
+        arr = (C.c_int * self.batch)(*[int(t) for t in tokens])
+        lib.t12_engine_forward(self.state, arr)
+
+    def sync(self):
+        check(lib.t12_engine_sync(self.state), "stream sync")
+
+    def logits(self, n_vocab):
+        """fp32 [batch, n_vocab] view of the device logits (synchronises the engine stream first)."""
+        torch = _torch()
+        self.sync()
+        ptr = lib.t12_engine_logits(self.state)
+        n = self.batch * n_vocab
+        out = torch.empty((self.batch, n_vocab), dtype=torch.float32, device="cuda")
+        rc = _hip_memcpy_d2d(out.data_ptr(), ptr, n * 4)
+        if rc:
+            raise T12Error("hipMemcpy failed (%d)" % rc)
+        return out
+
+    def sample(self):
+        arr = (C.c_int * self.batch)()
+        lib.t12_engine_sample(self.state, arr)
+        return list(arr)
+
+    def generate(self, prompt, max_tokens):
+        p = (C.c_int * len(prompt))(*[int(t) for t in prompt])
+        out = (C.c_int * max(max_tokens, 1))()
+        n = lib.t12_engine_generate(self.state, p, len(prompt), max_tokens, out)
+        return list(out[:n])
+
+    def weight(self, layer, which):
+        seg, K, P = Segment(), C.c_int(), C.c_int()
+        check(lib.t12_engine_weight(self.model, layer, which, C.byref(seg), C.byref(K), C.byref(P)), "engine_weight")
+        return seg, K.value, P.value
+
+    def close(self):
+        if self.state:
+            lib.t12_engine_free_state(self.state)
+            self.state = None
+        if self.model and not getattr(self, "_borrowed", False):
+            lib.t12_engine_free_model(self.model)
+        self.model = None
+
+
+_hip = None
+
+
+def _hip_memcpy_d2d(dst, src, nbytes):
+    global _hip
+    if _hip is None:
+        _hip = C.CDLL("libamdhip64.so")
+        _hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        _hip.hipMemcpy.restype = C.c_int
+    return _hip.hipMemcpy(dst, src, nbytes, 3)   # hipMemcpyDeviceToDevice

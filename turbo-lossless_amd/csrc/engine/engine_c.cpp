@@ -1,0 +1,101 @@
+// C face of the engine's C++ API (model.h / inference.h / sampler.h) for callers
+// that cannot pass std::string / std::vector (ctypes, cgo, JNI).
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "t12_abi.h"
+#include "turbo/inference.h"
+#include "turbo/sampler.h"
+
+extern "C" {
+
+void* t12_engine_load(const char* path, int device) { return load_model(path ? path : "", device); }
+
+void* t12_engine_create_synthetic(int n_vocab, int n_embd, int n_head, int n_head_kv, int n_layer, int n_ff, int n_ctx,
+                                  float rope_theta, float rms_eps, uint64_t seed, int max_seq, float p_outlier)
+{
+    ModelConfig c = {n_vocab, n_embd, n_head, n_head_kv, n_layer, n_ff, n_ctx, rope_theta, rms_eps};
+    return create_synthetic_model(c, seed, max_seq, p_outlier);
+}
+
+int t12_engine_save(void* model, const char* dir) { return save_model((Model*)model, dir) ? 0 : -1; }
+void t12_engine_free_model(void* model) { free_model((Model*)model); }
+
+void* t12_engine_create_state(void* model, int batch, int max_seq)
+{
+    return create_inference_state((Model*)model, batch, max_seq);
+}
+void t12_engine_free_state(void* state) { free_inference_state((InferenceState*)state); }
+
+int t12_engine_forward(void* state, const int* tokens_host)
+{
+    forward((InferenceState*)state, tokens_host);
+    return 0;
+}
+void* t12_engine_logits(void* state) { return ((InferenceState*)state)->logits; }
+void* t12_engine_stream(void* state) { return ((InferenceState*)state)->stream; }
+int t12_engine_max_seq(void* model) { return ((Model*)model)->max_seq_len; }
+
+void t12_engine_set_positions(void* state, const int* pos)
+{
+    auto* s = (InferenceState*)state;
+    memcpy(s->positions, pos, sizeof(int) * s->batch_size);
+}
+void t12_engine_get_positions(void* state, int* pos)
+{
+    auto* s = (InferenceState*)state;
+    memcpy(pos, s->positions, sizeof(int) * s->batch_size);
+}
+
+// Greedy sample of the logits of the last forward; tokens_out is a host array [batch].
+int t12_engine_sample(void* state, int* tokens_out)
+{
+    auto* s = (InferenceState*)state;
+    sample_greedy_batch(s->logits, tokens_out, s->model->config.n_vocab, s->batch_size, s->stream);
+    return 0;
+}
+
+// generate(); returns the number of tokens written to out (<= max_tokens).
+int t12_engine_generate(void* state, const int* prompt, int n_prompt, int max_tokens, int* out)
+{
+    std::vector<int> p(prompt, prompt + n_prompt);
+    std::vector<int> r = generate((InferenceState*)state, p, max_tokens);
+    for (size_t i = 0; i < r.size(); i++) out[i] = r[i];
+    return (int)r.size();
+}
+
+int t12_engine_sync(void* state)
+{
+    return hipStreamSynchronize(((InferenceState*)state)->stream) == hipSuccess ? 0 : -1;
+}
+
+// The tensors of the model as segments (out = NULL), for tests that check the
+// loader against the files.  which: 0 wq 1 wk 2 wv 3 wo 4 w_gate 5 w_up 6 w_down; layer -1 = output_proj.
+int t12_engine_weight(void* model, int layer, int which, T12Segment* seg, int* K, int* num_patches)
+{
+    Model* m = (Model*)model;
+    const CompressedWeight* w = nullptr;
+    if (layer < 0) w = &m->output_proj;
+    else if (layer < (int)m->layers.size()) {
+        TransformerLayer& L = m->layers[layer];
+        const CompressedWeight* all[7] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.w_gate, &L.w_up, &L.w_down};
+        if (which >= 0 && which < 7) w = all[which];
+    }
+    if (!w || !w->split_sm) return -1;
+    seg->sm = w->split_sm;
+    seg->gr = w->split_gr;
+    seg->row_off = w->row_offsets;
+    seg->cols = w->patch_cols;
+    seg->correct = w->patch_correct;
+    seg->wrong = w->patch_wrong;
+    seg->out = nullptr;
+    seg->M = w->M;
+    seg->base_exp = w->base_exp;
+    seg->out_stride = seg->reserved = 0;
+    *K = w->K;
+    *num_patches = w->num_patches;
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,248 @@
+// Decode loop: the layer wiring of the reference's forward_b1 / forward_b8 /
+// forward_batch_tiled (engine/inference.cpp:198-366, 459-533, 572-666) on the
+// gfx950 kernels of this library:
+//   * wq|wk|wv and gate|up are ONE launch each (segment tables), with the escape
+//     corrections fused, instead of 3 + 1 and 1 + 1 launches;
+//   * RoPE and the INT8 KV store are one launch;
+//   * B = 1 uses the decode-GEMV, every B > 1 the decode+GEMM (all sequences
+//     run; the reference silently runs sequence 0 only for B not in {1,4,8,8k}).
+// Like the reference's batched modes, the B sequences share ONE KV-cache region
+// (kv_stride = 0, inference.cpp:427-435): the B > 1 modes are meant for B
+// identical streams in lock-step, which is what generate() feeds.
+#include "turbo/inference.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+
+#include "t12_abi.h"
+#include "turbo/sampler.h"
+
+extern "C" {
+void launch_embed_lookup(const int16_t*, const int*, float*, int, int, int, hipStream_t);
+void launch_rms_norm_bf16_batch(const float*, const float*, int16_t*, int, float, int, hipStream_t);
+void launch_add_rms_norm_bf16_batch(float*, const float*, const float*, int16_t*, int, float, int, hipStream_t);
+void launch_silu_mul_bf16_batch(const float*, const float*, int16_t*, int, int, hipStream_t);
+void launch_rope_store_kv_batch(float*, float*, const float*, int8_t*, int8_t*, float*, float*, const int*, int, int,
+                                int, int, int, float, int, hipStream_t);
+void launch_rope_store_kv(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int, int, int, int, int,
+                          float, hipStream_t);
+void launch_attention_all_heads(const float*, const int8_t*, const int8_t*, const float*, const float*, int16_t*, int,
+                                int, int, int, int, float, hipStream_t);
+void launch_attention_all_heads_batch(const float*, const int8_t*, const int8_t*, const float*, const float*, int16_t*,
+                                      const int*, int, int, int, int, float, int, int, hipStream_t);
+}
+
+namespace {
+
+struct LayerSegs {
+    T12Segment qkv[3], o[1], gateup[2], down[1];
+};
+struct Impl {
+    std::vector<LayerSegs> layers;
+    T12Segment head[1];
+};
+
+void check_gpu(hipError_t e, const char* what)
+{
+    if (e != hipSuccess) {
+        fprintf(stderr, "GPU error (%s): %s\n", what, hipGetErrorString(e));
+        exit(1);
+    }
+}
+
+T12Segment seg_of(const CompressedWeight& w, float* out, int out_stride)
+{
+    if (!w.split_sm) {   // same failure mode as the reference (inference.cpp:73,223,306)
+        fprintf(stderr, "ERROR: split12 data missing for weight %dx%d\n", w.M, w.K);
+        exit(1);
+    }
+    T12Segment s;
+    s.sm = w.split_sm;
+    s.gr = w.split_gr;
+    const bool has = w.num_patches > 0 && w.row_offsets;
+    s.row_off = has ? w.row_offsets : nullptr;
+    s.cols = has ? w.patch_cols : nullptr;
+    s.correct = has ? w.patch_correct : nullptr;
+    s.wrong = has ? w.patch_wrong : nullptr;
+    s.out = out;
+    s.M = w.M;
+    s.base_exp = w.base_exp;
+    s.out_stride = out_stride;
+    s.reserved = 0;
+    return s;
+}
+
+void run_linear(const T12Segment* segs, int nseg, const int16_t* act, int K, int B, hipStream_t st)
+{
+    int rc;
+    if (B == 1) rc = t12_gemv(segs, nseg, act, K, st);
+    else rc = t12_gemm(segs, nseg, act, K, segs[0].out_stride, K, B, st);
+    if (rc != T12_OK) {
+        fprintf(stderr, "ERROR: split-12 linear launch failed: %s\n", t12_last_error());
+        exit(1);
+    }
+}
+
+}  // namespace
+
+InferenceState* create_inference_state(Model* model, int batch_size, int max_seq_len)
+{
+    (void)max_seq_len;   // the cache belongs to the model (engine/model.cpp:271-282)
+    auto* s = new InferenceState();
+    s->model = model;
+    s->batch_size = batch_size;
+    s->positions = new int[batch_size]();
+    const ModelConfig& c = model->config;
+    const int n = c.n_embd, n_ff = c.n_ff, n_vocab = c.n_vocab;
+    const int kv_dim = c.n_head_kv * (n / c.n_head);
+    const size_t bs = (size_t)batch_size;
+    auto fbuf = [&](size_t count) {
+        float* p = nullptr;
+        check_gpu(hipMalloc((void**)&p, count * sizeof(float)), "hipMalloc");
+        return p;
+    };
+    s->hidden = fbuf(bs * n);
+    s->hidden2 = fbuf(bs * n);
+    s->attn_out = fbuf(bs * n);
+    s->q_buf = fbuf(bs * n);
+    s->k_buf = fbuf(bs * kv_dim);
+    s->v_buf = fbuf(bs * kv_dim);
+    s->ffn_gate = fbuf(bs * n_ff);
+    s->ffn_up = fbuf(bs * n_ff);
+    s->ffn_down = nullptr;
+    s->logits = fbuf(bs * n_vocab);
+    s->attn_scores_buf = nullptr;
+    check_gpu(hipMalloc((void**)&s->d_positions, bs * sizeof(int)), "hipMalloc");
+    check_gpu(hipMalloc((void**)&s->d_tokens, bs * sizeof(int)), "hipMalloc");
+    const size_t max_act = (size_t)std::max(n, n_ff);
+    check_gpu(hipMalloc((void**)&s->bf16_act, bs * max_act * sizeof(int16_t)), "hipMalloc");
+    check_gpu(hipMalloc((void**)&s->bf16_act2, bs * max_act * sizeof(int16_t)), "hipMalloc");
+    check_gpu(hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking), "stream");
+    check_gpu(hipStreamCreateWithFlags(&s->stream2, hipStreamNonBlocking), "stream");
+    check_gpu(hipEventCreateWithFlags(&s->sync_event, hipEventDisableTiming), "event");
+    s->patch_descs_gpu = nullptr;
+
+    auto* impl = new Impl();
+    impl->layers.resize(c.n_layer);
+    s->impl = impl;
+    init_sampler(batch_size);
+    return s;
+}
+
+void free_inference_state(InferenceState* state)
+{
+    if (!state) return;
+    delete[] state->positions;
+    for (void* p : {(void*)state->hidden, (void*)state->hidden2, (void*)state->attn_out, (void*)state->q_buf,
+                    (void*)state->k_buf, (void*)state->v_buf, (void*)state->ffn_gate, (void*)state->ffn_up,
+                    (void*)state->ffn_down, (void*)state->logits, (void*)state->attn_scores_buf,
+                    (void*)state->d_positions, (void*)state->d_tokens, (void*)state->bf16_act,
+                    (void*)state->bf16_act2, state->patch_descs_gpu})
+        if (p) (void)hipFree(p);
+    if (state->stream) (void)hipStreamDestroy(state->stream);
+    if (state->stream2) (void)hipStreamDestroy(state->stream2);
+    if (state->sync_event) (void)hipEventDestroy(state->sync_event);
+    delete (Impl*)state->impl;
+    delete state;
+}
+
+void forward(InferenceState* state, const int* token_ids)
+{
+    Model* m = state->model;
+    const ModelConfig& c = m->config;
+    hipStream_t st = state->stream;
+    const int B = state->batch_size;
+    const int n = c.n_embd, n_ff = c.n_ff, head_dim = n / c.n_head;
+    const int kv_dim = c.n_head_kv * head_dim;
+    const float scale = 1.0f / sqrtf((float)head_dim);
+    Impl* impl = (Impl*)state->impl;
+
+    int max_pos = 0;
+    for (int b = 0; b < B; b++) max_pos = std::max(max_pos, state->positions[b]);
+    if (max_pos >= m->max_seq_len) {
+        fprintf(stderr, "ERROR: position %d exceeds the KV cache (%d)\n", max_pos, m->max_seq_len);
+        exit(1);
+    }
+    (void)hipMemcpyAsync(state->d_tokens, token_ids, B * sizeof(int), hipMemcpyHostToDevice, st);
+    if (B > 1) (void)hipMemcpyAsync(state->d_positions, state->positions, B * sizeof(int), hipMemcpyHostToDevice, st);
+    launch_embed_lookup(m->token_embd, state->d_tokens, state->hidden, n, B, c.n_vocab, st);
+
+    float* cur = state->hidden;    // residual stream
+    float* res = state->hidden2;
+    int16_t* bf16_a = state->bf16_act;
+    int16_t* bf16_b = state->bf16_act2;
+
+    for (int layer = 0; layer < c.n_layer; layer++) {
+        TransformerLayer& L = m->layers[layer];
+        LayerSegs& S = impl->layers[layer];
+        if (layer == 0) launch_rms_norm_bf16_batch(cur, L.attn_norm, bf16_a, n, c.rms_norm_eps, B, st);
+
+        S.qkv[0] = seg_of(L.wq, state->q_buf, n);
+        S.qkv[1] = seg_of(L.wk, state->k_buf, kv_dim);
+        S.qkv[2] = seg_of(L.wv, state->v_buf, kv_dim);
+        run_linear(S.qkv, 3, bf16_a, n, B, st);
+
+        const size_t kv_off = (size_t)layer * m->max_seq_len * kv_dim;
+        const size_t sc_off = (size_t)layer * m->max_seq_len * c.n_head_kv;
+        if (B == 1) {
+            launch_rope_store_kv(state->q_buf, state->k_buf, state->v_buf, m->kv_cache_k + kv_off,
+                                 m->kv_cache_v + kv_off, m->kv_scale_k + sc_off, m->kv_scale_v + sc_off, head_dim,
+                                 c.n_head, c.n_head_kv, state->positions[0], m->max_seq_len, c.rope_theta, st);
+            launch_attention_all_heads(state->q_buf, m->kv_cache_k + kv_off, m->kv_cache_v + kv_off,
+                                       m->kv_scale_k + sc_off, m->kv_scale_v + sc_off, bf16_a, c.n_head, c.n_head_kv,
+                                       head_dim, state->positions[0] + 1, m->max_seq_len, scale, st);
+        } else {
+            launch_rope_store_kv_batch(state->q_buf, state->k_buf, state->v_buf, m->kv_cache_k + kv_off,
+                                       m->kv_cache_v + kv_off, m->kv_scale_k + sc_off, m->kv_scale_v + sc_off,
+                                       state->d_positions, head_dim, c.n_head, c.n_head_kv, n, kv_dim, c.rope_theta, B,
+                                       st);
+            launch_attention_all_heads_batch(state->q_buf, m->kv_cache_k + kv_off, m->kv_cache_v + kv_off,
+                                             m->kv_scale_k + sc_off, m->kv_scale_v + sc_off, bf16_a, state->d_positions,
+                                             c.n_head, c.n_head_kv, head_dim, max_pos + 1, scale, B, 0, st);
+        }
+
+        S.o[0] = seg_of(L.wo, res, n);
+        run_linear(S.o, 1, bf16_a, n, B, st);
+        launch_add_rms_norm_bf16_batch(res, cur, L.ffn_norm, bf16_a, n, c.rms_norm_eps, B, st);
+
+        S.gateup[0] = seg_of(L.w_gate, state->ffn_gate, n_ff);
+        S.gateup[1] = seg_of(L.w_up, state->ffn_up, n_ff);
+        run_linear(S.gateup, 2, bf16_a, n, B, st);
+        launch_silu_mul_bf16_batch(state->ffn_gate, state->ffn_up, bf16_b, n_ff, B, st);
+
+        S.down[0] = seg_of(L.w_down, cur, n);
+        run_linear(S.down, 1, bf16_b, n_ff, B, st);
+        const float* next_norm = layer + 1 < c.n_layer ? m->layers[layer + 1].attn_norm : m->output_norm;
+        launch_add_rms_norm_bf16_batch(cur, res, next_norm, bf16_a, n, c.rms_norm_eps, B, st);
+    }
+    if (c.n_layer == 0) launch_rms_norm_bf16_batch(cur, m->output_norm, bf16_a, n, c.rms_norm_eps, B, st);
+
+    impl->head[0] = seg_of(m->output_proj, state->logits, c.n_vocab);
+    run_linear(impl->head, 1, bf16_a, n, B, st);
+    for (int b = 0; b < B; b++) state->positions[b]++;
+}
+
+std::vector<int> generate(InferenceState* state, const std::vector<int>& prompt_tokens, int max_tokens)
+{
+    std::vector<int> output;
+    const int n_vocab = state->model->config.n_vocab;
+    const int bs = state->batch_size;
+    std::vector<int> tokens(bs);
+    for (int i = 0; i < (int)prompt_tokens.size(); i++) {
+        for (int s = 0; s < bs; s++) {
+            state->positions[s] = i;
+            tokens[s] = prompt_tokens[i];
+        }
+        forward(state, tokens.data());
+    }
+    for (int t = 0; t < max_tokens; t++) {
+        if (bs == 1) tokens[0] = sample_greedy(state->logits, n_vocab, state->stream);
+        else sample_greedy_batch(state->logits, tokens.data(), n_vocab, bs, state->stream);
+        if (tokens[0] == 2) break;
+        output.push_back(tokens[0]);
+        forward(state, tokens.data());
+    }
+    return output;
+}

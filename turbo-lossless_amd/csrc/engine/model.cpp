@@ -1,0 +1,430 @@
+// Model store: reads the directory layout the reference's converter writes
+// (engine/convert_model.py:57-62,127-152) into HBM, as engine/model.cpp:32-328
+// does, with the file sizes checked against .dims; plus a GPU-side synthetic
+// model generator and a writer of the same layout.
+#include "turbo/model.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+
+#include "t12_abi.h"
+
+extern "C" int t12_synth_normal_bf16(void*, size_t, uint64_t, float, float, float, void*);
+extern "C" int t12_fill_f32(void*, size_t, float, void*);
+
+namespace {
+
+bool read_file(const std::string& path, std::vector<uint8_t>& data, bool quiet = false)
+{
+    std::ifstream f(path, std::ios::binary | std::ios::ate);
+    if (!f) {
+        if (!quiet) fprintf(stderr, "Cannot open: %s\n", path.c_str());
+        data.clear();
+        return false;
+    }
+    const std::streamoff size = f.tellg();
+    f.seekg(0);
+    data.resize((size_t)size);
+    if (size > 0) f.read((char*)data.data(), size);
+    return (bool)f;
+}
+
+bool gpu_ok(hipError_t e, const char* what)
+{
+    if (e == hipSuccess) return true;
+    fprintf(stderr, "GPU error (%s): %s\n", what, hipGetErrorString(e));
+    return false;
+}
+
+// Device copy of a host array; an allocation failure ends the process like the
+// reference's GPU_CHECK (gpu_compat.h:94-101).
+template <typename T>
+T* upload(const void* host, size_t count)
+{
+    if (count == 0) return nullptr;
+    T* d = nullptr;
+    if (!gpu_ok(hipMalloc((void**)&d, count * sizeof(T)), "hipMalloc")) exit(1);
+    if (!gpu_ok(hipMemcpy(d, host, count * sizeof(T), hipMemcpyHostToDevice), "hipMemcpy")) exit(1);
+    return d;
+}
+
+template <typename T>
+T* device_alloc(size_t count)
+{
+    T* d = nullptr;
+    if (!gpu_ok(hipMalloc((void**)&d, std::max<size_t>(count, 1) * sizeof(T)), "hipMalloc")) exit(1);
+    return d;
+}
+
+void clear_weight(CompressedWeight& w)
+{
+    memset(&w, 0, sizeof w);
+}
+
+// Derived escape tables, the layout of engine/model.cpp:86-160 with WG = 256:
+// row_base[r] = escapes before row r; esc_vals ordered (row, col % 256, ascending col);
+// list of rows that hold an escape.  escape_counts is never built (the kernels
+// here read the CSR list).
+void build_escape_tables(CompressedWeight& w, const int32_t* row_off, const int32_t* cols, const int16_t* correct)
+{
+    const int WG = 256;
+    std::vector<int32_t> row_base(w.M), nonempty;
+    std::vector<int16_t> vals(w.num_patches);
+    std::vector<int32_t> bucket(WG + 1);
+    for (int r = 0; r < w.M; r++) {
+        const int beg = row_off[r], end = row_off[r + 1];
+        row_base[r] = beg;
+        if (end == beg) continue;
+        nonempty.push_back(r);
+        std::fill(bucket.begin(), bucket.end(), 0);
+        for (int p = beg; p < end; p++) bucket[cols[p] % WG + 1]++;
+        for (int t = 0; t < WG; t++) bucket[t + 1] += bucket[t];
+        for (int p = beg; p < end; p++) vals[beg + bucket[cols[p] % WG]++] = correct[p];   // cols ascend in a row
+    }
+    w.escape_row_base = upload<int32_t>(row_base.data(), row_base.size());
+    w.escape_vals = upload<int16_t>(vals.data(), vals.size());
+    w.escape_counts = nullptr;
+    w.num_nonempty_rows = (int)nonempty.size();
+    w.patch_nonempty_rows = upload<int32_t>(nonempty.data(), nonempty.size());
+}
+
+bool load_compressed(const std::string& dir, const std::string& prefix, CompressedWeight& w)
+{
+    clear_weight(w);
+    const std::string base = dir + "/" + prefix;
+    std::ifstream df(base + ".dims");
+    if (!df) {
+        fprintf(stderr, "Missing: %s.dims\n", base.c_str());
+        return false;
+    }
+    int M = 0, K = 0, P = 0, be = 0;
+    if (!(df >> M >> K >> P) || M <= 0 || K <= 0 || P < 0) {
+        fprintf(stderr, "ERROR: malformed %s.dims\n", base.c_str());
+        return false;
+    }
+    if (!(df >> be)) be = 0;                       // 4th field optional (engine/model.cpp:38-42)
+    const size_t n = (size_t)M * K;
+
+    std::vector<uint8_t> sm, gr, ro, pc, pv, pw;
+    if (!read_file(base + ".sm.bin", sm, true) || !read_file(base + ".gr.bin", gr, true) || sm.empty() || gr.empty()) {
+        fprintf(stderr, "ERROR: split12 files missing for %s (need .sm.bin + .gr.bin)\n", prefix.c_str());
+        return false;
+    }
+    if (sm.size() != n || gr.size() != (n + 1) / 2) {
+        fprintf(stderr, "ERROR: %s: plane sizes %zu/%zu do not match dims %d x %d\n", prefix.c_str(), sm.size(),
+                gr.size(), M, K);
+        return false;
+    }
+    read_file(base + ".row_off.bin", ro, true);
+    read_file(base + ".patch_cols.bin", pc, true);
+    read_file(base + ".patch_correct.bin", pv, true);
+    read_file(base + ".patch_wrong.bin", pw, true);
+    if (P > 0) {
+        const bool sizes_ok = ro.size() == (size_t)(M + 1) * 4 && pc.size() == (size_t)P * 4 &&
+                              pv.size() == (size_t)P * 2 && pw.size() == (size_t)P * 2;
+        if (!sizes_ok || ((const int32_t*)ro.data())[M] != P) {
+            fprintf(stderr, "ERROR: %s: escape list files do not match num_patches %d\n", prefix.c_str(), P);
+            return false;
+        }
+        const int32_t* h_ro = (const int32_t*)ro.data();
+        const int32_t* h_pc = (const int32_t*)pc.data();
+        for (int r = 0; r < M; r++)
+            if (h_ro[r + 1] < h_ro[r]) { fprintf(stderr, "ERROR: %s: row_off not monotone\n", prefix.c_str()); return false; }
+        for (int p = 0; p < P; p++)
+            if (h_pc[p] < 0 || h_pc[p] >= K) { fprintf(stderr, "ERROR: %s: escape column out of range\n", prefix.c_str()); return false; }
+    }
+    w.M = M;
+    w.K = K;
+    w.num_patches = P;
+    w.base_exp = be;
+    w.split_sm = upload<uint8_t>(sm.data(), sm.size());
+    w.split_gr = upload<uint8_t>(gr.data(), gr.size());
+    if (P > 0) {
+        w.row_offsets = upload<int32_t>(ro.data(), M + 1);
+        w.patch_cols = upload<int32_t>(pc.data(), P);
+        w.patch_correct = upload<int16_t>(pv.data(), P);
+        w.patch_wrong = upload<int16_t>(pw.data(), P);
+        build_escape_tables(w, (const int32_t*)ro.data(), (const int32_t*)pc.data(), (const int16_t*)pv.data());
+    }
+    return true;
+}
+
+void free_weight(CompressedWeight& w)
+{
+    void* ptrs[] = {w.row_offsets, w.patch_cols, w.patch_correct, w.patch_wrong, w.escape_row_base, w.escape_counts,
+                    w.escape_vals, w.split_sm,   w.split_gr,      w.patch_nonempty_rows};
+    for (void* p : ptrs)
+        if (p) (void)hipFree(p);
+    clear_weight(w);
+}
+
+void alloc_kv_cache(Model* m, int max_seq)
+{
+    const ModelConfig& c = m->config;
+    const int head_dim = c.n_embd / c.n_head;
+    m->max_seq_len = std::max(max_seq, 128);
+    const size_t kv = (size_t)c.n_layer * m->max_seq_len * c.n_head_kv * head_dim;
+    const size_t sc = (size_t)c.n_layer * m->max_seq_len * c.n_head_kv;
+    m->kv_cache_k = device_alloc<int8_t>(kv);
+    m->kv_cache_v = device_alloc<int8_t>(kv);
+    m->kv_scale_k = device_alloc<float>(sc);
+    m->kv_scale_v = device_alloc<float>(sc);
+    (void)hipMemset(m->kv_cache_k, 0, kv);
+    (void)hipMemset(m->kv_cache_v, 0, kv);
+    (void)hipMemset(m->kv_scale_k, 0, sc * sizeof(float));
+    (void)hipMemset(m->kv_scale_v, 0, sc * sizeof(float));
+}
+
+int default_context(const ModelConfig& c)
+{
+    const char* env = getenv("TURBO_CTX");
+    if (env) return atoi(env);
+    const int head_dim = c.n_embd / c.n_head;
+    const size_t per_tok = (size_t)c.n_layer * c.n_head_kv * head_dim * 2 + (size_t)c.n_layer * c.n_head_kv * 2 * 4;
+    size_t free_b = 0, total_b = 0;
+    (void)hipMemGetInfo(&free_b, &total_b);
+    const size_t budget = free_b > (512u << 20) ? free_b - (512u << 20) : free_b / 2;
+    return (int)std::min<size_t>(8192, budget / std::max<size_t>(per_tok, 1));
+}
+
+}  // namespace
+
+Model* load_model(const std::string& model_path, int device_id)
+{
+    if (!gpu_ok(hipSetDevice(device_id), "hipSetDevice")) return nullptr;
+    std::vector<uint8_t> buf;
+    if (!read_file(model_path + "/config.bin", buf, true) || buf.size() < 36) {
+        fprintf(stderr, "No config.bin found in %s\n", model_path.c_str());
+        return nullptr;
+    }
+    Model* m = new Model();
+    struct { int32_t v[7]; float theta, eps; } raw;
+    static_assert(sizeof raw == 36, "config.bin is 36 bytes");
+    memcpy(&raw, buf.data(), sizeof raw);
+    ModelConfig& c = m->config;
+    c.n_vocab = raw.v[0]; c.n_embd = raw.v[1]; c.n_head = raw.v[2]; c.n_head_kv = raw.v[3];
+    c.n_layer = raw.v[4]; c.n_ff = raw.v[5]; c.n_ctx = raw.v[6];
+    c.rope_theta = raw.theta; c.rms_norm_eps = raw.eps;
+    if (c.n_vocab <= 0 || c.n_embd <= 0 || c.n_head <= 0 || c.n_head_kv <= 0 || c.n_layer < 0 || c.n_ff <= 0 ||
+        c.n_embd % c.n_head || c.n_head % c.n_head_kv) {
+        fprintf(stderr, "config.bin in %s holds an impossible shape\n", model_path.c_str());
+        delete m;
+        return nullptr;
+    }
+    printf("  Config: vocab=%d embd=%d heads=%d/%d layers=%d ff=%d\n", c.n_vocab, c.n_embd, c.n_head, c.n_head_kv,
+           c.n_layer, c.n_ff);
+
+    if (!read_file(model_path + "/tok_embd.bin", buf, true) || buf.size() != (size_t)c.n_vocab * c.n_embd * 2) {
+        fprintf(stderr, "Missing tok_embd.bin (or wrong size)\n");
+        delete m;
+        return nullptr;
+    }
+    m->token_embd = upload<int16_t>(buf.data(), buf.size() / 2);
+
+    auto load_norm = [&](const std::string& name) -> float* {
+        std::vector<uint8_t> nb;
+        if (!read_file(model_path + "/" + name, nb, true) || nb.size() != (size_t)c.n_embd * 4) {
+            fprintf(stderr, "Warning: %s missing or wrong size\n", name.c_str());
+            return nullptr;
+        }
+        return upload<float>(nb.data(), c.n_embd);
+    };
+    m->output_norm = load_norm("output_norm.bin");
+    if (!load_compressed(model_path, "output_proj", m->output_proj)) fprintf(stderr, "Warning: no output_proj\n");
+
+    m->layers.resize(c.n_layer);
+    for (int i = 0; i < c.n_layer; i++) {
+        TransformerLayer& L = m->layers[i];
+        const std::string p = "layer." + std::to_string(i) + ".";
+        L.attn_norm = load_norm(p + "attn_norm.bin");
+        L.ffn_norm = load_norm(p + "ffn_norm.bin");
+        load_compressed(model_path, p + "wq", L.wq);
+        load_compressed(model_path, p + "wk", L.wk);
+        load_compressed(model_path, p + "wv", L.wv);
+        load_compressed(model_path, p + "wo", L.wo);
+        load_compressed(model_path, p + "w_gate", L.w_gate);
+        load_compressed(model_path, p + "w_up", L.w_up);
+        load_compressed(model_path, p + "w_down", L.w_down);
+        if ((i + 1) % 8 == 0 || i == c.n_layer - 1) printf("  Loaded layer %d/%d\n", i + 1, c.n_layer);
+    }
+    alloc_kv_cache(m, default_context(c));
+    printf("  Context length: %d\n  Model loaded.\n", m->max_seq_len);
+    return m;
+}
+
+void free_model(Model* model)
+{
+    if (!model) return;
+    if (model->token_embd) (void)hipFree(model->token_embd);
+    if (model->output_norm) (void)hipFree(model->output_norm);
+    free_weight(model->output_proj);
+    for (auto& L : model->layers) {
+        if (L.attn_norm) (void)hipFree(L.attn_norm);
+        if (L.ffn_norm) (void)hipFree(L.ffn_norm);
+        for (CompressedWeight* w : {&L.wq, &L.wk, &L.wv, &L.wo, &L.w_gate, &L.w_up, &L.w_down}) free_weight(*w);
+    }
+    for (void* p : {(void*)model->kv_cache_k, (void*)model->kv_cache_v, (void*)model->kv_scale_k, (void*)model->kv_scale_v})
+        if (p) (void)hipFree(p);
+    delete model;
+}
+
+// ------------------------------------------------------------ synthetic model
+namespace {
+
+// Packs a bf16 matrix resident in HBM with the GPU packer; fills every field of w.
+bool pack_on_gpu(const void* w_bf16, int M, int K, CompressedWeight& w)
+{
+    clear_weight(w);
+    const size_t n = (size_t)M * K;
+    unsigned long long* d_hist = device_alloc<unsigned long long>(256);
+    uint64_t hist[256];
+    if (t12_pack_histogram(w_bf16, n, d_hist, nullptr) != T12_OK ||
+        !gpu_ok(hipMemcpy(hist, d_hist, sizeof hist, hipMemcpyDeviceToHost), "hist copy")) {
+        (void)hipFree(d_hist);
+        return false;
+    }
+    (void)hipFree(d_hist);
+    const int be = t12_pack_base_exp(hist);
+    w.M = M;
+    w.K = K;
+    w.base_exp = be;
+    w.split_sm = device_alloc<uint8_t>(n);
+    w.split_gr = device_alloc<uint8_t>((n + 1) / 2);
+    int32_t* cnt = device_alloc<int32_t>(M);
+    int32_t* ro = device_alloc<int32_t>(M + 1);
+    bool ok = t12_pack_planes(w_bf16, M, K, be, w.split_sm, w.split_gr, cnt, nullptr) == T12_OK &&
+              t12_pack_row_offsets(cnt, M, ro, nullptr) == T12_OK;
+    int P = 0;
+    ok = ok && gpu_ok(hipMemcpy(&P, ro + M, sizeof(int), hipMemcpyDeviceToHost), "P copy");
+    (void)hipFree(cnt);
+    if (!ok) { (void)hipFree(ro); return false; }
+    w.num_patches = P;
+    if (P == 0) {
+        (void)hipFree(ro);
+        return true;
+    }
+    w.row_offsets = ro;
+    w.patch_cols = device_alloc<int32_t>(P);
+    w.patch_correct = device_alloc<int16_t>(P);
+    w.patch_wrong = device_alloc<int16_t>(P);
+    if (t12_pack_escapes(w_bf16, M, K, be, ro, w.patch_cols, w.patch_correct, w.patch_wrong, nullptr) != T12_OK)
+        return false;
+    std::vector<int32_t> h_ro(M + 1), h_pc(P);
+    std::vector<int16_t> h_pv(P);
+    ok = gpu_ok(hipMemcpy(h_ro.data(), ro, (M + 1) * 4, hipMemcpyDeviceToHost), "row_off copy") &&
+         gpu_ok(hipMemcpy(h_pc.data(), w.patch_cols, (size_t)P * 4, hipMemcpyDeviceToHost), "cols copy") &&
+         gpu_ok(hipMemcpy(h_pv.data(), w.patch_correct, (size_t)P * 2, hipMemcpyDeviceToHost), "correct copy");
+    if (ok) build_escape_tables(w, h_ro.data(), h_pc.data(), h_pv.data());
+    return ok;
+}
+
+template <typename T>
+bool dump(const std::string& path, const T* dev, size_t count)
+{
+    std::vector<T> h(count);
+    if (count && !gpu_ok(hipMemcpy(h.data(), dev, count * sizeof(T), hipMemcpyDeviceToHost), "download")) return false;
+    std::ofstream f(path, std::ios::binary);
+    if (!f) return false;
+    if (count) f.write((const char*)h.data(), (std::streamsize)(count * sizeof(T)));
+    return (bool)f;
+}
+
+bool save_weight(const std::string& dir, const std::string& prefix, const CompressedWeight& w)
+{
+    const std::string b = dir + "/" + prefix;
+    const size_t n = (size_t)w.M * w.K;
+    const size_t P = (size_t)w.num_patches;
+    bool ok = dump<uint8_t>(b + ".sm.bin", w.split_sm, n) && dump<uint8_t>(b + ".gr.bin", w.split_gr, (n + 1) / 2);
+    if (P > 0) {
+        ok = ok && dump<int32_t>(b + ".row_off.bin", w.row_offsets, w.M + 1);
+    } else {                                         // the packer always writes M+1 zeros
+        std::vector<int32_t> z(w.M + 1, 0);
+        std::ofstream f(b + ".row_off.bin", std::ios::binary);
+        f.write((const char*)z.data(), (std::streamsize)(z.size() * 4));
+        ok = ok && (bool)f;
+    }
+    ok = ok && dump<int32_t>(b + ".patch_cols.bin", w.patch_cols, P) &&
+         dump<int16_t>(b + ".patch_correct.bin", w.patch_correct, P) &&
+         dump<int16_t>(b + ".patch_wrong.bin", w.patch_wrong, P);
+    std::ofstream d(b + ".dims");
+    d << w.M << " " << w.K << " " << w.num_patches << " " << w.base_exp;   // no newline (convert_model.py:133-134)
+    return ok && (bool)d;
+}
+
+}  // namespace
+
+Model* create_synthetic_model(const ModelConfig& cfg, uint64_t seed, int max_seq_len, float p_outlier)
+{
+    if (cfg.n_vocab <= 0 || cfg.n_embd <= 0 || cfg.n_head <= 0 || cfg.n_head_kv <= 0 || cfg.n_ff <= 0 ||
+        cfg.n_embd % cfg.n_head || cfg.n_head % cfg.n_head_kv)
+        return nullptr;
+    Model* m = new Model();
+    m->config = cfg;
+    const int n = cfg.n_embd, ff = cfg.n_ff;
+    const int kv = cfg.n_head_kv * (n / cfg.n_head);
+    const size_t biggest = std::max({(size_t)cfg.n_vocab * n, (size_t)ff * n});
+    uint16_t* stage = device_alloc<uint16_t>(biggest);
+    uint64_t s = seed;
+    bool ok = true;
+    auto make = [&](int M, int K, CompressedWeight& w) {
+        ok = ok && t12_synth_normal_bf16(stage, (size_t)M * K, ++s, 0.02f, p_outlier, 8.0f, nullptr) == T12_OK &&
+             pack_on_gpu(stage, M, K, w);
+    };
+    auto ones = [&]() {
+        float* d = device_alloc<float>(n);
+        ok = ok && t12_fill_f32(d, n, 1.0f, nullptr) == T12_OK;
+        return d;
+    };
+    m->token_embd = device_alloc<int16_t>((size_t)cfg.n_vocab * n);
+    ok = ok && t12_synth_normal_bf16(m->token_embd, (size_t)cfg.n_vocab * n, ++s, 0.02f, 0.0f, 0.0f, nullptr) == T12_OK;
+    m->output_norm = ones();
+    m->layers.resize(cfg.n_layer);
+    for (auto& L : m->layers) {
+        L.attn_norm = ones();
+        L.ffn_norm = ones();
+        make(n, n, L.wq);
+        make(kv, n, L.wk);
+        make(kv, n, L.wv);
+        make(n, n, L.wo);
+        make(ff, n, L.w_gate);
+        make(ff, n, L.w_up);
+        make(n, ff, L.w_down);
+    }
+    make(cfg.n_vocab, n, m->output_proj);
+    ok = ok && gpu_ok(hipDeviceSynchronize(), "synthetic model");
+    (void)hipFree(stage);
+    if (!ok) {
+        free_model(m);
+        return nullptr;
+    }
+    alloc_kv_cache(m, max_seq_len > 0 ? max_seq_len : default_context(cfg));
+    return m;
+}
+
+bool save_model(const Model* m, const std::string& dir)
+{
+    const ModelConfig& c = m->config;
+    struct { int32_t v[7]; float theta, eps; } raw = {{c.n_vocab, c.n_embd, c.n_head, c.n_head_kv, c.n_layer, c.n_ff,
+                                                       c.n_ctx}, c.rope_theta, c.rms_norm_eps};
+    {
+        std::ofstream f(dir + "/config.bin", std::ios::binary);
+        if (!f) return false;
+        f.write((const char*)&raw, sizeof raw);
+    }
+    bool ok = dump<int16_t>(dir + "/tok_embd.bin", m->token_embd, (size_t)c.n_vocab * c.n_embd) &&
+              dump<float>(dir + "/output_norm.bin", m->output_norm, c.n_embd) &&
+              save_weight(dir, "output_proj", m->output_proj);
+    for (int i = 0; ok && i < c.n_layer; i++) {
+        const TransformerLayer& L = m->layers[i];
+        const std::string p = "layer." + std::to_string(i) + ".";
+        ok = dump<float>(dir + "/" + p + "attn_norm.bin", L.attn_norm, c.n_embd) &&
+             dump<float>(dir + "/" + p + "ffn_norm.bin", L.ffn_norm, c.n_embd) && save_weight(dir, p + "wq", L.wq) &&
+             save_weight(dir, p + "wk", L.wk) && save_weight(dir, p + "wv", L.wv) && save_weight(dir, p + "wo", L.wo) &&
+             save_weight(dir, p + "w_gate", L.w_gate) && save_weight(dir, p + "w_up", L.w_up) &&
+             save_weight(dir, p + "w_down", L.w_down);
+    }
+    return ok;
+}

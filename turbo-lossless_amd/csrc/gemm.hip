@@ -45,7 +45,7 @@ struct GemmParams {
     int seg_row0[T12_MAX_SEGMENTS];        // first row of each segment in the workspace
     int nseg;
     int K, B;
-    int act_stride, out_stride;
+    int act_stride;
     int ksplit;                            // workgroups along K
     int kslice;                            // columns per K split (multiple of KC)
     int m_total;                           // sum of M over segments (workspace row length)
@@ -216,7 +216,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
         col_off = p.seg_row0[s];
     } else {
         dst = sg.out;
-        ld = p.out_stride;
+        ld = sg.out_stride;
         col_off = 0;
     }
 #pragma unroll
@@ -259,7 +259,7 @@ __global__ __launch_bounds__(64) void gemm_epilogue_kernel(const GemmParams p)
     if (sg.row_off) {
         const int beg = sg.row_off[m], end = sg.row_off[m + 1];
         if (end > beg) {
-            if (!dirty) v = sg.out[(size_t)b * p.out_stride + m];
+            if (!dirty) v = sg.out[(size_t)b * sg.out_stride + m];
             const uint16_t* x = p.act + (size_t)b * p.act_stride;
             for (int q = beg; q < end; q++)
                 v += (t12_bf16_to_f32((uint16_t)sg.correct[q]) - t12_bf16_to_f32((uint16_t)sg.wrong[q])) *
@@ -267,7 +267,7 @@ __global__ __launch_bounds__(64) void gemm_epilogue_kernel(const GemmParams p)
             dirty = true;
         }
     }
-    if (dirty) sg.out[(size_t)b * p.out_stride + m] = v;
+    if (dirty) sg.out[(size_t)b * sg.out_stride + m] = v;
 }
 
 // ---------------------------------------------------------------------------
@@ -309,7 +309,7 @@ __global__ __launch_bounds__(256) void gemm_general_kernel(const GemmParams p)
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const float v = t12_wave_sum(acc[j]);
-        if (lane == 0 && j < nb) sg.out[(size_t)(b0 + j) * p.out_stride + row] = v;
+        if (lane == 0 && j < nb) sg.out[(size_t)(b0 + j) * sg.out_stride + row] = v;
     }
 }
 
@@ -378,7 +378,6 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
     p.K = K;
     p.B = B;
     p.act_stride = act_stride;
-    p.out_stride = out_stride;
     p.act = (const uint16_t*)act_bf16;
     p.ws = nullptr;
     bool fast = (K % KC == 0) && (act_stride % 8 == 0) && ((uintptr_t)act_bf16 % 16 == 0);
@@ -386,13 +385,15 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
     for (int i = 0; i < nseg; i++) {
         const T12Segment& g = segs[i];
         T12_REQUIRE(g.M >= 1 && g.sm && g.gr && g.out, "t12_gemm: segment %d has M < 1 or a null pointer", i);
-        T12_REQUIRE(out_stride >= g.M, "t12_gemm: out_stride %d < M %d of segment %d", out_stride, g.M, i);
         T12_REQUIRE(!g.row_off || (g.cols && g.correct && g.wrong), "t12_gemm: segment %d: row_off without lists", i);
         T12_REQUIRE(g.base_exp >= -1 && g.base_exp <= 254, "t12_gemm: segment %d: base_exp %d out of range", i,
                     g.base_exp);
         if (g.base_exp < 0 || g.base_exp > 240) fast = false;
         if (g.row_off) any_patch = 1;
         p.seg[i] = g;
+        if (p.seg[i].out_stride == 0) p.seg[i].out_stride = out_stride;
+        T12_REQUIRE(p.seg[i].out_stride >= g.M, "t12_gemm: out_stride %d < M %d of segment %d", p.seg[i].out_stride,
+                    g.M, i);
         p.seg_row0[i] = m_total;
         m_total += g.M;
     }

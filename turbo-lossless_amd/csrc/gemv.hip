@@ -359,7 +359,7 @@ int launch_split12_v2_async(const void* sign_mantissa, const void* groups, int b
                             const void* activations, void* output, int M, int K, void* stream)
 {
     T12Segment g = {(const uint8_t*)sign_mantissa, (const uint8_t*)groups, nullptr, nullptr, nullptr, nullptr,
-                    (float*)output, M, base_exp};
+                    (float*)output, M, base_exp, 0, 0};
     return t12_gemv(&g, 1, activations, K, stream);
 }
 
@@ -369,8 +369,8 @@ int launch_split12_v2_dual_async(const void* sm_a, const void* gr_a, int base_ex
                                  int M, int K, void* stream)
 {
     T12Segment g[2] = {
-        {(const uint8_t*)sm_a, (const uint8_t*)gr_a, nullptr, nullptr, nullptr, nullptr, (float*)output_a, M, base_exp_a},
-        {(const uint8_t*)sm_b, (const uint8_t*)gr_b, nullptr, nullptr, nullptr, nullptr, (float*)output_b, M, base_exp_b}};
+        {(const uint8_t*)sm_a, (const uint8_t*)gr_a, nullptr, nullptr, nullptr, nullptr, (float*)output_a, M, base_exp_a, 0, 0},
+        {(const uint8_t*)sm_b, (const uint8_t*)gr_b, nullptr, nullptr, nullptr, nullptr, (float*)output_b, M, base_exp_b, 0, 0}};
     return t12_gemv(g, 2, activations, K, stream);
 }
 
@@ -393,6 +393,7 @@ static int launch_patch_descs(const PatchBatchDesc* d, int n, hipStream_t st)
             g.out = d[i].output;
             g.M = d[i].M;
             g.base_exp = 0;
+            g.out_stride = g.reserved = 0;
             p.blk_start[cnt] = total;
             total += (d[i].M + 3) / 4;
             cnt++;

@@ -1,0 +1,606 @@
+// Engine glue kernels for gfx950: embedding lookup, RMSNorm (+ residual add) ->
+// bf16, SiLU*mul -> bf16, RoPE, INT8 KV store, decode attention over the INT8
+// cache, argmax.  Same C signatures and arithmetic as the reference's launch
+// layer (engine/kernels.hip; cited per function), different kernels:
+//   * RoPE and the INT8 KV store of the B = 1 path are one launch (the reference
+//     uses two, kernels.hip:308-333);
+//   * one decode-attention kernel serves both of the reference's variants
+//     (attention_all_heads, kernels.hip:499-586, and flash_attention, :883-993):
+//     online softmax over 256-position tiles, all query heads of a KV group in
+//     one workgroup so the INT8 cache is read once per group, not once per head;
+//   * argmax is two-phase (many workgroups per row, then one) so that a single
+//     row of 128256 logits is not read by one CU.
+// All math is fp32; bf16 is produced with round-to-nearest-even exactly as
+// float_to_bf16 (kernels.hip:21-27).
+
+#include <cmath>
+#include <mutex>
+#include <vector>
+
+#include "t12_device.h"
+#include "t12_host.h"
+
+namespace {
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, T12_WAVE));
+    return v;
+}
+
+// Block-wide sum / max over up to 16 waves; every thread gets the result.
+template <bool IS_MAX>
+__device__ __forceinline__ float block_reduce(float v, float* red /* >= 17 floats */)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    v = IS_MAX ? wave_max(v) : t12_wave_sum(v);
+    __syncthreads();                       // red may still be read from a previous call
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float r = red[0];
+    for (int w = 1; w < nw; w++) r = IS_MAX ? fmaxf(r, red[w]) : r + red[w];
+    return r;
+}
+
+// ---------------------------------------------------------------- embedding
+// hidden[b, i] = f32(embd[token_b, i]); an out-of-range id gives zeros (kernels.hip:57-73).
+__global__ __launch_bounds__(256) void embed_kernel(const uint16_t* __restrict__ embd, const int* __restrict__ tok,
+                                                    float* __restrict__ out, int n_embd, int n_vocab)
+{
+    const int b = blockIdx.y;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n_embd) return;
+    const int t = tok[b];
+    out[(size_t)b * n_embd + i] =
+        (t >= 0 && t < n_vocab) ? t12_bf16_to_f32(embd[(size_t)t * n_embd + i]) : 0.0f;
+}
+
+// ------------------------------------------------------------------ RMSNorm
+// y = bf16(x * rsqrt(mean(x^2) + eps) * w); with ADD: x += residual first, written back
+// (kernels.hip:355-392 and :399-442).  One workgroup per row, values kept in registers
+// between the two passes.
+template <bool ADD>
+__global__ __launch_bounds__(1024) void rms_norm_kernel(float* __restrict__ x, const float* __restrict__ res,
+                                                        const float* __restrict__ w, uint16_t* __restrict__ y,
+                                                        int n, float eps)
+{
+    __shared__ float red[17];
+    const size_t off = (size_t)blockIdx.x * n;
+    constexpr int MAXV = 8;                // up to 8 values per thread in registers (n <= 8 * blockDim)
+    float v[MAXV];
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < MAXV; j++) {
+        const int i = threadIdx.x + j * blockDim.x;
+        v[j] = 0.0f;
+        if (i < n) {
+            float t = x[off + i];
+            if (ADD) {
+                t += res[off + i];
+                x[off + i] = t;
+            }
+            v[j] = t;
+            ss += t * t;
+        }
+    }
+    for (int i = threadIdx.x + MAXV * blockDim.x; i < n; i += blockDim.x) {   // very wide rows
+        float t = x[off + i];
+        if (ADD) {
+            t += res[off + i];
+            x[off + i] = t;
+        }
+        ss += t * t;
+    }
+    ss = block_reduce<false>(ss, red);
+    const float r = rsqrtf(ss / (float)n + eps);
+#pragma unroll
+    for (int j = 0; j < MAXV; j++) {
+        const int i = threadIdx.x + j * blockDim.x;
+        if (i < n) y[off + i] = t12_f32_to_bf16(v[j] * r * w[i]);
+    }
+    for (int i = threadIdx.x + MAXV * blockDim.x; i < n; i += blockDim.x)
+        y[off + i] = t12_f32_to_bf16(x[off + i] * r * w[i]);
+}
+
+// ----------------------------------------------------------------- SiLU*mul
+// out = bf16( g / (1 + exp(-g)) * up )   (kernels.hip:447-459)
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                       uint16_t* __restrict__ out, size_t total)
+{
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i + 3 < total) {
+        const float4 g = *(const float4*)(gate + i);
+        const float4 u = *(const float4*)(up + i);
+        const uint32_t lo = t12_f32_to_bf16(g.x / (1.0f + expf(-g.x)) * u.x) |
+                            ((uint32_t)t12_f32_to_bf16(g.y / (1.0f + expf(-g.y)) * u.y) << 16);
+        const uint32_t hi = t12_f32_to_bf16(g.z / (1.0f + expf(-g.z)) * u.z) |
+                            ((uint32_t)t12_f32_to_bf16(g.w / (1.0f + expf(-g.w)) * u.w) << 16);
+        *(uint2*)(out + i) = make_uint2(lo, hi);
+    } else {
+        for (size_t j = i; j < total; j++) {
+            const float g = gate[j];
+            out[j] = t12_f32_to_bf16(g / (1.0f + expf(-g)) * up[j]);
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void add_kernel(float* __restrict__ y, const float* __restrict__ x, size_t total)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < total) y[i] += x[i];
+}
+
+// --------------------------------------------------------- RoPE + KV store
+// Rotate-half RoPE: pairs (d, d + hd/2), angle = pos * freq[d]  (kernels.hip:174-213, 717-754).
+// INT8 store per (position, kv head): scale = absmax / 127,
+// q = clamp(rint(v * (127 / absmax)), +-127)                    (kernels.hip:220-304, 760-845).
+// Grid: (n_head + 2 * n_head_kv, B); one wave per head.
+//   blocks [0, n_head)                     rotate a Q head in place
+//   blocks [n_head, n_head + nkv)          rotate a K head in place, then quantise + store it
+//   blocks [n_head + nkv, n_head + 2 nkv)  quantise + store a V head
+// MODE bit 0: do the rotations; bit 1: do the stores.
+template <int MODE>
+__global__ __launch_bounds__(64) void rope_kv_kernel(float* __restrict__ q, float* __restrict__ k,
+                                                     const float* __restrict__ v, int8_t* __restrict__ ck,
+                                                     int8_t* __restrict__ cv, float* __restrict__ sk,
+                                                     float* __restrict__ sv, const float* __restrict__ freqs,
+                                                     const int* __restrict__ positions, int position,
+                                                     int head_dim, int n_head, int n_head_kv, int q_stride,
+                                                     int k_stride)
+{
+    const int b = blockIdx.y;
+    const int pos = positions ? positions[b] : position;
+    const int lane = threadIdx.x;
+    const int half = head_dim >> 1;
+    int blk = blockIdx.x;
+    float* rot = nullptr;
+    const float* src = nullptr;
+    int8_t* dst = nullptr;
+    float* sdst = nullptr;
+    int kvh = 0;
+    if (blk < n_head) {
+        rot = q + (size_t)b * q_stride + (size_t)blk * head_dim;
+    } else if (blk < n_head + n_head_kv) {
+        kvh = blk - n_head;
+        rot = k + (size_t)b * k_stride + (size_t)kvh * head_dim;
+        src = rot;
+        dst = ck;
+        sdst = sk;
+    } else {
+        kvh = blk - n_head - n_head_kv;
+        src = v + (size_t)b * k_stride + (size_t)kvh * head_dim;
+        dst = cv;
+        sdst = sv;
+    }
+    // lane owns the pair (lane, lane + half); head_dim <= 128 so one pair per lane
+    const bool own = lane < half;
+    float r0 = 0.0f, r1 = 0.0f;
+    if ((MODE & 1) && rot) {
+        if (own) {
+            const float ang = (float)pos * freqs[lane];
+            float sn, cs;
+            sincosf(ang, &sn, &cs);
+            const float x0 = rot[lane], x1 = rot[lane + half];
+            r0 = x0 * cs - x1 * sn;
+            r1 = x0 * sn + x1 * cs;
+            rot[lane] = r0;
+            rot[lane + half] = r1;
+        }
+    } else if (src && own) {
+        r0 = src[lane];
+        r1 = src[lane + half];
+    }
+    if ((MODE & 2) && dst) {
+        const float amax = wave_max(fmaxf(fabsf(r0), fabsf(r1)));
+        const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+        const size_t kv_dim = (size_t)n_head_kv * head_dim;
+        int8_t* row = dst + (size_t)pos * kv_dim + (size_t)kvh * head_dim;
+        if (own) {
+            row[lane] = (int8_t)(int)fminf(fmaxf(rintf(r0 * inv), -127.0f), 127.0f);
+            row[lane + half] = (int8_t)(int)fminf(fmaxf(rintf(r1 * inv), -127.0f), 127.0f);
+        }
+        if (lane == 0) sdst[(size_t)pos * n_head_kv + kvh] = amax / 127.0f;
+    }
+}
+
+// ------------------------------------------------------- decode attention
+// out[b, h, :] = bf16( softmax_t( q[b,h] . (K8[t] * sk[t]) * scale ) . (V8[t] * sv[t]) ),
+// t in [0, seq_len), GQA: kv head = h / ratio.
+// Workgroup = (kv head, sequence b), 256 lanes; the `ratio` query heads of the
+// group are processed together.  Per 256-position tile:
+//   phase 1  lane = position: dot(q_h, K[t]) for every head of the group (K row read once)
+//   phase 2  online softmax bookkeeping per head (running max m, sum l)
+//   phase 3  wave = head (round robin), lane = 2 output dims: acc += p[t] * V[t]
+constexpr int ATT_TILE = 256;
+constexpr int ATT_MAX_RATIO = 16;
+
+__global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, const int8_t* __restrict__ ck,
+                                                          const int8_t* __restrict__ cv, const float* __restrict__ sk,
+                                                          const float* __restrict__ sv, uint16_t* __restrict__ out,
+                                                          const int* __restrict__ positions, int seq_len_arg,
+                                                          int n_head, int n_head_kv, int head_dim, float scale,
+                                                          size_t kv_stride)
+{
+    extern __shared__ float smem[];
+    const int ratio = n_head / n_head_kv;
+    float* qs = smem;                                   // [ratio][head_dim]
+    float* ps = qs + ratio * head_dim;                  // [ratio][ATT_TILE] scores / probabilities
+    float* red = ps + ratio * ATT_TILE;                 // [17]
+    float* stat = red + 17;                             // [ratio][2]: running max, tile rescale
+    const int kvh = blockIdx.x, b = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int seq_len = positions ? positions[b] + 1 : seq_len_arg;
+    const size_t kv_dim = (size_t)n_head_kv * head_dim;
+    const int8_t* kbase = ck + (size_t)b * kv_stride + (size_t)kvh * head_dim;
+    const int8_t* vbase = cv + (size_t)b * kv_stride + (size_t)kvh * head_dim;
+    const size_t sstride = kv_stride / head_dim;        // scale arrays: kv_stride / head_dim per sequence
+    const float* skb = sk + (size_t)b * sstride + kvh;
+    const float* svb = sv + (size_t)b * sstride + kvh;
+    const float* qb = q + (size_t)b * n_head * head_dim + (size_t)kvh * ratio * head_dim;
+
+    for (int i = tid; i < ratio * head_dim; i += 256) qs[i] = qb[i];
+    if (tid < ratio) stat[2 * tid] = -1e30f;
+    __syncthreads();
+
+    // per-head running sums live in the lanes that own the output: wave w owns heads w, w+4, ...
+    constexpr int MAX_OWN = ATT_MAX_RATIO / 4;
+    float o0[MAX_OWN], o1[MAX_OWN], lsum[MAX_OWN];
+#pragma unroll
+    for (int j = 0; j < MAX_OWN; j++) o0[j] = o1[j] = lsum[j] = 0.0f;
+    const int nd2 = head_dim >> 1;                      // lanes cover dims 2*lane, 2*lane+1 (+128 per extra pass)
+
+    for (int t0 = 0; t0 < seq_len; t0 += ATT_TILE) {
+        const int tl = min(ATT_TILE, seq_len - t0);
+        // phase 1: scores
+        if (tid < tl) {
+            const int t = t0 + tid;
+            const int8_t* kr = kbase + (size_t)t * kv_dim;
+            const float kscale = skb[(size_t)t * n_head_kv] * scale;
+            float dot[ATT_MAX_RATIO];
+#pragma unroll
+            for (int h = 0; h < ATT_MAX_RATIO; h++) dot[h] = 0.0f;
+            for (int d = 0; d < head_dim; d += 16) {
+                const uint4 kk = *(const uint4*)(kr + d);
+                const uint32_t w4[4] = {kk.x, kk.y, kk.z, kk.w};
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const float kv = (float)(int8_t)((w4[e >> 2] >> (8 * (e & 3))) & 0xFF);
+#pragma unroll
+                    for (int h = 0; h < ATT_MAX_RATIO; h++)
+                        if (h < ratio) dot[h] += qs[h * head_dim + d + e] * kv;
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < ATT_MAX_RATIO; h++)
+                if (h < ratio) ps[h * ATT_TILE + tid] = dot[h] * kscale;
+        }
+        __syncthreads();
+        // phase 2: per head tile max -> new running max, rescale factor, probabilities
+        for (int h = 0; h < ratio; h++) {
+            const float sc = tid < tl ? ps[h * ATT_TILE + tid] : -1e30f;
+            const float tmax = block_reduce<true>(sc, red);
+            const float m_old = stat[2 * h];
+            const float m_new = fmaxf(m_old, tmax);
+            if (tid < tl) ps[h * ATT_TILE + tid] = expf(sc - m_new);
+            __syncthreads();                             // everyone has read m_old
+            if (tid == 0) {
+                stat[2 * h] = m_new;
+                stat[2 * h + 1] = expf(m_old - m_new);
+            }
+        }
+        __syncthreads();
+        // phase 3: P.V for the heads this wave owns
+#pragma unroll
+        for (int j = 0; j < MAX_OWN; j++) {
+            const int h = wave + 4 * j;
+            if (h < ratio) {
+                const float corr = stat[2 * h + 1];
+                float a0 = o0[j] * corr, a1 = o1[j] * corr, ls = lsum[j] * corr;
+                if (lane < nd2) {
+                    for (int t = 0; t < tl; t++) {
+                        const float pv = ps[h * ATT_TILE + t];
+                        const float w = pv * svb[(size_t)(t0 + t) * n_head_kv];
+                        const uint16_t two = *(const uint16_t*)(vbase + (size_t)(t0 + t) * kv_dim + 2 * lane);
+                        a0 += w * (float)(int8_t)(two & 0xFF);
+                        a1 += w * (float)(int8_t)(two >> 8);
+                        ls += pv;
+                    }
+                }
+                o0[j] = a0;
+                o1[j] = a1;
+                lsum[j] = ls;
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int j = 0; j < MAX_OWN; j++) {
+        const int h = wave + 4 * j;
+        if (h < ratio && lane < nd2) {
+            const float inv = 1.0f / lsum[j];
+            uint16_t* o = out + (size_t)b * n_head * head_dim + (size_t)(kvh * ratio + h) * head_dim + 2 * lane;
+            *(uint32_t*)o = t12_f32_to_bf16(o0[j] * inv) | ((uint32_t)t12_f32_to_bf16(o1[j] * inv) << 16);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ argmax
+// Lowest index among equal maxima (the reference's tie rule depends on its
+// thread layout, kernels.hip:103-118; exact ties between fp32 logits do not
+// occur in practice).  NaN never wins, like the reference's strict '>'.
+struct ArgPair {
+    float v;
+    int i;
+};
+__device__ __forceinline__ ArgPair better(ArgPair a, ArgPair b)
+{
+    return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a;
+}
+__device__ __forceinline__ ArgPair block_argmax(ArgPair p, ArgPair* sh /* [4] */)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        ArgPair o;
+        o.v = __shfl_xor(p.v, off, T12_WAVE);
+        o.i = __shfl_xor(p.i, off, T12_WAVE);
+        p = better(p, o);
+    }
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = p;
+    __syncthreads();
+    ArgPair r = sh[0];
+    for (int w = 1; w < (int)(blockDim.x >> 6); w++) r = better(r, sh[w]);
+    return r;
+}
+
+constexpr int ARG_CHUNKS = 64;
+
+__global__ __launch_bounds__(256) void argmax_part_kernel(const float* __restrict__ logits, int n,
+                                                          ArgPair* __restrict__ part)
+{
+    __shared__ ArgPair sh[4];
+    const int row = blockIdx.y, chunk = blockIdx.x;
+    const int per = (n + ARG_CHUNKS - 1) / ARG_CHUNKS;
+    const int lo = chunk * per, hi = min(n, lo + per);
+    const float* x = logits + (size_t)row * n;
+    ArgPair p = {-INFINITY, 0x7FFFFFFF};
+    for (int i = lo + threadIdx.x; i < hi; i += 256) {
+        const float v = x[i];
+        if (v > p.v) { p.v = v; p.i = i; }
+    }
+    p = block_argmax(p, sh);
+    if (threadIdx.x == 0) part[(size_t)row * ARG_CHUNKS + chunk] = p;
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(const ArgPair* __restrict__ part, int* __restrict__ result)
+{
+    __shared__ ArgPair sh[1];
+    ArgPair p = part[(size_t)blockIdx.x * ARG_CHUNKS + threadIdx.x];
+    p = block_argmax(p, sh);
+    if (threadIdx.x == 0) result[blockIdx.x] = p.i == 0x7FFFFFFF ? 0 : p.i;
+}
+
+// ---- library-owned device state: RoPE table (keyed by head_dim AND theta) and the
+//      argmax partial buffer.  Guarded for use from several host threads.
+std::mutex g_mu;
+float* g_freqs = nullptr;
+int g_freqs_dim = 0;
+float g_freqs_theta = 0.0f;
+ArgPair* g_part = nullptr;
+int g_part_rows = 0;
+
+const float* rope_table(int head_dim, float theta)
+{
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (g_freqs && g_freqs_dim == head_dim && g_freqs_theta == theta) return g_freqs;
+    const int half = head_dim / 2;
+    std::vector<float> h(half);
+    for (int d = 0; d < half; d++) h[d] = 1.0f / powf(theta, (float)(2 * d) / (float)head_dim);   // kernels.hip:133-134
+    if (g_freqs) (void)hipFree(g_freqs);
+    g_freqs = nullptr;
+    if (hipMalloc((void**)&g_freqs, half * sizeof(float)) != hipSuccess) return nullptr;
+    if (hipMemcpy(g_freqs, h.data(), half * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) return nullptr;
+    g_freqs_dim = head_dim;
+    g_freqs_theta = theta;
+    return g_freqs;
+}
+
+ArgPair* argmax_scratch(int rows)
+{
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (g_part_rows < rows) {
+        if (g_part) (void)hipFree(g_part);
+        g_part = nullptr;
+        g_part_rows = 0;
+        const int want = rows < 256 ? 256 : rows;
+        if (hipMalloc((void**)&g_part, (size_t)want * ARG_CHUNKS * sizeof(ArgPair)) != hipSuccess) return nullptr;
+        g_part_rows = want;
+    }
+    return g_part;
+}
+
+void report(const char* what)
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        t12_set_error("%s: %s", what, hipGetErrorString(e));
+        fprintf(stderr, "turbo12: %s: %s\n", what, hipGetErrorString(e));
+    }
+}
+
+template <int MODE>
+void launch_rope_kv(float* q, float* k, const float* v, int8_t* ck, int8_t* cv, float* sk, float* sv,
+                    const int* positions, int position, int head_dim, int n_head, int n_head_kv, int q_stride,
+                    int k_stride, float theta, int batch, hipStream_t st)
+{
+    const float* f = nullptr;
+    if (MODE & 1) {
+        f = rope_table(head_dim, theta);
+        if (!f) { t12_set_error("rope: cannot build the frequency table"); return; }
+    }
+    if (head_dim > 128 || (head_dim & 1)) {
+        t12_set_error("rope/kv-store: head_dim %d unsupported (even, <= 128)", head_dim);
+        fprintf(stderr, "turbo12: %s\n", t12_last_error());
+        return;
+    }
+    hipLaunchKernelGGL(rope_kv_kernel<MODE>, dim3(n_head + 2 * n_head_kv, batch), dim3(64), 0, st, q, k, v, ck, cv, sk,
+                       sv, f, positions, position, head_dim, n_head, n_head_kv, q_stride, k_stride);
+    report("rope/kv-store");
+}
+
+void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float* sk, const float* sv, int16_t* out,
+                 const int* positions, int seq_len, int n_head, int n_head_kv, int head_dim, float scale, int batch,
+                 size_t kv_stride, hipStream_t st)
+{
+    const int ratio = n_head / n_head_kv;
+    if (ratio < 1 || ratio > ATT_MAX_RATIO || n_head % n_head_kv || head_dim % 16 || head_dim > 128) {
+        t12_set_error("attention: unsupported heads %d/%d or head_dim %d (needs ratio <= %d, head_dim %% 16 == 0, <= 128)",
+                      n_head, n_head_kv, head_dim, ATT_MAX_RATIO);
+        fprintf(stderr, "turbo12: %s\n", t12_last_error());
+        return;
+    }
+    const size_t smem = ((size_t)ratio * head_dim + (size_t)ratio * ATT_TILE + 17 + 2 * ratio) * sizeof(float);
+    hipLaunchKernelGGL(attn_decode_kernel, dim3(n_head_kv, batch), dim3(256), smem, st, q, ck, cv, sk, sv,
+                       (uint16_t*)out, positions, seq_len, n_head, n_head_kv, head_dim, scale, kv_stride);
+    report("attention");
+}
+
+}  // namespace
+
+// ---- C launchers: names and signatures of engine/inference.cpp:9-20 / sampler.cpp:4-5 ----
+extern "C" {
+
+void launch_rope_init(int head_dim, float theta_base) { (void)rope_table(head_dim, theta_base); }
+
+void launch_embed_lookup(const int16_t* embd_table, const int* token_ids, float* output, int n_embd, int batch_size,
+                         int n_vocab, hipStream_t stream)
+{
+    hipLaunchKernelGGL(embed_kernel, dim3((n_embd + 255) / 256, batch_size), dim3(256), 0, stream,
+                       (const uint16_t*)embd_table, token_ids, output, n_embd, n_vocab);
+    report("embed_lookup");
+}
+
+static int norm_threads(int n)
+{
+    int t = (n + 7) / 8;                   // 8 values per thread stay in registers
+    t = (t + 63) / 64 * 64;
+    return t < 64 ? 64 : (t > 1024 ? 1024 : t);
+}
+
+void launch_rms_norm_bf16_batch(const float* x, const float* weight, int16_t* y, int n, float eps, int batch_size,
+                                hipStream_t stream)
+{
+    hipLaunchKernelGGL(rms_norm_kernel<false>, dim3(batch_size), dim3(norm_threads(n)), 0, stream, (float*)x,
+                       (const float*)nullptr, weight, (uint16_t*)y, n, eps);
+    report("rms_norm");
+}
+
+void launch_add_rms_norm_bf16_batch(float* x, const float* residual, const float* weight, int16_t* y, int n, float eps,
+                                    int batch_size, hipStream_t stream)
+{
+    hipLaunchKernelGGL(rms_norm_kernel<true>, dim3(batch_size), dim3(norm_threads(n)), 0, stream, x, residual, weight,
+                       (uint16_t*)y, n, eps);
+    report("add_rms_norm");
+}
+
+void launch_silu_mul_bf16_batch(const float* gate, const float* up, int16_t* out, int n, int batch_size,
+                                hipStream_t stream)
+{
+    const size_t total = (size_t)n * batch_size;
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0, stream, gate, up,
+                       (uint16_t*)out, total);
+    report("silu_mul");
+}
+
+void launch_add_batch(float* y, const float* x, int n, int batch_size, hipStream_t stream)
+{
+    const size_t total = (size_t)n * batch_size;
+    hipLaunchKernelGGL(add_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, y, x, total);
+    report("add");
+}
+
+void launch_rope_batch(float* q, float* k, const int* positions, int head_dim, int n_head, int n_head_kv, int q_stride,
+                       int k_stride, float theta, int batch_size, hipStream_t stream)
+{
+    launch_rope_kv<1>(q, k, nullptr, nullptr, nullptr, nullptr, nullptr, positions, 0, head_dim, n_head, n_head_kv,
+                      q_stride, k_stride, theta, batch_size, stream);
+}
+
+void launch_store_kv_batch(const float* k, const float* v, int8_t* kv_k, int8_t* kv_v, float* scale_k, float* scale_v,
+                           const int* positions, int kv_dim, int max_seq, int n_head_kv, int head_dim, int batch_size,
+                           hipStream_t stream)
+{
+    (void)max_seq;
+    launch_rope_kv<2>(nullptr, (float*)k, v, kv_k, kv_v, scale_k, scale_v, positions, 0, head_dim, 0, n_head_kv, 0,
+                      kv_dim, 1.0f, batch_size, stream);
+}
+
+void launch_rope_store_kv(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v, float* scale_k,
+                          float* scale_v, int head_dim, int n_head, int n_head_kv, int position, int max_seq,
+                          float theta, hipStream_t stream)
+{
+    (void)max_seq;
+    launch_rope_kv<3>(q, k, v, kv_k, kv_v, scale_k, scale_v, nullptr, position, head_dim, n_head, n_head_kv,
+                      n_head * head_dim, n_head_kv * head_dim, theta, 1, stream);
+}
+
+// Extension of the reference's launch layer: RoPE + INT8 store for a whole batch in one launch.
+void launch_rope_store_kv_batch(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v, float* scale_k,
+                                float* scale_v, const int* positions, int head_dim, int n_head, int n_head_kv,
+                                int q_stride, int k_stride, float theta, int batch_size, hipStream_t stream)
+{
+    launch_rope_kv<3>(q, k, v, kv_k, kv_v, scale_k, scale_v, positions, 0, head_dim, n_head, n_head_kv, q_stride,
+                      k_stride, theta, batch_size, stream);
+}
+
+void launch_attention_all_heads(const float* q, const int8_t* k_cache, const int8_t* v_cache, const float* scale_k,
+                                const float* scale_v, int16_t* output, int n_head, int n_head_kv, int head_dim,
+                                int seq_len, int max_seq, float scale, hipStream_t stream)
+{
+    (void)max_seq;
+    launch_attn(q, k_cache, v_cache, scale_k, scale_v, output, nullptr, seq_len, n_head, n_head_kv, head_dim, scale, 1,
+                0, stream);
+}
+
+void launch_flash_attention(const float* q, const int8_t* k_cache, const int8_t* v_cache, const float* scale_k,
+                            const float* scale_v, int16_t* output, int n_head, int n_head_kv, int head_dim, int seq_len,
+                            int max_seq, float scale, hipStream_t stream)
+{
+    launch_attention_all_heads(q, k_cache, v_cache, scale_k, scale_v, output, n_head, n_head_kv, head_dim, seq_len,
+                               max_seq, scale, stream);
+}
+
+void launch_attention_all_heads_batch(const float* q, const int8_t* kv_k, const int8_t* kv_v, const float* scale_k,
+                                      const float* scale_v, int16_t* output, const int* positions, int n_head,
+                                      int n_head_kv, int head_dim, int max_seq, float scale, int batch_size,
+                                      int kv_stride, hipStream_t stream)
+{
+    (void)max_seq;
+    launch_attn(q, kv_k, kv_v, scale_k, scale_v, output, positions, 0, n_head, n_head_kv, head_dim, scale, batch_size,
+                (size_t)kv_stride, stream);
+}
+
+void launch_flash_attention_batch(const float* q, const int8_t* kv_k, const int8_t* kv_v, const float* scale_k,
+                                  const float* scale_v, int16_t* output, const int* positions, int n_head,
+                                  int n_head_kv, int head_dim, int max_seq, float scale, int batch_size, int kv_stride,
+                                  hipStream_t stream)
+{
+    launch_attention_all_heads_batch(q, kv_k, kv_v, scale_k, scale_v, output, positions, n_head, n_head_kv, head_dim,
+                                     max_seq, scale, batch_size, kv_stride, stream);
+}
+
+void launch_argmax_batch(const float* logits, int* results, int n_vocab, int batch_size, hipStream_t stream)
+{
+    ArgPair* part = argmax_scratch(batch_size);
+    if (!part) { t12_set_error("argmax: cannot allocate scratch"); return; }
+    hipLaunchKernelGGL(argmax_part_kernel, dim3(ARG_CHUNKS, batch_size), dim3(256), 0, stream, logits, n_vocab, part);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(batch_size), dim3(64), 0, stream, part, results);
+    report("argmax");
+}
+
+void launch_argmax(const float* logits, int* result, int n, hipStream_t stream)
+{
+    launch_argmax_batch(logits, result, n, 1, stream);
+}
+
+}  // extern "C"
