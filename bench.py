@@ -7,6 +7,13 @@ Workloads (synthetic, seeded, random-init weights of the Llama-3.1-8B shape:
 32 layers, hidden 4096, FFN 14336, 32/8 heads, vocab 128256; N(0, 0.02) with
 3e-4 of the entries replaced by N(0, 8) outliers so that ~0.045 % escape):
 
+  decode (default) one step = one greedy decode step of the full engine (embedding, 32 x [RMSNorm, fused
+                  QKV decode-GEMV, RoPE + INT8 KV store, GQA attention, O, add+RMSNorm, fused gate|up,
+                  SiLU*mul, down, add+RMSNorm], lm_head, argmax + D2H) on a model generated and packed on
+                  the GPU; prompt 128 random ids, 2048-token KV cache (BASELINE config 4).  B = 1 is
+                  `value`; B = 256 is measured in the same run and reported under "b256"; the
+                  decode-GEMV launches of a step are also timed alone for `roofline`.
+
   gemv_stack_b1   one step = every linear layer of one decode step at B = 1 through
                   the fused split-12 decode-GEMV: per layer QKV (3 segments, one
                   launch), O, gate+up (2 segments, one launch), down; then lm_head.
@@ -83,14 +90,11 @@ def build_stack(t12, torch, dev, cfg, base_seed=4000):
     return launches
 
 
-def cpu_baseline(torch, launches, cfg, runs=3):
+def cpu_baseline(torch, launches, cfg, runs=3, n_weights_model=None):
     """Times the CPU oracle on the first decoder layer (7 tensors, 218 M weights) and scales
     the per-weight rate to the whole model."""
     import numpy as np
     from oracle import oracle
-
-    class P:  # the oracle's Packed duck type, filled from device arrays
-        pass
 
     packs = []
     for tensors, key in launches[:4]:
@@ -109,7 +113,7 @@ def cpu_baseline(torch, launches, cfg, runs=3):
         times.append(time.perf_counter() - t0)
     t_layer = sorted(times)[len(times) // 2]
     w_layer = sum(p.M * p.K for p in packs)
-    w_model = sum(t.M * t.K for tensors, _ in launches for t in tensors)
+    w_model = n_weights_model or sum(t.M * t.K for tensors, _ in launches for t in tensors)
     t_model = t_layer * w_model / w_layer
     return {
         "value": 1.0 / t_model, "unit": "tok/s", "cores": oracle.num_threads(), "kind": "port",
@@ -119,12 +123,162 @@ def cpu_baseline(torch, launches, cfg, runs=3):
     }
 
 
+def ext_stream(torch, ptr):
+    return torch.cuda.ExternalStream(ptr)
+
+
+def timed(torch, stream, fn, steps):
+    """HIP events recorded on the stream the kernels run on, bracketed by synchronisation."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    w0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(steps):
+        fn()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - w0) * 1e3 / steps
+    return max(e0.elapsed_time(e1) / steps, wall), e0.elapsed_time(e1) / steps
+
+
+def run_decode(args, t12, torch, dev):
+    """Full greedy decode on a random-init Llama-3.1-8B-shaped model generated and packed on the GPU
+    (BASELINE config 4): prompt of 128 random ids, 2048-token KV cache, one forward + one greedy sample
+    per step; B = 1 is `value`, B = 256 (256 lock-step copies sharing the cache, the reference's batched
+    mode) is reported next to it."""
+    import numpy as np
+    cfg = dict(LLAMA8B, n_layer=args.layers, n_ctx=2048, rope_theta=500000.0, rms_norm_eps=1e-5)
+    t0 = time.time()
+    eng = t12.Engine.synthetic(cfg, seed=4000, max_seq=2048, batch=1)
+    torch.cuda.synchronize()
+    t_build = time.time() - t0
+    rng = np.random.default_rng(4001)
+    prompt = [int(t) for t in rng.integers(3, cfg["n_vocab"], size=args.prompt)]
+
+    def decode_loop(e, B):
+        st = ext_stream(torch, t12.lib.t12_engine_stream(e.state))
+        for i, t in enumerate(prompt):                      # prefill, one token per forward (inference.cpp:721-724)
+            e.set_positions([i] * B)
+            e.forward([t] * B)
+        state = {"tok": e.sample()}
+
+        def step():
+            e.forward(state["tok"])
+            state["tok"] = e.sample()                       # D2H + stream sync per token (sampler.cpp:18-32)
+        for _ in range(args.warmup):
+            step()
+        return timed(torch, st, step, args.steps)
+
+    ms1, _ = decode_loop(eng, 1)
+
+    # ---- roofline of the dominant kernel: the GEMV launches of one step, alone, on the current stream
+    n_l = cfg["n_layer"]
+    hd = cfg["n_embd"] // cfg["n_head"]
+    kvd = cfg["n_head_kv"] * hd
+    g = torch.Generator(device=dev)
+    g.manual_seed(99)
+    acts = {cfg["n_embd"]: torch.randn(cfg["n_embd"], generator=g, device=dev).to(torch.bfloat16),
+            cfg["n_ff"]: torch.randn(cfg["n_ff"], generator=g, device=dev).to(torch.bfloat16)}
+    scratch = torch.empty(cfg["n_vocab"] + 2 * cfg["n_ff"], dtype=torch.float32, device=dev)
+    tabs, alg_bytes, plane_bytes, n_weights, n_esc = [], 0.0, 0.0, 0, 0
+    groups = [(0, 1, 2), (3,), (4, 5), (6,)]
+    for layer in list(range(n_l)) + [-1]:
+        for grp in (groups if layer >= 0 else [(0,)]):
+            segs, off, K = [], 0, None
+            for which in grp:
+                seg, K, P = eng.weight(layer, which)
+                seg.out = scratch.data_ptr() + 4 * off
+                off += seg.M
+                segs.append(seg)
+                alg_bytes += 1.5 * seg.M * K + 8 * P + 4 * (seg.M + 1) + 4 * seg.M
+                plane_bytes += 1.5 * seg.M * K
+                n_weights += seg.M * K
+                n_esc += P
+            alg_bytes += 2 * K
+            tabs.append((t12._seg_array(segs), len(segs), acts[K].data_ptr(), K))
+    cur = torch.cuda.current_stream()
+
+    def gemv_pass():
+        for segs, n, act, K in tabs:
+            rc = t12.lib.t12_gemv(segs, n, act, K, cur.cuda_stream)
+            if rc:
+                t12.check(rc, "t12_gemv")
+    for _ in range(3):
+        gemv_pass()
+    _, ms_gemv = timed(torch, cur, gemv_pass, max(args.steps, 10))
+    achieved = alg_bytes / (ms_gemv * 1e-3) / 1e9
+
+    # ---- B = 256
+    b256 = None
+    if args.batch256:
+        e256 = eng.new_state(256)
+        ms256, _ = decode_loop(e256, 256)
+        b256 = {"tok_s": 256e3 / ms256, "ms_per_step": ms256, "batch": 256,
+                "note": "256 lock-step copies of one stream sharing one KV-cache region (the reference's batched mode)"}
+        e256.close()
+
+    result = {
+        "metric": "tok/s at B=1 (Llama-3.1-8B shape), greedy decode of a split-12 model; B=256 and decode-GEMV GB/s alongside",
+        "value": 1e3 / ms1, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms1, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": (1e3 / ms1) / 57.0 if n_l == LLAMA8B["n_layer"] else None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "decode_b1: random-init Llama-3.1-8B shape (32 layers, 4096/14336, 32/8 heads, vocab 128256), "
+                               "split-12 weights N(0,0.02)+3e-4 outliers, prompt %d random ids, greedy decode, 2048-token INT8 "
+                               "KV cache, one forward + sample per step" % args.prompt,
+                   "batch": 1, "n_layer": n_l, "weights": n_weights, "compressed_GB_per_step": plane_bytes / 1e9,
+                   "escape_fraction": n_esc / max(n_weights, 1),
+                   "baseline": "57.0 tok/s, Llama 3.1 8B B=1 on RTX 5070 Ti (reference README.md:46)"},
+        "b256": b256,
+        "gemv_compressed_GBps": plane_bytes / (ms_gemv * 1e-3) / 1e9,
+        "gemv_only_ms_per_step": ms_gemv,
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["gemv_stack_b1"] if n_l == LLAMA8B["n_layer"] else None,
+                     "kernel": "gemv_stream_kernel", "bytes_per_launch": alg_bytes / len(tabs),
+                     "us_per_launch": ms_gemv * 1e3 / len(tabs)},
+        "setup_s": t_build,
+    }
+    if not args.no_cpu_baseline:
+        # the same oracle leg as the stack workload, on layer 0 of this model
+        class T:
+            pass
+        launches = []
+        for grp in groups:
+            ts = []
+            for which in grp:
+                seg, K, P = eng.weight(0, which)
+                t = T()
+                t.M, t.K, t.base_exp = seg.M, K, seg.base_exp
+
+                def pull(ptr, n, dt):
+                    if n == 0 or not ptr:
+                        return torch.zeros(0, dtype=dt)
+                    out = torch.empty(n, dtype=dt, device=dev)
+                    t12._hip_memcpy_d2d(out.data_ptr(), ptr, n * out.element_size())
+                    return out.cpu()
+                t.sm = pull(seg.sm, seg.M * K, torch.uint8)
+                t.gr = pull(seg.gr, (seg.M * K + 1) // 2, torch.uint8)
+                t.row_off = pull(seg.row_off, seg.M + 1, torch.int32) if P else torch.zeros(seg.M + 1, dtype=torch.int32)
+                t.cols = pull(seg.cols, P, torch.int32)
+                t.correct = pull(seg.correct, P, torch.int16)
+                t.wrong = pull(seg.wrong, P, torch.int16)
+                t.P = P
+                ts.append(t)
+            launches.append((ts, None))
+        result["cpu_baseline"] = cpu_baseline(torch, launches, cfg, n_weights_model=n_weights)
+    eng.close()
+    return result
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gemv_stack_b1")
+    ap.add_argument("--workload", default="decode", choices=["decode", "gemv_stack_b1"])
+    ap.add_argument("--prompt", type=int, default=128)
+    ap.add_argument("--no-batch256", dest="batch256", action="store_false")
     ap.add_argument("--layers", type=int, default=LLAMA8B["n_layer"], help="debug: fewer layers (invalid as a result)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
@@ -141,6 +295,9 @@ def main():
     t12 = ge.load_package()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "decode":
+        print(json.dumps(run_decode(args, t12, torch, dev)))
+        return
     cfg = dict(LLAMA8B, n_layer=args.layers)
 
     t0 = time.time()

@@ -78,9 +78,10 @@ int t12_tune_gemv(int variant);
  * array (it travels as a kernel argument; no device copy is made). */
 int t12_gemv(const T12Segment* segs, int nseg, const void* act_bf16, int K, void* stream);
 
-/* ---- (a') small-batch decode-GEMV, 1 <= B <= 8 ----------------------------
- * Same as t12_gemm but guaranteed to take the bandwidth-bound vector path.
- * Replaces launch_split12_batch4_async / _batch8_async (decompress_v2.hip:860,877). */
+/* ---- (a') small batch, 1 <= B <= 8 -----------------------------------------
+ * Same contract as t12_gemm, restricted to the batch sizes of the reference's
+ * launch_split12_batch4_async / _batch8_async (decompress_v2.hip:860,877), with
+ * the escapes taken from the CSR list instead of the derived escape tables. */
 int t12_gemv_batch(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride,
                    int out_stride, int K, int B, void* stream);
 

@@ -195,3 +195,42 @@ def test_full_size_linearity(t12, oracle, synth):
     assert rel_err((o1 + o2).cpu().numpy(), o.cpu().numpy()) < 1e-5
     ref = oracle.gemv(p, x)
     assert rel_err(o.cpu().numpy(), ref) < TOL
+
+
+@pytest.mark.parametrize("NB", [4, 8])
+def test_reference_named_batch_launchers(t12, oracle, synth, NB):
+    """launch_split12_batch4/8_async take the derived escape tables of the reference's loader
+    (esc_row_base / esc_counts / esc_vals, engine/model.cpp:86-160); esc_counts may be NULL here."""
+    M, K = 96, 2304
+    p = oracle.pack(synth.weights_llm(M, K, seed=50 + NB, p_outlier=5e-3))
+    row_base, counts, vals, _ = oracle.escape_tables(p)
+    X = synth.activations(NB, K, seed=60)
+    ref = oracle.gemm(p, X)
+    d = t12.DeviceTensor12.from_packed(p, dev())
+    acts = [to_dev_bits(X[j]) for j in range(NB)]
+    rb, cn, vl = (torch.from_numpy(a).to(dev()) for a in (row_base, counts, vals))
+    fn = t12.lib.launch_split12_batch4_async if NB == 4 else t12.lib.launch_split12_batch8_async
+    for use_counts in (True, False):
+        outs = [torch.zeros(M, device=dev()) for _ in range(NB)]
+        args = [d.sm.data_ptr(), d.gr.data_ptr(), d.base_exp] + [a.data_ptr() for a in acts] + \
+               [rb.data_ptr(), cn.data_ptr() if use_counts else None, vl.data_ptr()] + \
+               [o.data_ptr() for o in outs] + [M, K, t12.current_stream()]
+        t12.check(fn(*args))
+        torch.cuda.synchronize()
+        for j in range(NB):
+            assert rel_err(outs[j].cpu().numpy(), ref[j]) < TOL, (use_counts, j)
+
+
+def test_gemv_batch_entry_point(t12, oracle, synth):
+    M, K = 200, 2048
+    p = oracle.pack(synth.weights_llm(M, K, seed=70, p_outlier=2e-3))
+    d = t12.DeviceTensor12.from_packed(p, dev())
+    for B in (1, 3, 8):
+        X = synth.activations(B, K, seed=71 + B)
+        Xd = to_dev_bits(X).reshape(B, K)
+        out = torch.zeros((B, M), device=dev())
+        segs = t12._seg_array([d.segment(out)])
+        t12.check(t12.lib.t12_gemv_batch(segs, 1, Xd.data_ptr(), K, M, K, B, t12.current_stream()))
+        torch.cuda.synchronize()
+        assert rel_err(out.cpu().numpy(), oracle.gemm(p, X)) < TOL
+    assert t12.lib.t12_gemv_batch(segs, 1, Xd.data_ptr(), K, M, K, 9, None) == -1

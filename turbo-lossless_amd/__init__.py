@@ -84,6 +84,9 @@ _SIGS = {
     "t12_engine_generate": (_i, [_vp, C.POINTER(C.c_int), _i, _i, C.POINTER(C.c_int)]),
     "t12_engine_sync": (_i, [_vp]),
     "t12_engine_weight": (_i, [_vp, _i, _i, C.POINTER(Segment), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "t12_gemv_batch": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
+    "launch_split12_batch4_async": (_i, [_vp] * 2 + [_i] + [_vp] * 4 + [_vp] * 3 + [_vp] * 4 + [_i, _i, _vp]),
+    "launch_split12_batch8_async": (_i, [_vp] * 2 + [_i] + [_vp] * 8 + [_vp] * 3 + [_vp] * 8 + [_i, _i, _vp]),
     "t12_gemm": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_tune_gemm": (_i, [_i]),
     "t12_decompress": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
