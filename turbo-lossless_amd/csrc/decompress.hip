@@ -22,6 +22,7 @@ __global__ __launch_bounds__(256) void decompress_vec_kernel(const uint8_t* __re
                                                              size_t n16)
 {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
+    be2 = t12_opaque(be2);
     for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < n16; q += stride) {
         const uint4 S = t12_ldg_stream16(sm + q * 16);
         const uint2 G = t12_ldg_stream8(gr + q * 8);

@@ -96,19 +96,18 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
     const int k_begin = blockIdx.z * p.kslice;
     const int k_end = min(K, k_begin + p.kslice);
     const int nstage = (k_end - k_begin) / KC;
-    const uint32_t be2 = ((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23);
+    const uint32_t be2 = t12_opaque(((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23));
 
     // ---- this thread's share of the global -> LDS staging
     //  acts: unit idx = tid + 256*i -> row idx / 8, unit idx % 8 (8 lanes = 128 contiguous bytes)
     //  sm / gr: unit idx = tid + 256*i (i < 2) -> row idx / 4, unit idx % 4
+    // batch rows >= B are clamped to row B-1: their products are computed and never stored
     const uint16_t* a_src[ACT_LD];
     int a_dst[ACT_LD];
-    bool a_ok[ACT_LD];
 #pragma unroll
     for (int i = 0; i < ACT_LD; i++) {
         const int idx = tid + 256 * i;
         const int r = idx >> 3, u = idx & 7;
-        a_ok[i] = b0 + r < B;
         a_src[i] = p.act + (size_t)min(b0 + r, B - 1) * p.act_stride + k_begin + u * 8;
         a_dst[i] = (u * TB + r) * 16;
     }
@@ -126,31 +125,32 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
         g_dst[i] = ACT_UNITS * 16 + TM * 64 + (c * TM + r) * 8;
     }
 
-    uint4 ra[ACT_LD];
-    uint4 rs[2];
-    uint2 rg[2];
-    auto load_stage = [&](int st) {
-#pragma unroll
-        for (int i = 0; i < ACT_LD; i++) {
-            ra[i] = make_uint4(0, 0, 0, 0);
-            if (a_ok[i]) ra[i] = *(const uint4*)(a_src[i] + (size_t)st * KC);
-        }
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            rs[i] = t12_ldg_stream16(s_src[i] + (size_t)st * KC);
-            rg[i] = t12_ldg_stream8(g_src[i] + (size_t)st * (KC / 2));
-        }
-    };
-    auto store_stage = [&](int buf) {
-        uint8_t* base = lds + buf * STAGE_BYTES;
-#pragma unroll
-        for (int i = 0; i < ACT_LD; i++) *(uint4*)(base + a_dst[i]) = t12_pair_acts(ra[i]);
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            *(uint4*)(base + s_dst[i]) = rs[i];
-            *(uint2*)(base + g_dst[i]) = rg[i];
-        }
-    };
+    // Register ring: the global loads of stage st + D are issued while stage st is
+    // being multiplied (HBM latency is longer than one stage of MFMAs); a stage moves
+    // registers -> LDS one iteration before it is consumed (double-buffered LDS).
+    constexpr int D = 3;
+    uint4 ra[D][ACT_LD];
+    uint4 rs[D][2];
+    uint2 rg[D][2];
+#define T12_LOAD_STAGE(slot, st)                                                        \
+    {                                                                                   \
+        _Pragma("unroll") for (int i = 0; i < ACT_LD; i++)                              \
+            ra[slot][i] = *(const uint4*)(a_src[i] + (size_t)(st) * KC);                \
+        _Pragma("unroll") for (int i = 0; i < 2; i++) {                                 \
+            rs[slot][i] = t12_ldg_stream16(s_src[i] + (size_t)(st) * KC);               \
+            rg[slot][i] = t12_ldg_stream8(g_src[i] + (size_t)(st) * (KC / 2));          \
+        }                                                                               \
+    }
+#define T12_STORE_STAGE(slot, buf)                                                                  \
+    {                                                                                               \
+        uint8_t* base_ = lds + (buf) * STAGE_BYTES;                                                 \
+        _Pragma("unroll") for (int i = 0; i < ACT_LD; i++)                                          \
+            *(uint4*)(base_ + a_dst[i]) = t12_pair_acts(ra[slot][i]);                               \
+        _Pragma("unroll") for (int i = 0; i < 2; i++) {                                             \
+            *(uint4*)(base_ + s_dst[i]) = rs[slot][i];                                              \
+            *(uint2*)(base_ + g_dst[i]) = rg[slot][i];                                              \
+        }                                                                                           \
+    }
 
     t12_f32x16 acc[FB][FM];
 #pragma unroll
@@ -160,16 +160,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    if (nstage > 0) {
-        load_stage(0);
-        store_stage(0);
-    }
-    __syncthreads();
-
-    for (int st = 0; st < nstage; st++) {
-        const int buf = st & 1;
-        if (st + 1 < nstage) load_stage(st + 1);          // global loads fly under the MFMAs
-
+    auto compute_stage = [&](int buf) {
         const uint8_t* base = lds + buf * STAGE_BYTES;
         const uint4* lact = (const uint4*)base;
         const uint4* lsm = (const uint4*)(base + ACT_UNITS * 16);
@@ -201,11 +192,66 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
                 }
             }
         }
-        if (st + 1 < nstage) store_stage(buf ^ 1);
-        __syncthreads();
+    };
+
+    // prologue: stages 0..D-1 in flight, stage 0 into LDS
+#pragma unroll
+    for (int d = 0; d < D; d++)
+        if (d < nstage) T12_LOAD_STAGE(d, d)
+    if (nstage > 0) T12_STORE_STAGE(0, 0)
+    __syncthreads();
+
+    int st = 0;
+    // steady state, unrolled by D so that ring slots are compile-time; no guards inside
+    for (; st + 2 * D <= nstage; st += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            T12_LOAD_STAGE(d, st + d + D)                    // slot d held stage st + d: already in LDS
+            compute_stage((st + d) & 1);
+            T12_STORE_STAGE((d + 1) % D, (st + d + 1) & 1)
+            __syncthreads();
+        }
+    }
+    // drain
+    for (; st < nstage; st += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            if (st + d < nstage) {
+                if (st + d + D < nstage) T12_LOAD_STAGE(d, st + d + D)
+                compute_stage((st + d) & 1);
+                if (st + d + 1 < nstage) T12_STORE_STAGE((d + 1) % D, (st + d + 1) & 1)
+                __syncthreads();
+            }
+        }
+    }
+#undef T12_LOAD_STAGE
+#undef T12_STORE_STAGE
+
+    // ---- escape corrections, by the K split that owns column 0 only: the streamed value of an
+    //      escape is its "wrong" decode, so acc[b, m] += (correct - wrong) * X[b, col]
+    if (blockIdx.z == 0 && sg.row_off) {
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            const int m = m0 + (wm * FM + j) * 32 + ln;
+            if (m < M) {
+                const int beg = sg.row_off[m], end = sg.row_off[m + 1];
+                for (int pp = beg; pp < end; pp++) {
+                    const float delta = t12_bf16_to_f32((uint16_t)sg.correct[pp]) -
+                                        t12_bf16_to_f32((uint16_t)sg.wrong[pp]);
+                    const uint16_t* xc = p.act + sg.cols[pp];
+#pragma unroll
+                    for (int i = 0; i < FB; i++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const int bb = b0 + (wb * FB + i) * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                            if (bb < B) acc[i][j][r] += delta * t12_bf16_to_f32(xc[(size_t)bb * p.act_stride]);
+                        }
+                }
+            }
+        }
     }
 
-    // ---- epilogue: accumulator register r of lane (ln, lh) is
+    // ---- store: accumulator register r of lane (ln, lh) is
     //      D[row = 8*(r/4) + 4*lh + r%4][col = ln]   (row = batch, col = m)
     float* dst;
     size_t ld;
@@ -233,41 +279,23 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
 }
 
 // ---------------------------------------------------------------------------
-// Epilogue kernel: out[b, m] = sum over K splits of the partials (fixed order)
-// + escape corrections.  One workgroup per (row block of 64 m, batch row b).
-// With ksplit == 1 only the corrections are added (rows without escapes are
-// left untouched).
+// K-split reduction: out[b, m] = sum over splits z of ws[z][b][m], in ascending z
+// (a fixed order: the result does not depend on which workgroup finished first).
+// Grid: (blocks of 256 workspace columns, B).
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void gemm_epilogue_kernel(const GemmParams p)
+__global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmParams p)
 {
-    const int tile = blockIdx.x;            // 64-row blocks; blk_start here counts 64-row blocks
-    const int s = find_segment(p, tile);
-    const T12Segment& sg = p.seg[s];
-    const int m = (tile - p.blk_start[s]) * 64 + threadIdx.x;
+    const int col = blockIdx.x * 256 + threadIdx.x;
     const int b = blockIdx.y;
-    if (m >= sg.M) return;
-    float v;
-    bool dirty = false;
-    if (p.ksplit > 1) {
-        v = 0.0f;
-        for (int z = 0; z < p.ksplit; z++)
-            v += p.ws[((size_t)z * p.B + b) * p.m_total + p.seg_row0[s] + m];
-        dirty = true;
-    } else {
-        v = 0.0f;
-    }
-    if (sg.row_off) {
-        const int beg = sg.row_off[m], end = sg.row_off[m + 1];
-        if (end > beg) {
-            if (!dirty) v = sg.out[(size_t)b * sg.out_stride + m];
-            const uint16_t* x = p.act + (size_t)b * p.act_stride;
-            for (int q = beg; q < end; q++)
-                v += (t12_bf16_to_f32((uint16_t)sg.correct[q]) - t12_bf16_to_f32((uint16_t)sg.wrong[q])) *
-                     t12_bf16_to_f32(x[sg.cols[q]]);
-            dirty = true;
-        }
-    }
-    if (dirty) sg.out[(size_t)b * sg.out_stride + m] = v;
+    if (col >= p.m_total) return;
+    int s = 0;
+#pragma unroll
+    for (int i = 1; i < T12_MAX_SEGMENTS; i++)
+        if (i < p.nseg && col >= p.seg_row0[i]) s = i;
+    float v = 0.0f;
+    for (int z = 0; z < p.ksplit; z++) v += p.ws[((size_t)z * p.B + b) * p.m_total + col];
+    const T12Segment& sg = p.seg[s];
+    sg.out[(size_t)b * sg.out_stride + (col - p.seg_row0[s])] = v;
 }
 
 // ---------------------------------------------------------------------------
@@ -381,7 +409,7 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
     p.act = (const uint16_t*)act_bf16;
     p.ws = nullptr;
     bool fast = (K % KC == 0) && (act_stride % 8 == 0) && ((uintptr_t)act_bf16 % 16 == 0);
-    int m_total = 0, any_patch = 0;
+    int m_total = 0;
     for (int i = 0; i < nseg; i++) {
         const T12Segment& g = segs[i];
         T12_REQUIRE(g.M >= 1 && g.sm && g.gr && g.out, "t12_gemm: segment %d has M < 1 or a null pointer", i);
@@ -389,7 +417,6 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
         T12_REQUIRE(g.base_exp >= -1 && g.base_exp <= 254, "t12_gemm: segment %d: base_exp %d out of range", i,
                     g.base_exp);
         if (g.base_exp < 0 || g.base_exp > 240) fast = false;
-        if (g.row_off) any_patch = 1;
         p.seg[i] = g;
         if (p.seg[i].out_stride == 0) p.seg[i].out_stride = out_stride;
         T12_REQUIRE(p.seg[i].out_stride >= g.M, "t12_gemm: out_stride %d < M %d of segment %d", p.seg[i].out_stride,
@@ -419,12 +446,15 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
         tiles += (segs[i].M + TM - 1) / TM;
     }
     p.blk_start[nseg] = tiles;
-    // K split: aim at >= 256 workgroups (one per CU) while every split keeps >= 8 stages
+    // K split: fill the chip.  A 256-row batch tile needs a whole CU (LDS, accumulators);
+    // smaller batch tiles fit 2-4 workgroups per CU.  Every split keeps >= 4 stages.
     const int btiles = (B + 255) / 256;
+    const int per_cu = B > 128 ? 1 : (B > 64 ? 2 : 4);
+    const int want = 256 * per_cu;
     int ks = 1;
     if (g_gemm_ksplit > 0) ks = g_gemm_ksplit;
     else
-        while (tiles * btiles * ks < 192 && K / (ks * 2) >= 8 * KC && ks < 16) ks *= 2;
+        while (tiles * btiles * ks * 4 < want * 3 && K / (ks * 2) >= 4 * KC && ks < 16) ks *= 2;
     int kslice = ((K / KC + ks - 1) / ks) * KC;
     ks = (K + kslice - 1) / kslice;
     p.ksplit = ks;
@@ -444,15 +474,9 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
     else rc = launch_mfma<2, 2, 4, 2>(p, tiles, st);
     if (rc) return rc;
 
-    if (ks > 1 || any_patch) {
-        int t64 = 0;
-        for (int i = 0; i < nseg; i++) {
-            p.blk_start[i] = t64;
-            t64 += (segs[i].M + 63) / 64;
-        }
-        p.blk_start[nseg] = t64;
-        hipLaunchKernelGGL(gemm_epilogue_kernel, dim3(t64, B), dim3(64), 0, st, p);
-        T12_CHECK_LAUNCH("t12_gemm(epilogue)");
+    if (ks > 1) {
+        hipLaunchKernelGGL(gemm_reduce_kernel, dim3((m_total + 255) / 256, B), dim3(256), 0, st, p);
+        T12_CHECK_LAUNCH("t12_gemm(reduce)");
     }
     return T12_OK;
 }

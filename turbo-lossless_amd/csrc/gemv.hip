@@ -100,7 +100,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
     const int M = sg.M;
     const int row0 = (blk - p.blk_start[s]) * (NW * R) + wave * R;
     const bool live = row0 < M;                // wave-uniform
-    const uint32_t be2 = ((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23);
+    const uint32_t be2 = t12_opaque(((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23));
     const bool patched = sg.row_off != nullptr;
 
     int ro = 0;                                // lane l <= R: row_off[row0 + l]

@@ -33,7 +33,8 @@ __device__ __forceinline__ uint16_t t12_decode_scalar(uint32_t sm, uint32_t g, i
 // ---------------------------------------------------------------------------
 // Packed decode of 8 consecutive weights.
 //   s0 = sm bytes 0..3, s1 = sm bytes 4..7, g = their eight nibbles (nibble i in
-//   bits 4i+3..4i), be2 = (base_exp << 7) | (base_exp << 23) with 0 <= base_exp <= 240.
+//   bits 4i+3..4i), be2 = (base_exp << 7) | (base_exp << 23) with 0 <= base_exp <= 240,
+//   passed through t12_opaque() once by the caller.
 // Result w[i] = bf16x2 { weight i (low half), weight i+4 (high half) }, i = 0..3.
 // Pairing i with i+4 puts both nibbles of a pair exactly 16 bits apart, so one
 // AND isolates both exponents offsets of a pair and one shift-add rebases them:
@@ -42,22 +43,22 @@ __device__ __forceinline__ uint16_t t12_decode_scalar(uint32_t sm, uint32_t g, i
 // Cost: per pair 1 v_perm_b32 + 1 v_and_or_b32 + 1 v_and_b32 (+1 shift for the
 // two right-shifted pairs) + 1 v_lshl_add_u32/v_add_u32.
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ uint32_t t12_and_or(uint32_t a, uint32_t mask_sgpr, uint32_t c)
+// An empty asm that makes a value opaque to the optimiser without emitting an
+// instruction.  Used to keep (g & mask) in the form that selects to
+// v_and_b32 + v_lshl_add_u32, and to keep the rebased-exponent constant in a
+// VGPR so that (m & keep) | be2 selects to one v_and_or_b32.  No real
+// instruction hides in inline asm: every VALU result that feeds an MFMA is
+// written by an instruction the compiler's hazard recogniser can see (a VALU
+// write inside an asm block followed directly by an MFMA reading it is a
+// hardware hazard the compiler does not pad).
+__device__ __forceinline__ uint32_t t12_opaque(uint32_t v)
 {
-    // (a & mask) | c in one VOP3; written as asm because gfx9 VOP3 takes no
-    // literal and the compiler then splits it into v_and + v_or.
-    uint32_t d;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask_sgpr), "v"(c));
-    return d;
-}
-__device__ __forceinline__ uint32_t t12_lshl_add(uint32_t a, uint32_t sh_const, uint32_t c)
-{
-    uint32_t d;
-    asm("v_lshl_add_u32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "n"(sh_const), "v"(c));
-    return d;
+    asm("" : "+v"(v));
+    return v;
 }
 
-__device__ __forceinline__ void t12_decode8(uint32_t s0, uint32_t s1, uint32_t g, uint32_t be2,
+// be2v must come from t12_opaque(be2) (a VGPR).
+__device__ __forceinline__ void t12_decode8(uint32_t s0, uint32_t s1, uint32_t g, uint32_t be2v,
                                             uint32_t w[4])
 {
     // v_perm_b32: selector bytes 0-3 pick from the 2nd operand, 4-7 from the 1st.
@@ -67,12 +68,12 @@ __device__ __forceinline__ void t12_decode8(uint32_t s0, uint32_t s1, uint32_t g
     const uint32_t m3 = __builtin_amdgcn_perm(s1, s0, 0x07070303u);
     // byte duplicated in both bytes of its half: keep sign (bit 15) + mantissa (bits 6..0)
     const uint32_t keep = 0x807F807Fu;
-    const uint32_t t0 = t12_and_or(m0, keep, be2);
-    const uint32_t t1 = t12_and_or(m1, keep, be2);
-    const uint32_t t2 = t12_and_or(m2, keep, be2);
-    const uint32_t t3 = t12_and_or(m3, keep, be2);
-    w[0] = t12_lshl_add(g & 0x000F000Fu, 7, t0);
-    w[1] = t12_lshl_add(g & 0x00F000F0u, 3, t1);
+    const uint32_t t0 = (m0 & keep) | be2v;
+    const uint32_t t1 = (m1 & keep) | be2v;
+    const uint32_t t2 = (m2 & keep) | be2v;
+    const uint32_t t3 = (m3 & keep) | be2v;
+    w[0] = (t12_opaque(g & 0x000F000Fu) << 7) + t0;
+    w[1] = (t12_opaque(g & 0x00F000F0u) << 3) + t1;
     w[2] = ((g >> 1) & 0x07800780u) + t2;
     w[3] = ((g >> 5) & 0x07800780u) + t3;
 }
