@@ -25,8 +25,10 @@
 //   * Few row tiles (small M) are split along K across workgroups; the partial
 //     sums go to a workspace and a second kernel adds them in a fixed order
 //     (deterministic) together with the escape corrections.
-//   * Escapes: the streamed value of a group-0 weight is the "wrong" value; the
-//     epilogue kernel adds (correct - wrong) * X[b, col] for every batch row.
+//   * Escapes are EXACT and cost no extra pass: the (column, exact bf16) pairs of
+//     the workgroup's 128 rows -- one contiguous slice of the CSR list -- are
+//     staged in LDS once; every lane walks its own row's slice in step with the
+//     K loop and overwrites the decoded half-word in its MFMA operand register.
 //
 // Fast path requirements: K % 64 == 0, 0 <= base_exp <= 240, 16-byte aligned
 // activation rows.  Everything else goes to the general kernel below.
@@ -38,6 +40,9 @@ namespace {
 
 constexpr int KC = 64;          // K columns staged per pipeline stage
 constexpr int TM = 128;         // weight rows per workgroup
+constexpr int PCAP = 4096;      // escape entries a workgroup can stage in LDS
+constexpr int PATCH_BYTES = PCAP * 4 + (TM + 1) * 4 + 12;
+constexpr int NO_ESCAPE = 0x7FFFFFFF;
 
 struct GemmParams {
     T12Segment seg[T12_MAX_SEGMENTS];
@@ -160,38 +165,100 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    auto compute_stage = [&](int buf) {
+    // ---- escape list of this workgroup's rows -> LDS.  The rows are consecutive, so
+    //      their entries are one contiguous slice [e0, e1) of cols[] / correct[].
+    //      esc_mode: 0 none, 1 staged (exact, in registers), 2 too many for LDS
+    //      (or K > 65536): streamed wrong values + correction in the epilogue.
+    uint32_t* lpat = (uint32_t*)(lds + 2 * STAGE_BYTES);       // col | correct << 16
+    int* lrow = (int*)(lpat + PCAP);                           // [TM + 1] offsets into lpat
+    int esc_mode = 0;
+    if (sg.row_off) {
+        const int e0 = sg.row_off[min(m0, M)], e1 = sg.row_off[min(m0 + TM, M)];
+        esc_mode = (e1 - e0 <= PCAP && K <= 65536) ? 1 : 2;
+        if (esc_mode == 1) {
+            for (int t = tid; t < e1 - e0; t += 256)
+                lpat[t] = (uint32_t)sg.cols[e0 + t] | ((uint32_t)(uint16_t)sg.correct[e0 + t] << 16);
+            for (int t = tid; t <= TM; t += 256) lrow[t] = sg.row_off[min(m0 + t, M)] - e0;
+        }
+    }
+    // per lane: cursor into its rows' slices (FM rows), next escape column and its exact value
+    int pp[FM], pe[FM], nc[FM];
+    uint32_t cv[FM];
+#pragma unroll
+    for (int j = 0; j < FM; j++) { pp[j] = pe[j] = 0; nc[j] = NO_ESCAPE; cv[j] = 0; }
+
+    // One stage = 64 columns = 4 MFMA k-steps t = 0..3 (block q = t / 2, step ks = t % 2).
+    // Fragment loads run one k-step ahead of the MFMAs that use them, and the decode of
+    // block q = 1 is placed under the MFMAs of block q = 0.
+    auto load_w = [&](const uint4* lsm, const uint2* lgr, int q, uint4 (&S)[FM], uint2 (&G)[FM]) {
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            const int row = (wm * FM + j) * 32 + ln;
+            S[j] = lsm[(2 * q + lh) * TM + row];
+            G[j] = lgr[(2 * q + lh) * TM + row];
+        }
+    };
+    auto decode_w = [&](const uint4 (&S)[FM], const uint2 (&G)[FM], int kq, uint32_t (&wf)[FM][2][4]) {
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            t12_decode8(S[j].x, S[j].y, G[j].x, be2, wf[j][0]);
+            t12_decode8(S[j].z, S[j].w, G[j].y, be2, wf[j][1]);
+            // exact escapes: columns [kq, kq + 32) of this row; this lane owns the 16 of its half
+            while (nc[j] < kq + 32) {
+                const int e = nc[j] - kq;
+                if ((e >> 4) == lh) {
+                    const int i8 = e & 7, kst = (e >> 3) & 1;
+                    const uint32_t keep = (i8 >> 2) ? 0x0000FFFFu : 0xFFFF0000u;
+                    const uint32_t ins = (i8 >> 2) ? (cv[j] << 16) : cv[j];
+#pragma unroll
+                    for (int a = 0; a < 2; a++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            if (a == kst && r == (i8 & 3)) wf[j][a][r] = (wf[j][a][r] & keep) | ins;
+                }
+                pp[j]++;
+                const uint32_t ent = pp[j] < pe[j] ? lpat[pp[j]] : (uint32_t)NO_ESCAPE;
+                nc[j] = pp[j] < pe[j] ? (int)(ent & 0xFFFFu) : NO_ESCAPE;
+                cv[j] = ent >> 16;
+            }
+        }
+    };
+    auto load_a = [&](const uint4* lact, int t, uint4 (&A)[FB]) {
+#pragma unroll
+        for (int i = 0; i < FB; i++) A[i] = lact[(4 * (t >> 1) + 2 * lh + (t & 1)) * TB + (wb * FB + i) * 32 + ln];
+    };
+    auto mma = [&](const uint4 (&A)[FB], const uint32_t (&wf)[FM][2][4], int ks) {
+#pragma unroll
+        for (int i = 0; i < FB; i++) {
+            const t12_bf16x8 av = __builtin_bit_cast(t12_bf16x8, A[i]);
+#pragma unroll
+            for (int j = 0; j < FM; j++) {
+                const uint4 Wv = make_uint4(wf[j][ks][0], wf[j][ks][1], wf[j][ks][2], wf[j][ks][3]);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(t12_bf16x8, Wv),
+                                                                    acc[i][j], 0, 0, 0);
+            }
+        }
+    };
+    auto compute_stage = [&](int buf, int kabs) {
         const uint8_t* base = lds + buf * STAGE_BYTES;
         const uint4* lact = (const uint4*)base;
         const uint4* lsm = (const uint4*)(base + ACT_UNITS * 16);
         const uint2* lgr = (const uint2*)(base + ACT_UNITS * 16 + TM * 64);
-#pragma unroll
-        for (int q = 0; q < 2; q++) {
-            uint32_t wf[FM][2][4];
-#pragma unroll
-            for (int j = 0; j < FM; j++) {
-                const int row = (wm * FM + j) * 32 + ln;
-                const uint4 S = lsm[(2 * q + lh) * TM + row];
-                const uint2 G = lgr[(2 * q + lh) * TM + row];
-                t12_decode8(S.x, S.y, G.x, be2, wf[j][0]);
-                t12_decode8(S.z, S.w, G.y, be2, wf[j][1]);
-            }
-#pragma unroll
-            for (int ks = 0; ks < 2; ks++) {
-#pragma unroll
-                for (int i = 0; i < FB; i++) {
-                    const int brow = (wb * FB + i) * 32 + ln;
-                    const uint4 A = lact[(4 * q + 2 * lh + ks) * TB + brow];
-                    const t12_bf16x8 av = __builtin_bit_cast(t12_bf16x8, A);
-#pragma unroll
-                    for (int j = 0; j < FM; j++) {
-                        const uint4 Wv = make_uint4(wf[j][ks][0], wf[j][ks][1], wf[j][ks][2], wf[j][ks][3]);
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            av, __builtin_bit_cast(t12_bf16x8, Wv), acc[i][j], 0, 0, 0);
-                    }
-                }
-            }
-        }
+        uint4 S0[FM], S1[FM], A0[FB], A1[FB];
+        uint2 G0[FM], G1[FM];
+        uint32_t w0[FM][2][4], w1[FM][2][4];
+        load_w(lsm, lgr, 0, S0, G0);
+        load_a(lact, 0, A0);
+        load_w(lsm, lgr, 1, S1, G1);
+        decode_w(S0, G0, kabs, w0);
+        load_a(lact, 1, A1);
+        mma(A0, w0, 0);                 // t = 0
+        decode_w(S1, G1, kabs + 32, w1);
+        load_a(lact, 2, A0);
+        mma(A1, w0, 1);                 // t = 1
+        load_a(lact, 3, A1);
+        mma(A0, w1, 0);                 // t = 2
+        mma(A1, w1, 1);                 // t = 3
     };
 
     // prologue: stages 0..D-1 in flight, stage 0 into LDS
@@ -200,6 +267,20 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
         if (d < nstage) T12_LOAD_STAGE(d, d)
     if (nstage > 0) T12_STORE_STAGE(0, 0)
     __syncthreads();
+    if (esc_mode == 1) {
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            const int r = (wm * FM + j) * 32 + ln;
+            pp[j] = lrow[r];
+            pe[j] = lrow[r + 1];
+            while (pp[j] < pe[j] && (int)(lpat[pp[j]] & 0xFFFFu) < k_begin) pp[j]++;   // K split: skip earlier columns
+            if (pp[j] < pe[j]) {
+                const uint32_t ent = lpat[pp[j]];
+                nc[j] = (int)(ent & 0xFFFFu);
+                cv[j] = ent >> 16;
+            }
+        }
+    }
 
     int st = 0;
     // steady state, unrolled by D so that ring slots are compile-time; no guards inside
@@ -207,7 +288,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
 #pragma unroll
         for (int d = 0; d < D; d++) {
             T12_LOAD_STAGE(d, st + d + D)                    // slot d held stage st + d: already in LDS
-            compute_stage((st + d) & 1);
+            compute_stage((st + d) & 1, k_begin + (st + d) * KC);
             T12_STORE_STAGE((d + 1) % D, (st + d + 1) & 1)
             __syncthreads();
         }
@@ -218,7 +299,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
         for (int d = 0; d < D; d++) {
             if (st + d < nstage) {
                 if (st + d + D < nstage) T12_LOAD_STAGE(d, st + d + D)
-                compute_stage((st + d) & 1);
+                compute_stage((st + d) & 1, k_begin + (st + d) * KC);
                 if (st + d + 1 < nstage) T12_STORE_STAGE((d + 1) % D, (st + d + 1) & 1)
                 __syncthreads();
             }
@@ -227,9 +308,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
 #undef T12_LOAD_STAGE
 #undef T12_STORE_STAGE
 
-    // ---- escape corrections, by the K split that owns column 0 only: the streamed value of an
-    //      escape is its "wrong" decode, so acc[b, m] += (correct - wrong) * X[b, col]
-    if (blockIdx.z == 0 && sg.row_off) {
+    // ---- overflow path only (more escapes than the LDS list holds): the streamed value of an
+    //      escape was its "wrong" decode, so acc[b, m] += (correct - wrong) * X[b, col], added by
+    //      the K split that owns column 0
+    if (blockIdx.z == 0 && esc_mode == 2) {
 #pragma unroll
         for (int j = 0; j < FM; j++) {
             const int m = m0 + (wm * FM + j) * 32 + ln;
@@ -370,14 +452,15 @@ int launch_mfma(GemmParams& p, int tiles, hipStream_t st)
     auto kfn = gemm_mfma_kernel<WB, WM, FB, FM>;
     static bool attr_set = false;
     if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE_BYTES) !=
+        if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                2 * STAGE_BYTES + PATCH_BYTES) !=
             hipSuccess) {
             t12_set_error("t12_gemm: cannot reserve %d bytes of LDS", 2 * STAGE_BYTES);
             return T12_ELAUNCH;
         }
         attr_set = true;
     }
-    hipLaunchKernelGGL(kfn, grid, dim3(256), 2 * STAGE_BYTES, st, p);
+    hipLaunchKernelGGL(kfn, grid, dim3(256), 2 * STAGE_BYTES + PATCH_BYTES, st, p);
     T12_CHECK_LAUNCH("t12_gemm");
     return T12_OK;
 }
