@@ -78,6 +78,13 @@ int t12_tune_gemv(int variant);
  * array (it travels as a kernel argument; no device copy is made). */
 int t12_gemv(const T12Segment* segs, int nseg, const void* act_bf16, int K, void* stream);
 
+/* SwiGLU front half in one launch: out_bf16[m] = bf16( silu(gate[m,:].x) * (up[m,:].x) ).
+ * Replaces launch_split12_v2_dual_async (decompress_v2.hip:549) + its patch launch +
+ * launch_silu_mul_bf16_batch (engine/kernels.hip:480); bit-identical to that sequence.
+ * Requires gate->M == up->M, K % 16 == 0, base_exp in 0..240. */
+int t12_gemv_swiglu(const T12Segment* gate, const T12Segment* up, const void* act_bf16, int K,
+                    void* out_bf16, void* stream);
+
 /* ---- (a') small batch, 1 <= B <= 8 -----------------------------------------
  * Same contract as t12_gemm, restricted to the batch sizes of the reference's
  * launch_split12_batch4_async / _batch8_async (decompress_v2.hip:860,877), with

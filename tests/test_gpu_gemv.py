@@ -234,3 +234,29 @@ def test_gemv_batch_entry_point(t12, oracle, synth):
         torch.cuda.synchronize()
         assert rel_err(out.cpu().numpy(), oracle.gemm(p, X)) < TOL
     assert t12.lib.t12_gemv_batch(segs, 1, Xd.data_ptr(), K, M, K, 9, None) == -1
+
+
+@pytest.mark.parametrize("M,K", [(14336, 4096), (520, 2048), (77, 1040), (9, 16)])
+def test_gemv_swiglu_fused_is_bit_identical_to_unfused(t12, oracle, synth, M, K):
+    """t12_gemv_swiglu == t12_gemv(gate|up) followed by launch_silu_mul_bf16_batch, bit for bit,
+    and both match the oracle's closed form."""
+    pg = oracle.pack(synth.weights_llm(M, K, seed=81, sigma=0.05, p_outlier=2e-3))
+    pu = oracle.pack(synth.weights_llm(M, K, seed=82, sigma=0.2, p_outlier=2e-3))
+    x = synth.activations(1, K, seed=83)[0]
+    dg, du = (t12.DeviceTensor12.from_packed(p, dev()) for p in (pg, pu))
+    xd = to_dev_bits(x)
+    og, ou = t12.gemv([dg, du], xd)
+    unfused = torch.zeros(M, dtype=torch.int16, device=dev())
+    st = t12.current_stream()
+    t12.lib.launch_silu_mul_bf16_batch(og.data_ptr(), ou.data_ptr(), unfused.data_ptr(), M, 1, st)
+    fused = torch.zeros(M, dtype=torch.int16, device=dev())
+    sg, su = dg.segment(None), du.segment(None)
+    import ctypes
+    t12.check(t12.lib.t12_gemv_swiglu(ctypes.byref(sg), ctypes.byref(su), xd.data_ptr(), K, fused.data_ptr(), st))
+    torch.cuda.synchronize()
+    assert torch.equal(fused, unfused)
+    ref = oracle.silu_mul_bf16(oracle.gemv(pg, x), oracle.gemv(pu, x))
+    got = fused.cpu().numpy().view(np.uint16)
+    gf, rf = oracle.bf16_bits_to_f32(got), oracle.bf16_bits_to_f32(ref)
+    assert np.abs(gf - rf).max() <= 2e-2 * np.abs(rf).max()
+    assert (got == ref).mean() > 0.97

@@ -130,9 +130,16 @@ def test_rope_and_store_batch_launchers(t12, oracle):
     assert torch.equal(ck, ck2) and torch.equal(cv, cv2) and torch.equal(sk, sk2) and torch.equal(q2, qd)
 
 
+@pytest.fixture(params=[1, 0], ids=["fast", "general"])
+def attn_mode(request, t12):
+    t12.lib.t12_tune_attention(request.param)
+    yield request.param
+    t12.lib.t12_tune_attention(1)
+
+
 @pytest.mark.parametrize("nh,nkv,hd,seq", [(32, 8, 128, 1), (32, 8, 128, 300), (32, 8, 128, 1500), (4, 4, 64, 77),
-                                            (16, 1, 32, 513)])
-def test_attention_b1_both_names(t12, oracle, nh, nkv, hd, seq):
+                                            (16, 1, 32, 513), (8, 8, 128, 130), (16, 2, 128, 65), (16, 4, 64, 257)])
+def test_attention_b1_both_names(t12, oracle, attn_mode, nh, nkv, hd, seq):
     rng = np.random.default_rng(seq)
     max_seq = seq + 3
     q = rng.standard_normal(nh * hd).astype(np.float32)
@@ -152,7 +159,7 @@ def test_attention_b1_both_names(t12, oracle, nh, nkv, hd, seq):
         assert np.abs(got - want).max() <= 2e-2 * np.abs(want).max()   # bf16 output: 2^-8 relative steps
 
 
-def test_attention_batch_shared_and_strided_cache(t12, oracle):
+def test_attention_batch_shared_and_strided_cache(t12, oracle, attn_mode):
     rng = np.random.default_rng(9)
     nh, nkv, hd, B, max_seq = 8, 2, 64, 3, 50
     positions = [4, 30, 49]

@@ -51,6 +51,8 @@ _SIGS = {
     "t12_synth_normal_bf16": (_i, [_vp, C.c_size_t, C.c_uint64, C.c_float, C.c_float, C.c_float, _vp]),
     "t12_fill_f32": (_i, [_vp, C.c_size_t, C.c_float, _vp]),
     # glue launchers (reference names; void return)
+    "t12_tune_attention": (_i, [_i]),
+    "t12_debug_gemm": (_i, [_i]),
     "launch_rope_init": (None, [_i, C.c_float]),
     "launch_embed_lookup": (None, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "launch_rms_norm_bf16_batch": (None, [_vp, _vp, _vp, _i, C.c_float, _i, _vp]),
@@ -84,6 +86,7 @@ _SIGS = {
     "t12_engine_generate": (_i, [_vp, C.POINTER(C.c_int), _i, _i, C.POINTER(C.c_int)]),
     "t12_engine_sync": (_i, [_vp]),
     "t12_engine_weight": (_i, [_vp, _i, _i, C.POINTER(Segment), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "t12_gemv_swiglu": (_i, [C.POINTER(Segment), C.POINTER(Segment), _vp, _i, _vp, _vp]),
     "t12_gemv_batch": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
     "launch_split12_batch4_async": (_i, [_vp] * 2 + [_i] + [_vp] * 4 + [_vp] * 3 + [_vp] * 4 + [_i, _i, _vp]),
     "launch_split12_batch8_async": (_i, [_vp] * 2 + [_i] + [_vp] * 8 + [_vp] * 3 + [_vp] * 8 + [_i, _i, _vp]),

@@ -209,8 +209,17 @@ void forward(InferenceState* state, const int* token_ids)
 
         S.gateup[0] = seg_of(L.w_gate, state->ffn_gate, n_ff);
         S.gateup[1] = seg_of(L.w_up, state->ffn_up, n_ff);
-        run_linear(S.gateup, 2, bf16_a, n, B, st);
-        launch_silu_mul_bf16_batch(state->ffn_gate, state->ffn_up, bf16_b, n_ff, B, st);
+        const bool fuse_swiglu = B == 1 && n % 16 == 0 && L.w_gate.base_exp >= 0 && L.w_gate.base_exp <= 240 &&
+                                 L.w_up.base_exp >= 0 && L.w_up.base_exp <= 240;
+        if (fuse_swiglu) {      // gate|up decode-GEMV with the SiLU*mul epilogue: one launch, no fp32 round trip
+            if (t12_gemv_swiglu(&S.gateup[0], &S.gateup[1], bf16_a, n, bf16_b, st) != T12_OK) {
+                fprintf(stderr, "ERROR: fused gate|up launch failed: %s\n", t12_last_error());
+                exit(1);
+            }
+        } else {
+            run_linear(S.gateup, 2, bf16_a, n, B, st);
+            launch_silu_mul_bf16_batch(state->ffn_gate, state->ffn_up, bf16_b, n_ff, B, st);
+        }
 
         S.down[0] = seg_of(L.w_down, cur, n);
         run_linear(S.down, 1, bf16_b, n_ff, B, st);

@@ -77,7 +77,9 @@ __device__ __forceinline__ int find_segment(const GemmParams& p, int tile)
 // One 32-column block q of a stage feeds two MFMA k-steps s = 0, 1; MFMA slot
 // (half h of the wave, element j) stands for column 32q + 16h + 8s + j.
 // ---------------------------------------------------------------------------
-template <int WB, int WM, int FB, int FM>
+// DBG (benchmark probes, 0 in production): bit 0 skips the MFMAs, bit 1 skips the global->LDS
+// staging inside the loop, bit 2 skips the barrier per stage.
+template <int WB, int WM, int FB, int FM, int DBG = 0>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
 {
     constexpr int TB = WB * FB * 32;                  // batch rows per workgroup
@@ -234,8 +236,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
 #pragma unroll
             for (int j = 0; j < FM; j++) {
                 const uint4 Wv = make_uint4(wf[j][ks][0], wf[j][ks][1], wf[j][ks][2], wf[j][ks][3]);
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(t12_bf16x8, Wv),
-                                                                    acc[i][j], 0, 0, 0);
+                if (DBG & 1) acc[i][j][0] += __builtin_bit_cast(float, A[i].x ^ Wv.x ^ Wv.y ^ Wv.z ^ Wv.w);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(t12_bf16x8, Wv),
+                                                                        acc[i][j], 0, 0, 0);
             }
         }
     };
@@ -287,10 +291,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
     for (; st + 2 * D <= nstage; st += D) {
 #pragma unroll
         for (int d = 0; d < D; d++) {
-            T12_LOAD_STAGE(d, st + d + D)                    // slot d held stage st + d: already in LDS
+            if (!(DBG & 2)) T12_LOAD_STAGE(d, st + d + D)    // slot d held stage st + d: already in LDS
             compute_stage((st + d) & 1, k_begin + (st + d) * KC);
-            T12_STORE_STAGE((d + 1) % D, (st + d + 1) & 1)
-            __syncthreads();
+            if (!(DBG & 2)) T12_STORE_STAGE((d + 1) % D, (st + d + 1) & 1)
+            if (!(DBG & 4)) __syncthreads();
         }
     }
     // drain
@@ -443,13 +447,15 @@ float* workspace(size_t bytes)
 
 int g_gemm_ksplit = 0;   // 0 = choose by shape
 
-template <int WB, int WM, int FB, int FM>
+int g_gemm_dbg = 0;
+
+template <int WB, int WM, int FB, int FM, int DBG = 0>
 int launch_mfma(GemmParams& p, int tiles, hipStream_t st)
 {
     constexpr int TB = WB * FB * 32;
     constexpr int STAGE_BYTES = TB * 8 * 16 + TM * 64 + TM * 32;
     const dim3 grid(tiles, (p.B + TB - 1) / TB, p.ksplit);
-    auto kfn = gemm_mfma_kernel<WB, WM, FB, FM>;
+    auto kfn = gemm_mfma_kernel<WB, WM, FB, FM, DBG>;
     static bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -473,6 +479,13 @@ extern "C" {
 int t12_tune_gemm(int ksplit)
 {
     g_gemm_ksplit = ksplit;
+    return T12_OK;
+}
+
+// Benchmark probe: runs the B > 128 kernel with parts of its loop removed (wrong results).
+int t12_debug_gemm(int mask)
+{
+    g_gemm_dbg = mask;
     return T12_OK;
 }
 
@@ -554,6 +567,10 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
     if (B <= 32) rc = launch_mfma<1, 4, 1, 1>(p, tiles, st);
     else if (B <= 64) rc = launch_mfma<1, 4, 2, 1>(p, tiles, st);
     else if (B <= 128) rc = launch_mfma<1, 4, 4, 1>(p, tiles, st);
+    else if (g_gemm_dbg == 1) rc = launch_mfma<2, 2, 4, 2, 1>(p, tiles, st);
+    else if (g_gemm_dbg == 2) rc = launch_mfma<2, 2, 4, 2, 2>(p, tiles, st);
+    else if (g_gemm_dbg == 3) rc = launch_mfma<2, 2, 4, 2, 3>(p, tiles, st);
+    else if (g_gemm_dbg == 6) rc = launch_mfma<2, 2, 4, 2, 6>(p, tiles, st);
     else rc = launch_mfma<2, 2, 4, 2>(p, tiles, st);
     if (rc) return rc;
 

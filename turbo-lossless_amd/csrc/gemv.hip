@@ -27,6 +27,7 @@ struct GemvParams {
     int nseg;
     int K;
     const uint16_t* act;
+    uint16_t* out_bf16;                    // SwiGLU mode only
 };
 
 __device__ __forceinline__ int find_segment(const GemvParams& p, int blk)
@@ -85,9 +86,14 @@ __device__ __forceinline__ float lds_act_at(const uint4* lds_act, int k)
     return t12_bf16_to_f32(h[(i & 3) * 2 + (i >> 2)]);
 }
 
-template <int NW, int R, int D, int MINB>
+// SWIGLU (R must be 2): row 0 of a wave is row m of segment 0 (gate), row 1 is row m of
+// segment 1 (up); the wave writes bf16( silu(gate.x) * (up.x) ) to p.out_bf16[m] instead of two
+// fp32 sums -- the reference's split12_matvec_v2_dual (decompress_v2.hip:387-523) with its
+// silu_mul_bf16 kernel (engine/kernels.hip:447-459) folded into the epilogue.
+template <int NW, int R, int D, int MINB, bool SWIGLU = false>
 __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvParams p)
 {
+    static_assert(!SWIGLU || R == 2, "the SwiGLU epilogue pairs exactly two rows");
     extern __shared__ uint4 lds_act[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K = p.K;
@@ -95,24 +101,33 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
     const int nchunk = (K + 1023) >> 10;
 
     const int blk = blockIdx.x;
-    const int s = find_segment(p, blk);
+    const int s = SWIGLU ? 0 : find_segment(p, blk);
     const T12Segment& sg = p.seg[s];
     const int M = sg.M;
-    const int row0 = (blk - p.blk_start[s]) * (NW * R) + wave * R;
+    // row r of this wave: tensor SEG(r), matrix row ROW(r)
+#define SEG(r) (SWIGLU ? p.seg[r] : sg)
+#define ROW(r) (SWIGLU ? row0 : row0 + (r))
+    const int row0 = SWIGLU ? blk * NW + wave : (blk - p.blk_start[s]) * (NW * R) + wave * R;
     const bool live = row0 < M;                // wave-uniform
-    const uint32_t be2 = t12_opaque(((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23));
-    const bool patched = sg.row_off != nullptr;
+    uint32_t be2r[R];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+        be2r[r] = t12_opaque(((uint32_t)SEG(r).base_exp << 7) | ((uint32_t)SEG(r).base_exp << 23));
 
-    int ro = 0;                                // lane l <= R: row_off[row0 + l]
-    if (patched && live && lane <= R) ro = sg.row_off[min(row0 + lane, M)];
+    // CSR row pointers: lane 2r holds the begin and lane 2r+1 the end of row r's escape slice
+    int ro = 0;
+    if (live && lane < 2 * R) {
+        const T12Segment& g = SEG(lane >> 1);
+        if (g.row_off) ro = g.row_off[min(ROW(lane >> 1) + (lane & 1), M)];
+    }
 
     const uint8_t* smp[R];
     const uint8_t* grp[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        const size_t e = (size_t)min(row0 + r, M - 1) * K;      // clamp: loads stay in bounds
-        smp[r] = sg.sm + e + lane * 16;
-        grp[r] = sg.gr + (e >> 1) + lane * 8;
+        const size_t e = (size_t)min(ROW(r), M - 1) * K;        // clamp: loads stay in bounds
+        smp[r] = SEG(r).sm + e + lane * 16;
+        grp[r] = SEG(r).gr + (e >> 1) + lane * 8;
     }
 
     constexpr int DR = D > 0 ? D : 1;          // the K tail borrows slot 0
@@ -128,8 +143,8 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
         const uint4 a0 = lds_act[(tile) * 128 + lane];                                                 \
         const uint4 a1 = lds_act[(tile) * 128 + 64 + lane];                                            \
         _Pragma("unroll") for (int r = 0; r < R; r++) {                                                \
-            acc[r] = t12_decode_dot8(ringS[slot][r].x, ringS[slot][r].y, ringG[slot][r].x, be2, a0, acc[r]); \
-            acc[r] = t12_decode_dot8(ringS[slot][r].z, ringS[slot][r].w, ringG[slot][r].y, be2, a1, acc[r]); \
+            acc[r] = t12_decode_dot8(ringS[slot][r].x, ringS[slot][r].y, ringG[slot][r].x, be2r[r], a0, acc[r]); \
+            acc[r] = t12_decode_dot8(ringS[slot][r].z, ringS[slot][r].w, ringG[slot][r].y, be2r[r], a1, acc[r]); \
         }                                                                                              \
     }
 
@@ -155,15 +170,15 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
     int pend[R], pnext[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        const int beg = __builtin_amdgcn_readlane(ro, r), end = __builtin_amdgcn_readlane(ro, r + 1);
+        const int beg = __builtin_amdgcn_readlane(ro, 2 * r), end = __builtin_amdgcn_readlane(ro, 2 * r + 1);
         pend[r] = end;
         pnext[r] = beg + T12_WAVE;
         pcol[r] = -1;
         pdelta[r] = 0.0f;
-        if (beg + lane < end) {
-            pcol[r] = sg.cols[beg + lane];
-            pdelta[r] = t12_bf16_to_f32((uint16_t)sg.correct[beg + lane]) -
-                        t12_bf16_to_f32((uint16_t)sg.wrong[beg + lane]);
+        if (beg + lane < end) {                          // end > beg only when the tensor has a list
+            pcol[r] = SEG(r).cols[beg + lane];
+            pdelta[r] = t12_bf16_to_f32((uint16_t)SEG(r).correct[beg + lane]) -
+                        t12_bf16_to_f32((uint16_t)SEG(r).wrong[beg + lane]);
         }
     }
 
@@ -198,18 +213,26 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
 #undef T12_FETCH
 #undef T12_CONSUME
 
+    float tot[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        if (row0 + r < M) {                              // wave-uniform
+        tot[r] = 0.0f;
+        if (ROW(r) < M) {                                // wave-uniform
             float v = acc[r];
             if (pcol[r] >= 0) v += pdelta[r] * lds_act_at(lds_act, pcol[r]);
             for (int q = pnext[r] + lane; q < pend[r]; q += T12_WAVE)     // rows with > 64 escapes
-                v += (t12_bf16_to_f32((uint16_t)sg.correct[q]) - t12_bf16_to_f32((uint16_t)sg.wrong[q])) *
-                     lds_act_at(lds_act, sg.cols[q]);
-            v = t12_wave_sum_lane63(v);
-            if (lane == 63) sg.out[row0 + r] = v;
+                v += (t12_bf16_to_f32((uint16_t)SEG(r).correct[q]) - t12_bf16_to_f32((uint16_t)SEG(r).wrong[q])) *
+                     lds_act_at(lds_act, SEG(r).cols[q]);
+            tot[r] = t12_wave_sum_lane63(v);
+            if (!SWIGLU && lane == 63) sg.out[row0 + r] = tot[r];
         }
     }
+    if (SWIGLU && lane == 63) {
+        const float g = tot[0];
+        p.out_bf16[row0] = t12_f32_to_bf16(g / (1.0f + expf(-g)) * tot[R - 1]);
+    }
+#undef SEG
+#undef ROW
 }
 
 // ---------------------------------------------------------------------------
@@ -272,6 +295,21 @@ int launch_stream(GemvParams& p, const T12Segment* segs, int nseg, hipStream_t s
     return T12_OK;
 }
 
+int launch_swiglu(GemvParams& p, hipStream_t st)
+{
+    const int NW = 8;
+    const int total = (p.seg[0].M + NW - 1) / NW;
+    p.blk_start[0] = 0;
+    p.blk_start[1] = p.blk_start[2] = total;
+    const size_t lds = (size_t)((p.K + 1023) / 1024) * 2048;
+    const int T = p.K / 1024;
+    if (T >= 2) hipLaunchKernelGGL((gemv_stream_kernel<8, 2, 2, 1, true>), dim3(total), dim3(NW * 64), lds, st, p);
+    else if (T == 1) hipLaunchKernelGGL((gemv_stream_kernel<8, 2, 1, 1, true>), dim3(total), dim3(NW * 64), lds, st, p);
+    else hipLaunchKernelGGL((gemv_stream_kernel<8, 2, 0, 1, true>), dim3(total), dim3(NW * 64), lds, st, p);
+    T12_CHECK_LAUNCH("t12_gemv_swiglu");
+    return T12_OK;
+}
+
 int validate(const T12Segment* segs, int nseg, const void* act, int K, bool need_out)
 {
     T12_REQUIRE(segs && nseg >= 1 && nseg <= T12_MAX_SEGMENTS, "nseg must be 1..%d (got %d)", T12_MAX_SEGMENTS, nseg);
@@ -308,6 +346,7 @@ int t12_gemv(const T12Segment* segs, int nseg, const void* act_bf16, int K, void
     p.nseg = nseg;
     p.K = K;
     p.act = (const uint16_t*)act_bf16;
+    p.out_bf16 = nullptr;
     bool fast = (K % 16 == 0) && ((K + 1023) / 1024 * 2048 <= 160 * 1024);
     for (int i = 0; i < nseg; i++) {
         p.seg[i] = segs[i];
@@ -352,6 +391,28 @@ int t12_gemv(const T12Segment* segs, int nseg, const void* act_bf16, int K, void
             t12_set_error("t12_gemv: unknown kernel variant %d", v);
             return T12_EINVAL;
     }
+}
+
+// out_bf16[m] = bf16( silu(gate[m,:].x) * (up[m,:].x) ), escapes exact, one launch.
+int t12_gemv_swiglu(const T12Segment* gate, const T12Segment* up, const void* act_bf16, int K, void* out_bf16,
+                    void* stream)
+{
+    T12_REQUIRE(gate && up && out_bf16, "t12_gemv_swiglu: null operand");
+    T12Segment two[2] = {*gate, *up};
+    int rc = validate(two, 2, act_bf16, K, false);
+    if (rc) return rc;
+    T12_REQUIRE(gate->M == up->M, "t12_gemv_swiglu: gate has %d rows, up has %d", gate->M, up->M);
+    T12_REQUIRE(K % 16 == 0 && (K + 1023) / 1024 * 2048 <= 160 * 1024, "t12_gemv_swiglu: K %d must be a multiple of 16", K);
+    T12_REQUIRE(gate->base_exp >= 0 && gate->base_exp <= 240 && up->base_exp >= 0 && up->base_exp <= 240,
+                "t12_gemv_swiglu: base_exp outside 0..240 (use t12_gemv + launch_silu_mul_bf16_batch)");
+    GemvParams p;
+    p.seg[0] = two[0];
+    p.seg[1] = two[1];
+    p.nseg = 2;
+    p.K = K;
+    p.act = (const uint16_t*)act_bf16;
+    p.out_bf16 = (uint16_t*)out_bf16;
+    return launch_swiglu(p, (hipStream_t)stream);
 }
 
 // ---- reference-named launchers ---------------------------------------------

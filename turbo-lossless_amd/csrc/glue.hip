@@ -325,6 +325,157 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
     }
 }
 
+// ---- fast decode attention for the common shapes (head_dim 64 / 128, GQA ratio 1/2/4/8) ----
+// Same function as attn_decode_kernel; compile-time shapes let every loop unroll:
+//   phase 1  lane = position: the K row is fetched with HD/16 128-bit loads issued together,
+//            then dotted with the RATIO query vectors broadcast from LDS;
+//   phase 2  one wave per query head: tile max, exp, sum with wave reductions only
+//            (running max / sum are wave-uniform registers);
+//   phase 3  the same wave: P.V with 128-bit V loads -- 8 (HD=128) or 4 (HD=64) lanes span one
+//            position, so one load instruction covers 8 / 16 positions; each lane keeps 16
+//            output dims for its position class, classes are folded by xor shuffles at the end.
+template <int HD, int RATIO>
+__global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict__ q, const int8_t* __restrict__ ck,
+                                                        const int8_t* __restrict__ cv, const float* __restrict__ sk,
+                                                        const float* __restrict__ sv, uint16_t* __restrict__ out,
+                                                        const int* __restrict__ positions, int seq_len_arg,
+                                                        int n_head_kv, float scale, size_t kv_stride)
+{
+    constexpr int CH = HD / 16;                 // lanes per position in phase 3
+    constexpr int PG = 64 / CH;                 // positions per load instruction
+    constexpr int OWN = (RATIO + 3) / 4;        // heads per wave
+    __shared__ float qs[RATIO * HD];
+    __shared__ float ps[RATIO * ATT_TILE];
+    const int kvh = blockIdx.x, b = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int seq_len = positions ? positions[b] + 1 : seq_len_arg;
+    const int n_head = n_head_kv * RATIO;
+    const size_t kv_dim = (size_t)n_head_kv * HD;
+    const int8_t* kbase = ck + (size_t)b * kv_stride + (size_t)kvh * HD;
+    const int8_t* vbase = cv + (size_t)b * kv_stride + (size_t)kvh * HD;
+    const size_t sstride = kv_stride / HD;
+    const float* skb = sk + (size_t)b * sstride + kvh;
+    const float* svb = sv + (size_t)b * sstride + kvh;
+    const float* qb = q + (size_t)b * n_head * HD + (size_t)kvh * RATIO * HD;
+    for (int i = tid; i < RATIO * HD; i += 256) qs[i] = qb[i];
+    __syncthreads();
+
+    float m_run[OWN], l_run[OWN], acc[OWN][16];
+#pragma unroll
+    for (int j = 0; j < OWN; j++) {
+        m_run[j] = -1e30f;
+        l_run[j] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[j][e] = 0.0f;
+    }
+    const int g = lane / CH, c = lane % CH;     // phase 3: position class, 16-dim chunk
+
+    for (int t0 = 0; t0 < seq_len; t0 += ATT_TILE) {
+        const int tl = min(ATT_TILE, seq_len - t0);
+        // ---- phase 1
+        if (tid < tl) {
+            const int t = t0 + tid;
+            const uint4* kr = (const uint4*)(kbase + (size_t)t * kv_dim);
+            uint4 kk[CH];
+#pragma unroll
+            for (int u = 0; u < CH; u++) kk[u] = kr[u];
+            const float kscale = skb[(size_t)t * n_head_kv] * scale;
+            float dot[RATIO];
+#pragma unroll
+            for (int h = 0; h < RATIO; h++) dot[h] = 0.0f;
+#pragma unroll
+            for (int u = 0; u < CH; u++) {
+                const uint32_t w4[4] = {kk[u].x, kk[u].y, kk[u].z, kk[u].w};
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const float kv = (float)(int8_t)((w4[e >> 2] >> (8 * (e & 3))) & 0xFF);
+#pragma unroll
+                    for (int h = 0; h < RATIO; h++) dot[h] += qs[h * HD + u * 16 + e] * kv;
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < RATIO; h++) ps[h * ATT_TILE + tid] = dot[h] * kscale;
+        }
+        __syncthreads();
+        // ---- phases 2 + 3, one wave per head
+#pragma unroll
+        for (int j = 0; j < OWN; j++) {
+            const int h = wave + 4 * j;
+            if (h < RATIO) {                                     // wave-uniform
+                float* ph = ps + h * ATT_TILE;
+                float sc[ATT_TILE / 64];
+                float tmax = -1e30f;
+#pragma unroll
+                for (int i = 0; i < ATT_TILE / 64; i++) {
+                    const int t = lane + 64 * i;
+                    sc[i] = t < tl ? ph[t] : -1e30f;
+                    tmax = fmaxf(tmax, sc[i]);
+                }
+                tmax = wave_max(tmax);
+                const float m_new = fmaxf(m_run[j], tmax);
+                const float corr = expf(m_run[j] - m_new);
+                float psum = 0.0f;
+#pragma unroll
+                for (int i = 0; i < ATT_TILE / 64; i++) {
+                    const int t = lane + 64 * i;
+                    const float pv = t < tl ? expf(sc[i] - m_new) : 0.0f;
+                    if (t < tl) ph[t] = pv;
+                    psum += pv;
+                }
+                psum = t12_wave_sum(psum);
+                l_run[j] = l_run[j] * corr + psum;
+                m_run[j] = m_new;
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[j][e] *= corr;
+                // P.V: iteration it covers positions it*PG + g; loads of 4 iterations are issued together
+                for (int it = 0; it * PG < tl; it += 4) {
+                    uint4 vv[4];
+                    float w[4];
+#pragma unroll
+                    for (int x = 0; x < 4; x++) {
+                        const int t = (it + x) * PG + g;
+                        const bool ok = t < tl;
+                        const int tc = ok ? t : 0;
+                        vv[x] = *(const uint4*)(vbase + (size_t)(t0 + tc) * kv_dim + c * 16);
+                        w[x] = ok ? ph[tc] * svb[(size_t)(t0 + tc) * n_head_kv] : 0.0f;
+                    }
+#pragma unroll
+                    for (int x = 0; x < 4; x++) {
+                        const uint32_t w4[4] = {vv[x].x, vv[x].y, vv[x].z, vv[x].w};
+#pragma unroll
+                        for (int e = 0; e < 16; e++)
+                            acc[j][e] += w[x] * (float)(int8_t)((w4[e >> 2] >> (8 * (e & 3))) & 0xFF);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int j = 0; j < OWN; j++) {
+        const int h = wave + 4 * j;
+        if (h < RATIO) {
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                float v = acc[j][e];
+#pragma unroll
+                for (int off = CH; off < 64; off <<= 1) v += __shfl_xor(v, off, T12_WAVE);   // fold position classes
+                acc[j][e] = v;
+            }
+            if (g == 0) {
+                const float inv = 1.0f / l_run[j];
+                uint32_t o[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    o[e] = t12_f32_to_bf16(acc[j][2 * e] * inv) | ((uint32_t)t12_f32_to_bf16(acc[j][2 * e + 1] * inv) << 16);
+                uint4* dst = (uint4*)(out + (size_t)b * n_head * HD + (size_t)(kvh * RATIO + h) * HD + c * 16);
+                dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
+                dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------ argmax
 // Lowest index among equal maxima (the reference's tie rule depends on its
 // thread layout, kernels.hip:103-118; exact ties between fp32 logits do not
@@ -448,6 +599,8 @@ void launch_rope_kv(float* q, float* k, const float* v, int8_t* ck, int8_t* cv, 
     report("rope/kv-store");
 }
 
+int g_attn_fast = 1;   // 0: always the general kernel (tests compare the two)
+
 void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float* sk, const float* sv, int16_t* out,
                  const int* positions, int seq_len, int n_head, int n_head_kv, int head_dim, float scale, int batch,
                  size_t kv_stride, hipStream_t st)
@@ -459,6 +612,22 @@ void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float
         fprintf(stderr, "turbo12: %s\n", t12_last_error());
         return;
     }
+#define T12_ATT_FAST(HD_, R_)                                                                                   \
+    if (head_dim == HD_ && ratio == R_) {                                                                       \
+        hipLaunchKernelGGL((attn_fast_kernel<HD_, R_>), dim3(n_head_kv, batch), dim3(256), 0, st, q, ck, cv, sk, sv, \
+                           (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride);                    \
+        report("attention");                                                                                    \
+        return;                                                                                                 \
+    }
+    if (g_attn_fast) {
+        T12_ATT_FAST(128, 4)
+        T12_ATT_FAST(128, 1)
+        T12_ATT_FAST(128, 2)
+        T12_ATT_FAST(128, 8)
+        T12_ATT_FAST(64, 1)
+        T12_ATT_FAST(64, 4)
+    }
+#undef T12_ATT_FAST
     const size_t smem = ((size_t)ratio * head_dim + (size_t)ratio * ATT_TILE + 17 + 2 * ratio) * sizeof(float);
     hipLaunchKernelGGL(attn_decode_kernel, dim3(n_head_kv, batch), dim3(256), smem, st, q, ck, cv, sk, sv,
                        (uint16_t*)out, positions, seq_len, n_head, n_head_kv, head_dim, scale, kv_stride);
@@ -471,6 +640,13 @@ void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float
 extern "C" {
 
 void launch_rope_init(int head_dim, float theta_base) { (void)rope_table(head_dim, theta_base); }
+
+// 1 (default): shapes with a specialised attention kernel use it; 0: always the general kernel.
+int t12_tune_attention(int fast)
+{
+    g_attn_fast = fast;
+    return 0;
+}
 
 void launch_embed_lookup(const int16_t* embd_table, const int* token_ids, float* output, int n_embd, int batch_size,
                          int n_vocab, hipStream_t stream)
