@@ -85,6 +85,17 @@ int t12_gemv(const T12Segment* segs, int nseg, const void* act_bf16, int K, void
 int t12_gemv_swiglu(const T12Segment* gate, const T12Segment* up, const void* act_bf16, int K,
                     void* out_bf16, void* stream);
 
+/* The same two entry points with the reference's RMSNorm kernels folded into the prologue:
+ * activations = bf16( rmsnorm(x [+ residual]) * norm_w ), x / residual / norm_w fp32 [K]
+ * (engine/kernels.hip:355-442).  residual may be NULL (plain RMSNorm).  hidden_out, if not
+ * NULL, receives x + residual (the updated residual stream) and may not alias x or residual.
+ * Requires K % 16 == 0, K <= 8192, base_exp in 0..240. */
+int t12_gemv_norm(const T12Segment* segs, int nseg, const float* x, const float* residual,
+                  const float* norm_w, float eps, float* hidden_out, int K, void* stream);
+int t12_gemv_swiglu_norm(const T12Segment* gate, const T12Segment* up, const float* x,
+                         const float* residual, const float* norm_w, float eps, float* hidden_out,
+                         int K, void* out_bf16, void* stream);
+
 /* ---- (a') small batch, 1 <= B <= 8 -----------------------------------------
  * Same contract as t12_gemm, restricted to the batch sizes of the reference's
  * launch_split12_batch4_async / _batch8_async (decompress_v2.hip:860,877), with

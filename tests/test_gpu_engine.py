@@ -116,6 +116,28 @@ def test_batched_forward_equals_b1(t12, small_model):
             eb.close()
 
 
+def test_fused_and_unfused_b1_paths_agree(t12, small_model):
+    """TURBO_NO_FUSE=1 runs one launch per reference kernel; the default B = 1 path fuses norms, SiLU*mul,
+    RoPE and the KV store into the linears / attention.  Same logits up to bf16 rounding flips."""
+    path, _ = small_model
+    outs = {}
+    for flag in ("1", "0"):
+        os.environ["TURBO_NO_FUSE"] = flag
+        e = t12.Engine.load(path, batch=1)
+        try:
+            seq = []
+            for tok in [9, 200, 31, 7]:
+                e.forward([tok])
+                seq.append(e.logits(SMALL["n_vocab"]).clone())
+            outs[flag] = seq
+        finally:
+            e.close()
+    os.environ.pop("TURBO_NO_FUSE")
+    for a, b in zip(outs["0"], outs["1"]):
+        assert float((a - b).abs().max() / b.abs().max()) < 1e-2
+        assert int(a.argmax()) == int(b.argmax())
+
+
 def test_loader_reads_files_bit_exact(t12, oracle, small_model, modelio):
     path, _ = small_model
     eng = t12.Engine.load(path, batch=1)

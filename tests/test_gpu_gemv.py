@@ -260,3 +260,44 @@ def test_gemv_swiglu_fused_is_bit_identical_to_unfused(t12, oracle, synth, M, K)
     gf, rf = oracle.bf16_bits_to_f32(got), oracle.bf16_bits_to_f32(ref)
     assert np.abs(gf - rf).max() <= 2e-2 * np.abs(rf).max()
     assert (got == ref).mean() > 0.97
+
+
+@pytest.mark.parametrize("K,with_res", [(4096, True), (4096, False), (1040, True), (8192, True), (16, False)])
+def test_gemv_norm_prologue(t12, oracle, synth, K, with_res):
+    """t12_gemv_norm / t12_gemv_swiglu_norm: RMSNorm (+ residual add) folded into the GEMV prologue."""
+    import ctypes
+    rng = np.random.default_rng(K)
+    M = 264
+    pa = oracle.pack(synth.weights_llm(M, K, seed=91, p_outlier=2e-3))
+    pb = oracle.pack(synth.weights_llm(M, K, seed=92, sigma=0.1, p_outlier=2e-3))
+    x = rng.standard_normal(K).astype(np.float32) * 2
+    r = rng.standard_normal(K).astype(np.float32) if with_res else None
+    w = (1 + 0.1 * rng.standard_normal(K)).astype(np.float32)
+    s = x + r if with_res else x
+    a_bits = oracle.rms_norm_bf16(s, w, 1e-5)
+    da, db = (t12.DeviceTensor12.from_packed(p, dev()) for p in (pa, pb))
+    xd, wd = torch.from_numpy(x).to(dev()), torch.from_numpy(w).to(dev())
+    rd = torch.from_numpy(r).to(dev()) if with_res else None
+    hid = torch.zeros(K, device=dev())
+    oa, ob = torch.zeros(M, device=dev()), torch.zeros(M, device=dev())
+    segs = t12._seg_array([da.segment(oa), db.segment(ob)])
+    st = t12.current_stream()
+    t12.check(t12.lib.t12_gemv_norm(segs, 2, xd.data_ptr(), rd.data_ptr() if with_res else None, wd.data_ptr(), 1e-5,
+                                    hid.data_ptr() if with_res else None, K, st))
+    torch.cuda.synchronize()
+    for o, p in ((oa, pa), (ob, pb)):
+        assert rel_err(o.cpu().numpy(), oracle.gemv(p, a_bits)) < 2e-3     # a 1-ulp bf16 flip in the prologue is allowed
+    if with_res:
+        assert np.array_equal(hid.cpu().numpy(), s)
+    fused = torch.zeros(M, dtype=torch.int16, device=dev())
+    sg, su = da.segment(None), db.segment(None)
+    t12.check(t12.lib.t12_gemv_swiglu_norm(ctypes.byref(sg), ctypes.byref(su), xd.data_ptr(),
+                                           rd.data_ptr() if with_res else None, wd.data_ptr(), 1e-5, None, K,
+                                           fused.data_ptr(), st))
+    torch.cuda.synchronize()
+    ref = oracle.bf16_bits_to_f32(oracle.silu_mul_bf16(oracle.gemv(pa, a_bits), oracle.gemv(pb, a_bits)))
+    got = oracle.bf16_bits_to_f32(fused.cpu().numpy().view(np.uint16))
+    assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max()
+    # aliasing is rejected
+    if with_res:
+        assert t12.lib.t12_gemv_norm(segs, 2, xd.data_ptr(), rd.data_ptr(), wd.data_ptr(), 1e-5, xd.data_ptr(), K, st) == -1

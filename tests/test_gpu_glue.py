@@ -201,3 +201,39 @@ def test_argmax(t12, oracle):
     xd = torch.from_numpy(nanrow).to(dev()); r = torch.zeros(1, dtype=torch.int32, device=dev())
     t12.lib.launch_argmax(xd.data_ptr(), r.data_ptr(), 300, st(t12)); torch.cuda.synchronize()
     assert r.item() == 17
+
+
+@pytest.mark.parametrize("nh,nkv,hd,B", [(32, 8, 128, 1), (32, 8, 128, 5), (4, 4, 64, 2), (8, 2, 32, 3)])
+def test_fused_rope_store_attention_equals_separate_launches(t12, oracle, nh, nkv, hd, B):
+    """launch_rope_store_attention == launch_rope_store_kv_batch + launch_attention_all_heads_batch:
+    same caches, same scales, same bf16 output (the fused kernel leaves q unrotated)."""
+    rng = np.random.default_rng(B)
+    theta, max_seq, pos = 500000.0, 300, 277
+    q, k, v = make_qkv(rng, B, nh, nkv, hd)
+    q[1:], k[1:], v[1:] = q[0], k[0], v[0]          # lock-step copies: all sequences share one cache slot
+    kc = rng.integers(-127, 128, size=(max_seq, nkv, hd)).astype(np.int8)
+    vc = rng.integers(-127, 128, size=(max_seq, nkv, hd)).astype(np.int8)
+    ks = (rng.random((max_seq, nkv)).astype(np.float32) + 0.5) / 127
+    vs = (rng.random((max_seq, nkv)).astype(np.float32) + 0.5) / 127
+    pd = torch.full((B,), pos, dtype=torch.int32, device=dev())
+    sc = 1.0 / np.sqrt(hd)
+
+    def fresh():
+        return [torch.from_numpy(a.copy()).to(dev()) for a in (q, k, v, kc, vc, ks, vs)]
+
+    a = fresh(); oa = torch.zeros((B, nh * hd), dtype=torch.int16, device=dev())
+    t12.lib.launch_rope_store_kv_batch(a[0].data_ptr(), a[1].data_ptr(), a[2].data_ptr(), a[3].data_ptr(), a[4].data_ptr(),
+                                       a[5].data_ptr(), a[6].data_ptr(), pd.data_ptr(), hd, nh, nkv, nh * hd, nkv * hd,
+                                       theta, B, st(t12))
+    t12.lib.launch_attention_all_heads_batch(a[0].data_ptr(), a[3].data_ptr(), a[4].data_ptr(), a[5].data_ptr(),
+                                             a[6].data_ptr(), oa.data_ptr(), pd.data_ptr(), nh, nkv, hd, pos + 1, sc, B, 0,
+                                             st(t12))
+    for positions in ([pd.data_ptr()] if B > 1 else [pd.data_ptr(), None]):
+        f = fresh(); of = torch.zeros_like(oa)
+        t12.lib.launch_rope_store_attention(f[0].data_ptr(), f[1].data_ptr(), f[2].data_ptr(), f[3].data_ptr(),
+                                            f[4].data_ptr(), f[5].data_ptr(), f[6].data_ptr(), of.data_ptr(), positions,
+                                            pos, nh, nkv, hd, theta, sc, B, 0, st(t12))
+        torch.cuda.synchronize()
+        assert torch.equal(f[3], a[3]) and torch.equal(f[4], a[4])      # caches
+        assert torch.equal(f[5], a[5]) and torch.equal(f[6], a[6])      # scales
+        assert torch.equal(of, oa)

@@ -63,6 +63,7 @@ _SIGS = {
     "launch_store_kv_batch": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "launch_rope_store_kv": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _vp]),
     "launch_rope_store_kv_batch": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _i, _vp]),
+    "launch_rope_store_attention": (None, [_vp] * 9 + [_i, _i, _i, _i, C.c_float, C.c_float, _i, _i, _vp]),
     "launch_attention_all_heads": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _vp]),
     "launch_flash_attention": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _vp]),
     "launch_attention_all_heads_batch": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, C.c_float, _i, _i, _vp]),
@@ -87,6 +88,8 @@ _SIGS = {
     "t12_engine_sync": (_i, [_vp]),
     "t12_engine_weight": (_i, [_vp, _i, _i, C.POINTER(Segment), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "t12_gemv_swiglu": (_i, [C.POINTER(Segment), C.POINTER(Segment), _vp, _i, _vp, _vp]),
+    "t12_gemv_norm": (_i, [C.POINTER(Segment), _i, _vp, _vp, _vp, C.c_float, _vp, _i, _vp]),
+    "t12_gemv_swiglu_norm": (_i, [C.POINTER(Segment), C.POINTER(Segment), _vp, _vp, _vp, C.c_float, _vp, _i, _vp, _vp]),
     "t12_gemv_batch": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
     "launch_split12_batch4_async": (_i, [_vp] * 2 + [_i] + [_vp] * 4 + [_vp] * 3 + [_vp] * 4 + [_i, _i, _vp]),
     "launch_split12_batch8_async": (_i, [_vp] * 2 + [_i] + [_vp] * 8 + [_vp] * 3 + [_vp] * 8 + [_i, _i, _vp]),

@@ -32,6 +32,8 @@ void launch_attention_all_heads(const float*, const int8_t*, const int8_t*, cons
                                 int, int, int, int, float, hipStream_t);
 void launch_attention_all_heads_batch(const float*, const int8_t*, const int8_t*, const float*, const float*, int16_t*,
                                       const int*, int, int, int, int, float, int, int, hipStream_t);
+void launch_rope_store_attention(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int16_t*, const int*,
+                                 int, int, int, int, float, float, int, int, hipStream_t);
 }
 
 namespace {
@@ -42,6 +44,8 @@ struct LayerSegs {
 struct Impl {
     std::vector<LayerSegs> layers;
     T12Segment head[1];
+    bool fused_b1 = false;     // B = 1 takes the 5-launch-per-layer path
+    bool checked = false;
 };
 
 void check_gpu(hipError_t e, const char* what)
@@ -111,7 +115,7 @@ InferenceState* create_inference_state(Model* model, int batch_size, int max_seq
     s->v_buf = fbuf(bs * kv_dim);
     s->ffn_gate = fbuf(bs * n_ff);
     s->ffn_up = fbuf(bs * n_ff);
-    s->ffn_down = nullptr;
+    s->ffn_down = fbuf(bs * n);    // output of w_down on the fused B = 1 path
     s->logits = fbuf(bs * n_vocab);
     s->attn_scores_buf = nullptr;
     check_gpu(hipMalloc((void**)&s->d_positions, bs * sizeof(int)), "hipMalloc");
@@ -126,6 +130,8 @@ InferenceState* create_inference_state(Model* model, int batch_size, int max_seq
 
     auto* impl = new Impl();
     impl->layers.resize(c.n_layer);
+    const char* nofuse = getenv("TURBO_NO_FUSE");     // debugging aid: one kernel per reference kernel
+    impl->fused_b1 = !(nofuse && nofuse[0] == '1');   // confirmed against the tensors at the first forward
     s->impl = impl;
     init_sampler(batch_size);
     return s;
@@ -148,6 +154,97 @@ void free_inference_state(InferenceState* state)
     delete state;
 }
 
+namespace {
+
+bool exp_ok(const CompressedWeight& w) { return w.split_sm && w.base_exp >= 0 && w.base_exp <= 240; }
+
+// Every tensor can take the fast decode-GEMV with fused prologues / epilogues.
+bool fused_b1_eligible(const Model* m)
+{
+    const ModelConfig& c = m->config;
+    if (c.n_embd % 16 || c.n_embd > 8192 || c.n_ff % 16 || c.n_layer < 1) return false;
+    if (!exp_ok(m->output_proj)) return false;
+    for (const auto& L : m->layers)
+        for (const CompressedWeight* w : {&L.wq, &L.wk, &L.wv, &L.wo, &L.w_gate, &L.w_up, &L.w_down})
+            if (!exp_ok(*w)) return false;
+    return true;
+}
+
+void must(int rc, const char* what)
+{
+    if (rc != T12_OK) {
+        fprintf(stderr, "ERROR: %s failed: %s\n", what, t12_last_error());
+        exit(1);
+    }
+}
+
+// B = 1 decode step in 5 launches per layer:
+//   [RMSNorm (+ residual add)] + wq|wk|wv      t12_gemv_norm
+//   RoPE + INT8 KV store + GQA attention        launch_rope_store_attention
+//   wo                                          t12_gemv
+//   residual add + RMSNorm + gate|up + SiLU*mul t12_gemv_swiglu_norm
+//   w_down                                      t12_gemv
+// The residual stream ping-pongs between hidden and hidden2 (a norm prologue reads one and
+// workgroup 0 writes the sum into the other); the additions the reference does in
+// add_rms_norm_bf16_batch (inference.cpp:301,341-346) happen in the prologue of the next linear.
+void forward_b1_fused(InferenceState* state, const int* token_ids)
+{
+    Model* m = state->model;
+    const ModelConfig& c = m->config;
+    hipStream_t st = state->stream;
+    const int n = c.n_embd, n_ff = c.n_ff, head_dim = n / c.n_head;
+    const int kv_dim = c.n_head_kv * head_dim;
+    const float scale = 1.0f / sqrtf((float)head_dim);
+    Impl* impl = (Impl*)state->impl;
+    const int pos = state->positions[0];
+
+    (void)hipMemcpyAsync(state->d_tokens, token_ids, sizeof(int), hipMemcpyHostToDevice, st);
+    launch_embed_lookup(m->token_embd, state->d_tokens, state->hidden, n, 1, c.n_vocab, st);
+
+    float* h = state->hidden;          // residual stream
+    float* h_alt = state->hidden2;
+    float* o_out = state->attn_out;    // output of wo
+    float* d_out = state->ffn_down;    // output of w_down (pending addition)
+    int16_t* bf16_a = state->bf16_act;
+    int16_t* bf16_b = state->bf16_act2;
+    const float* pending = nullptr;    // residual not yet added into h
+
+    for (int layer = 0; layer < c.n_layer; layer++) {
+        TransformerLayer& L = m->layers[layer];
+        LayerSegs& S = impl->layers[layer];
+        S.qkv[0] = seg_of(L.wq, state->q_buf, n);
+        S.qkv[1] = seg_of(L.wk, state->k_buf, kv_dim);
+        S.qkv[2] = seg_of(L.wv, state->v_buf, kv_dim);
+        must(t12_gemv_norm(S.qkv, 3, h, pending, L.attn_norm, c.rms_norm_eps, pending ? h_alt : nullptr, n, st),
+             "qkv decode-GEMV");
+        if (pending) std::swap(h, h_alt);
+
+        const size_t kv_off = (size_t)layer * m->max_seq_len * kv_dim;
+        const size_t sc_off = (size_t)layer * m->max_seq_len * c.n_head_kv;
+        launch_rope_store_attention(state->q_buf, state->k_buf, state->v_buf, m->kv_cache_k + kv_off,
+                                    m->kv_cache_v + kv_off, m->kv_scale_k + sc_off, m->kv_scale_v + sc_off, bf16_a,
+                                    nullptr, pos, c.n_head, c.n_head_kv, head_dim, c.rope_theta, scale, 1, 0, st);
+
+        S.o[0] = seg_of(L.wo, o_out, n);
+        must(t12_gemv(S.o, 1, bf16_a, n, st), "wo decode-GEMV");
+
+        S.gateup[0] = seg_of(L.w_gate, nullptr, n_ff);
+        S.gateup[1] = seg_of(L.w_up, nullptr, n_ff);
+        must(t12_gemv_swiglu_norm(&S.gateup[0], &S.gateup[1], h, o_out, L.ffn_norm, c.rms_norm_eps, h_alt, n, bf16_b, st),
+             "gate|up decode-GEMV");
+        std::swap(h, h_alt);
+
+        S.down[0] = seg_of(L.w_down, d_out, n);
+        must(t12_gemv(S.down, 1, bf16_b, n_ff, st), "w_down decode-GEMV");
+        pending = d_out;
+    }
+    impl->head[0] = seg_of(m->output_proj, state->logits, c.n_vocab);
+    must(t12_gemv_norm(impl->head, 1, h, pending, m->output_norm, c.rms_norm_eps, nullptr, n, st), "lm_head decode-GEMV");
+    state->positions[0] = pos + 1;
+}
+
+}  // namespace
+
 void forward(InferenceState* state, const int* token_ids)
 {
     Model* m = state->model;
@@ -164,6 +261,16 @@ void forward(InferenceState* state, const int* token_ids)
     if (max_pos >= m->max_seq_len) {
         fprintf(stderr, "ERROR: position %d exceeds the KV cache (%d)\n", max_pos, m->max_seq_len);
         exit(1);
+    }
+    if (B == 1 && impl->fused_b1) {
+        if (!impl->checked) {
+            impl->checked = true;
+            impl->fused_b1 = fused_b1_eligible(m);
+        }
+        if (impl->fused_b1) {
+            forward_b1_fused(state, token_ids);
+            return;
+        }
     }
     (void)hipMemcpyAsync(state->d_tokens, token_ids, B * sizeof(int), hipMemcpyHostToDevice, st);
     if (B > 1) (void)hipMemcpyAsync(state->d_positions, state->positions, B * sizeof(int), hipMemcpyHostToDevice, st);
@@ -186,22 +293,11 @@ void forward(InferenceState* state, const int* token_ids)
 
         const size_t kv_off = (size_t)layer * m->max_seq_len * kv_dim;
         const size_t sc_off = (size_t)layer * m->max_seq_len * c.n_head_kv;
-        if (B == 1) {
-            launch_rope_store_kv(state->q_buf, state->k_buf, state->v_buf, m->kv_cache_k + kv_off,
-                                 m->kv_cache_v + kv_off, m->kv_scale_k + sc_off, m->kv_scale_v + sc_off, head_dim,
-                                 c.n_head, c.n_head_kv, state->positions[0], m->max_seq_len, c.rope_theta, st);
-            launch_attention_all_heads(state->q_buf, m->kv_cache_k + kv_off, m->kv_cache_v + kv_off,
-                                       m->kv_scale_k + sc_off, m->kv_scale_v + sc_off, bf16_a, c.n_head, c.n_head_kv,
-                                       head_dim, state->positions[0] + 1, m->max_seq_len, scale, st);
-        } else {
-            launch_rope_store_kv_batch(state->q_buf, state->k_buf, state->v_buf, m->kv_cache_k + kv_off,
-                                       m->kv_cache_v + kv_off, m->kv_scale_k + sc_off, m->kv_scale_v + sc_off,
-                                       state->d_positions, head_dim, c.n_head, c.n_head_kv, n, kv_dim, c.rope_theta, B,
-                                       st);
-            launch_attention_all_heads_batch(state->q_buf, m->kv_cache_k + kv_off, m->kv_cache_v + kv_off,
-                                             m->kv_scale_k + sc_off, m->kv_scale_v + sc_off, bf16_a, state->d_positions,
-                                             c.n_head, c.n_head_kv, head_dim, max_pos + 1, scale, B, 0, st);
-        }
+        // RoPE (Q, K) + INT8 KV store + GQA attention: one launch
+        launch_rope_store_attention(state->q_buf, state->k_buf, state->v_buf, m->kv_cache_k + kv_off,
+                                    m->kv_cache_v + kv_off, m->kv_scale_k + sc_off, m->kv_scale_v + sc_off, bf16_a,
+                                    B == 1 ? nullptr : state->d_positions, state->positions[0], c.n_head, c.n_head_kv,
+                                    head_dim, c.rope_theta, scale, B, 0, st);
 
         S.o[0] = seg_of(L.wo, res, n);
         run_linear(S.o, 1, bf16_a, n, B, st);

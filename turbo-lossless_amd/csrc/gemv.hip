@@ -28,6 +28,12 @@ struct GemvParams {
     int K;
     const uint16_t* act;
     uint16_t* out_bf16;                    // SwiGLU mode only
+    // RMSNorm prologue (NORM > 0): activations = bf16(rmsnorm(nx [+ nres]) * nw)
+    const float* nx;
+    const float* nres;
+    const float* nw;
+    float* hidden_out;                     // nx + nres, written by workgroup 0 (may be null)
+    float eps;
 };
 
 __device__ __forceinline__ int find_segment(const GemvParams& p, int blk)
@@ -90,7 +96,11 @@ __device__ __forceinline__ float lds_act_at(const uint4* lds_act, int k)
 // segment 1 (up); the wave writes bf16( silu(gate.x) * (up.x) ) to p.out_bf16[m] instead of two
 // fp32 sums -- the reference's split12_matvec_v2_dual (decompress_v2.hip:387-523) with its
 // silu_mul_bf16 kernel (engine/kernels.hip:447-459) folded into the epilogue.
-template <int NW, int R, int D, int MINB, bool SWIGLU = false>
+// NORM (1: RMSNorm, 2: residual add + RMSNorm): instead of reading bf16 activations, every
+// workgroup rebuilds them from the fp32 residual stream while its first weight tiles are in
+// flight -- the reference's (add_)rms_norm_bf16_batch kernels (engine/kernels.hip:355-442) as a
+// prologue.  K <= 16 * NW * 64.  Workgroup 0 also stores nx + nres for the residual path.
+template <int NW, int R, int D, int MINB, bool SWIGLU = false, int NORM = 0>
 __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvParams p)
 {
     static_assert(!SWIGLU || R == 2, "the SwiGLU epilogue pairs exactly two rows");
@@ -155,11 +165,62 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
         __builtin_amdgcn_sched_barrier(0);   // issue in ring order: waits can then be partial
     }
 
-    for (int q = tid; q < nchunk * 128; q += NW * 64) {
-        const int k = q * 8;
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (k < K) v = *(const uint4*)(p.act + k);
-        lds_act[(q >> 7) * 128 + (q & 1) * 64 + ((q & 127) >> 1)] = t12_pair_acts(v);
+    if (NORM == 0) {
+        for (int q = tid; q < nchunk * 128; q += NW * 64) {
+            const int k = q * 8;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (k < K) v = *(const uint4*)(p.act + k);
+            lds_act[(q >> 7) * 128 + (q & 1) * 64 + ((q & 127) >> 1)] = t12_pair_acts(v);
+        }
+    } else {
+        __shared__ float red[NW];
+        float v[2][8];
+        float ss = 0.0f;
+#pragma unroll
+        for (int gi = 0; gi < 2; gi++) {
+            const int k = (tid + gi * NW * 64) * 8;
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[gi][e] = 0.0f;
+            if (k < K) {
+                const float4 a = *(const float4*)(p.nx + k), b = *(const float4*)(p.nx + k + 4);
+                v[gi][0] = a.x; v[gi][1] = a.y; v[gi][2] = a.z; v[gi][3] = a.w;
+                v[gi][4] = b.x; v[gi][5] = b.y; v[gi][6] = b.z; v[gi][7] = b.w;
+                if (NORM == 2) {
+                    const float4 c = *(const float4*)(p.nres + k), d = *(const float4*)(p.nres + k + 4);
+                    v[gi][0] += c.x; v[gi][1] += c.y; v[gi][2] += c.z; v[gi][3] += c.w;
+                    v[gi][4] += d.x; v[gi][5] += d.y; v[gi][6] += d.z; v[gi][7] += d.w;
+                    if (blockIdx.x == 0 && p.hidden_out) {
+                        *(float4*)(p.hidden_out + k) = make_float4(v[gi][0], v[gi][1], v[gi][2], v[gi][3]);
+                        *(float4*)(p.hidden_out + k + 4) = make_float4(v[gi][4], v[gi][5], v[gi][6], v[gi][7]);
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 8; e++) ss += v[gi][e] * v[gi][e];
+            }
+        }
+        ss = t12_wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        float tot = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; w++) tot += red[w];
+        const float rn = rsqrtf(tot / (float)K + p.eps);
+#pragma unroll
+        for (int gi = 0; gi < 2; gi++) {
+            const int q = tid + gi * NW * 64;
+            const int k = q * 8;
+            if (q < nchunk * 128) {
+                uint4 y = make_uint4(0, 0, 0, 0);
+                if (k < K) {
+                    const float4 wa = *(const float4*)(p.nw + k), wb = *(const float4*)(p.nw + k + 4);
+                    y.x = t12_f32_to_bf16(v[gi][0] * rn * wa.x) | ((uint32_t)t12_f32_to_bf16(v[gi][1] * rn * wa.y) << 16);
+                    y.y = t12_f32_to_bf16(v[gi][2] * rn * wa.z) | ((uint32_t)t12_f32_to_bf16(v[gi][3] * rn * wa.w) << 16);
+                    y.z = t12_f32_to_bf16(v[gi][4] * rn * wb.x) | ((uint32_t)t12_f32_to_bf16(v[gi][5] * rn * wb.y) << 16);
+                    y.w = t12_f32_to_bf16(v[gi][6] * rn * wb.z) | ((uint32_t)t12_f32_to_bf16(v[gi][7] * rn * wb.w) << 16);
+                }
+                lds_act[(q >> 7) * 128 + (q & 1) * 64 + ((q & 127) >> 1)] = t12_pair_acts(y);
+            }
+        }
     }
     __syncthreads();
     if (!live) return;
@@ -295,6 +356,7 @@ int launch_stream(GemvParams& p, const T12Segment* segs, int nseg, hipStream_t s
     return T12_OK;
 }
 
+template <int NORM>
 int launch_swiglu(GemvParams& p, hipStream_t st)
 {
     const int NW = 8;
@@ -303,10 +365,47 @@ int launch_swiglu(GemvParams& p, hipStream_t st)
     p.blk_start[1] = p.blk_start[2] = total;
     const size_t lds = (size_t)((p.K + 1023) / 1024) * 2048;
     const int T = p.K / 1024;
-    if (T >= 2) hipLaunchKernelGGL((gemv_stream_kernel<8, 2, 2, 1, true>), dim3(total), dim3(NW * 64), lds, st, p);
-    else if (T == 1) hipLaunchKernelGGL((gemv_stream_kernel<8, 2, 1, 1, true>), dim3(total), dim3(NW * 64), lds, st, p);
-    else hipLaunchKernelGGL((gemv_stream_kernel<8, 2, 0, 1, true>), dim3(total), dim3(NW * 64), lds, st, p);
+    if (T >= 2)
+        hipLaunchKernelGGL((gemv_stream_kernel<8, 2, 2, 1, true, NORM>), dim3(total), dim3(NW * 64), lds, st, p);
+    else if (T == 1)
+        hipLaunchKernelGGL((gemv_stream_kernel<8, 2, 1, 1, true, NORM>), dim3(total), dim3(NW * 64), lds, st, p);
+    else
+        hipLaunchKernelGGL((gemv_stream_kernel<8, 2, 0, 1, true, NORM>), dim3(total), dim3(NW * 64), lds, st, p);
     T12_CHECK_LAUNCH("t12_gemv_swiglu");
+    return T12_OK;
+}
+
+template <int NORM>
+int launch_plain_norm(GemvParams& p, const T12Segment* segs, int nseg, hipStream_t st)
+{
+    const int NW = 8;
+    int total = 0;
+    for (int i = 0; i < nseg; i++) {
+        p.blk_start[i] = total;
+        total += (segs[i].M + NW - 1) / NW;
+    }
+    p.blk_start[nseg] = total;
+    const size_t lds = (size_t)((p.K + 1023) / 1024) * 2048;
+    const int T = p.K / 1024;
+    if (T >= 2)
+        hipLaunchKernelGGL((gemv_stream_kernel<8, 1, 2, 1, false, NORM>), dim3(total), dim3(NW * 64), lds, st, p);
+    else if (T == 1)
+        hipLaunchKernelGGL((gemv_stream_kernel<8, 1, 1, 1, false, NORM>), dim3(total), dim3(NW * 64), lds, st, p);
+    else
+        hipLaunchKernelGGL((gemv_stream_kernel<8, 1, 0, 1, false, NORM>), dim3(total), dim3(NW * 64), lds, st, p);
+    T12_CHECK_LAUNCH("t12_gemv_norm");
+    return T12_OK;
+}
+
+int check_norm_operands(const char* who, const T12Segment* segs, int nseg, const float* x, const float* residual,
+                        const float* norm_w, const float* hidden_out, int K)
+{
+    T12_REQUIRE(x && norm_w, "%s: x / norm weight is null", who);
+    T12_REQUIRE(K % 16 == 0 && K <= 8192, "%s: K %d must be a multiple of 16 and <= 8192", who, K);
+    T12_REQUIRE(!hidden_out || (hidden_out != x && hidden_out != residual), "%s: hidden_out may not alias x or residual", who);
+    for (int i = 0; i < nseg; i++)
+        T12_REQUIRE(segs[i].base_exp >= 0 && segs[i].base_exp <= 240, "%s: segment %d base_exp %d outside 0..240", who, i,
+                    segs[i].base_exp);
     return T12_OK;
 }
 
@@ -412,7 +511,55 @@ int t12_gemv_swiglu(const T12Segment* gate, const T12Segment* up, const void* ac
     p.K = K;
     p.act = (const uint16_t*)act_bf16;
     p.out_bf16 = (uint16_t*)out_bf16;
-    return launch_swiglu(p, (hipStream_t)stream);
+    return launch_swiglu<0>(p, (hipStream_t)stream);
+}
+
+// y_s = W_s . bf16(rmsnorm(x [+ residual]) * norm_w) with the norm computed in the kernel's prologue.
+int t12_gemv_norm(const T12Segment* segs, int nseg, const float* x, const float* residual, const float* norm_w, float eps,
+                  float* hidden_out, int K, void* stream)
+{
+    int rc = validate(segs, nseg, x, K, true);
+    if (rc) return rc;
+    rc = check_norm_operands("t12_gemv_norm", segs, nseg, x, residual, norm_w, hidden_out, K);
+    if (rc) return rc;
+    GemvParams p;
+    for (int i = 0; i < nseg; i++) p.seg[i] = segs[i];
+    p.nseg = nseg;
+    p.K = K;
+    p.act = nullptr;
+    p.out_bf16 = nullptr;
+    p.nx = x;
+    p.nres = residual;
+    p.nw = norm_w;
+    p.hidden_out = hidden_out;
+    p.eps = eps;
+    return residual ? launch_plain_norm<2>(p, segs, nseg, (hipStream_t)stream)
+                    : launch_plain_norm<1>(p, segs, nseg, (hipStream_t)stream);
+}
+
+int t12_gemv_swiglu_norm(const T12Segment* gate, const T12Segment* up, const float* x, const float* residual,
+                         const float* norm_w, float eps, float* hidden_out, int K, void* out_bf16, void* stream)
+{
+    T12_REQUIRE(gate && up && out_bf16, "t12_gemv_swiglu_norm: null operand");
+    T12Segment two[2] = {*gate, *up};
+    int rc = validate(two, 2, x, K, false);
+    if (rc) return rc;
+    T12_REQUIRE(gate->M == up->M, "t12_gemv_swiglu_norm: gate has %d rows, up has %d", gate->M, up->M);
+    rc = check_norm_operands("t12_gemv_swiglu_norm", two, 2, x, residual, norm_w, hidden_out, K);
+    if (rc) return rc;
+    GemvParams p;
+    p.seg[0] = two[0];
+    p.seg[1] = two[1];
+    p.nseg = 2;
+    p.K = K;
+    p.act = nullptr;
+    p.out_bf16 = (uint16_t*)out_bf16;
+    p.nx = x;
+    p.nres = residual;
+    p.nw = norm_w;
+    p.hidden_out = hidden_out;
+    p.eps = eps;
+    return residual ? launch_swiglu<2>(p, (hipStream_t)stream) : launch_swiglu<1>(p, (hipStream_t)stream);
 }
 
 // ---- reference-named launchers ---------------------------------------------

@@ -334,12 +334,26 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
 //   phase 3  the same wave: P.V with 128-bit V loads -- 8 (HD=128) or 4 (HD=64) lanes span one
 //            position, so one load instruction covers 8 / 16 positions; each lane keeps 16
 //            output dims for its position class, classes are folded by xor shuffles at the end.
-template <int HD, int RATIO>
+// FUSE: the kernel first does what rope_kv_kernel<3> does for its own heads -- rotates the
+// RATIO query heads while loading them, rotates this KV head's new K, quantises K and V to
+// INT8 and stores them at position pos -- and only then attends over positions 0..pos.
+// (All B workgroups of a shared cache, kv_stride = 0, store identical values into one slot.)
+struct AttnFuse {
+    const float* k_new;      // [B, n_head_kv * HD] fp32, unrotated
+    const float* v_new;
+    int8_t* ck_w;            // writable views of the caches / scales
+    int8_t* cv_w;
+    float* sk_w;
+    float* sv_w;
+    const float* freqs;      // [HD / 2]
+};
+
+template <int HD, int RATIO, bool FUSE = false>
 __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict__ q, const int8_t* __restrict__ ck,
                                                         const int8_t* __restrict__ cv, const float* __restrict__ sk,
                                                         const float* __restrict__ sv, uint16_t* __restrict__ out,
                                                         const int* __restrict__ positions, int seq_len_arg,
-                                                        int n_head_kv, float scale, size_t kv_stride)
+                                                        int n_head_kv, float scale, size_t kv_stride, AttnFuse fz)
 {
     constexpr int CH = HD / 16;                 // lanes per position in phase 3
     constexpr int PG = 64 / CH;                 // positions per load instruction
@@ -357,7 +371,46 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
     const float* skb = sk + (size_t)b * sstride + kvh;
     const float* svb = sv + (size_t)b * sstride + kvh;
     const float* qb = q + (size_t)b * n_head * HD + (size_t)kvh * RATIO * HD;
-    for (int i = tid; i < RATIO * HD; i += 256) qs[i] = qb[i];
+    if (!FUSE) {
+        for (int i = tid; i < RATIO * HD; i += 256) qs[i] = qb[i];
+    } else {
+        constexpr int HALF = HD / 2;
+        const int pos = seq_len - 1;
+        for (int i = tid; i < RATIO * HALF; i += 256) {              // rotate Q on the way into LDS
+            const int h = i / HALF, d = i % HALF;
+            float sn, cs;
+            sincosf((float)pos * fz.freqs[d], &sn, &cs);
+            const float x0 = qb[h * HD + d], x1 = qb[h * HD + d + HALF];
+            qs[h * HD + d] = x0 * cs - x1 * sn;
+            qs[h * HD + d + HALF] = x0 * sn + x1 * cs;
+        }
+        if (wave < 2) {                                              // wave 0: K (rotated), wave 1: V
+            const bool own = lane < HALF;
+            const float* src = (wave == 0 ? fz.k_new : fz.v_new) + (size_t)b * kv_dim + (size_t)kvh * HD;
+            float r0 = 0.0f, r1 = 0.0f;
+            if (own) {
+                r0 = src[lane];
+                r1 = src[lane + HALF];
+                if (wave == 0) {
+                    float sn, cs;
+                    sincosf((float)pos * fz.freqs[lane], &sn, &cs);
+                    const float x0 = r0, x1 = r1;
+                    r0 = x0 * cs - x1 * sn;
+                    r1 = x0 * sn + x1 * cs;
+                }
+            }
+            const float amax = wave_max(fmaxf(fabsf(r0), fabsf(r1)));
+            const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+            int8_t* row = (wave == 0 ? fz.ck_w : fz.cv_w) + (size_t)b * kv_stride + (size_t)pos * kv_dim + (size_t)kvh * HD;
+            if (own) {
+                row[lane] = (int8_t)(int)fminf(fmaxf(rintf(r0 * inv), -127.0f), 127.0f);
+                row[lane + HALF] = (int8_t)(int)fminf(fmaxf(rintf(r1 * inv), -127.0f), 127.0f);
+            }
+            if (lane == 0)
+                (wave == 0 ? fz.sk_w : fz.sv_w)[(size_t)b * sstride + (size_t)pos * n_head_kv + kvh] = amax / 127.0f;
+        }
+        __threadfence();      // the new row is read back through the cache pointers below
+    }
     __syncthreads();
 
     float m_run[OWN], l_run[OWN], acc[OWN][16];
@@ -601,9 +654,17 @@ void launch_rope_kv(float* q, float* k, const float* v, int8_t* ck, int8_t* cv, 
 
 int g_attn_fast = 1;   // 0: always the general kernel (tests compare the two)
 
+bool attn_has_fast(int n_head, int n_head_kv, int head_dim)
+{
+    if (!g_attn_fast || n_head_kv <= 0 || n_head % n_head_kv) return false;
+    const int r = n_head / n_head_kv;
+    return (head_dim == 128 && (r == 1 || r == 2 || r == 4 || r == 8)) || (head_dim == 64 && (r == 1 || r == 4));
+}
+
+// fuse != nullptr: RoPE + INT8 KV store happen inside the attention kernel (fast shapes only).
 void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float* sk, const float* sv, int16_t* out,
                  const int* positions, int seq_len, int n_head, int n_head_kv, int head_dim, float scale, int batch,
-                 size_t kv_stride, hipStream_t st)
+                 size_t kv_stride, hipStream_t st, const AttnFuse* fuse = nullptr)
 {
     const int ratio = n_head / n_head_kv;
     if (ratio < 1 || ratio > ATT_MAX_RATIO || n_head % n_head_kv || head_dim % 16 || head_dim > 128) {
@@ -614,8 +675,12 @@ void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float
     }
 #define T12_ATT_FAST(HD_, R_)                                                                                   \
     if (head_dim == HD_ && ratio == R_) {                                                                       \
-        hipLaunchKernelGGL((attn_fast_kernel<HD_, R_>), dim3(n_head_kv, batch), dim3(256), 0, st, q, ck, cv, sk, sv, \
-                           (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride);                    \
+        if (fuse)                                                                                               \
+            hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, true>), dim3(n_head_kv, batch), dim3(256), 0, st, q, ck, cv, \
+                               sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride, *fuse);  \
+        else                                                                                                    \
+            hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, false>), dim3(n_head_kv, batch), dim3(256), 0, st, q, ck, cv, \
+                               sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride, AttnFuse()); \
         report("attention");                                                                                    \
         return;                                                                                                 \
     }
@@ -727,6 +792,37 @@ void launch_rope_store_kv_batch(float* q, float* k, const float* v, int8_t* kv_k
 {
     launch_rope_kv<3>(q, k, v, kv_k, kv_v, scale_k, scale_v, positions, 0, head_dim, n_head, n_head_kv, q_stride,
                       k_stride, theta, batch_size, stream);
+}
+
+// Extension of the reference's launch layer: RoPE (Q and K) + INT8 KV store + attention in ONE
+// launch, for B >= 1.  positions: device array [batch] (NULL: every sequence is at `position`).
+// Shapes without a specialised kernel run the separate launches.  q is left unrotated.
+void launch_rope_store_attention(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v, float* scale_k,
+                                 float* scale_v, int16_t* output, const int* positions, int position, int n_head,
+                                 int n_head_kv, int head_dim, float theta, float scale, int batch_size, int kv_stride,
+                                 hipStream_t stream)
+{
+    // Fusing pays when every workgroup stores its own cache slot: one sequence, or per-sequence
+    // caches.  Lock-step copies on a shared cache (kv_stride = 0, batch > 1) would store the same
+    // slot from every workgroup, so they keep the separate store launch.
+    if (attn_has_fast(n_head, n_head_kv, head_dim) && (batch_size == 1 || kv_stride != 0)) {
+        AttnFuse fz;
+        fz.k_new = k;
+        fz.v_new = v;
+        fz.ck_w = kv_k;
+        fz.cv_w = kv_v;
+        fz.sk_w = scale_k;
+        fz.sv_w = scale_v;
+        fz.freqs = rope_table(head_dim, theta);
+        if (!fz.freqs) { t12_set_error("rope: cannot build the frequency table"); return; }
+        launch_attn(q, kv_k, kv_v, scale_k, scale_v, output, positions, position + 1, n_head, n_head_kv, head_dim,
+                    scale, batch_size, (size_t)kv_stride, stream, &fz);
+        return;
+    }
+    launch_rope_kv<3>(q, k, v, kv_k, kv_v, scale_k, scale_v, positions, position, head_dim, n_head, n_head_kv,
+                      n_head * head_dim, n_head_kv * head_dim, theta, batch_size, stream);
+    launch_attn(q, kv_k, kv_v, scale_k, scale_v, output, positions, position + 1, n_head, n_head_kv, head_dim, scale,
+                batch_size, (size_t)kv_stride, stream);
 }
 
 void launch_attention_all_heads(const float* q, const int8_t* k_cache, const int8_t* v_cache, const float* scale_k,
