@@ -40,7 +40,7 @@ namespace {
 
 constexpr int KC = 64;          // K columns staged per pipeline stage
 constexpr int TM = 128;         // weight rows per workgroup
-constexpr int PCAP = 4096;      // escape entries a workgroup can stage in LDS
+constexpr int PCAP = 2048;      // escape entries a workgroup can stage in LDS
 constexpr int PATCH_BYTES = PCAP * 4 + (TM + 1) * 4 + 12;
 constexpr int NO_ESCAPE = 0x7FFFFFFF;
 
@@ -58,6 +58,12 @@ struct GemmParams {
     float* ws;                             // [ksplit][B][m_total] partial sums when ksplit > 1
 };
 
+// LDS slot of (unit, row) in a [units][rows] array of 16-byte units.  Rows are rotated
+// inside their aligned block of eight by the unit index, so that both access patterns are
+// bank-conflict free: the staging writes (neighbouring lanes = the units of one row) and
+// the fragment reads (neighbouring lanes = consecutive rows of one unit).
+__device__ __forceinline__ int lds_slot(int u, int r, int rows) { return u * rows + (r & ~7) + ((r + u) & 7); }
+
 __device__ __forceinline__ int find_segment(const GemmParams& p, int tile)
 {
     int s = 0;
@@ -68,26 +74,24 @@ __device__ __forceinline__ int find_segment(const GemmParams& p, int tile)
 }
 
 // ---------------------------------------------------------------------------
-// LDS stage layout (one of two buffers):
-//   act  [8 units][TB rows] x 16 B   unit u = (k % 64) / 8, eight bf16 paired by
-//                                     t12_pair_acts
-//   sm   [4 units][TM rows] x 16 B   unit c = (k % 64) / 16
-//   gr   [4 units][TM rows] x  8 B
-// Consecutive lanes read consecutive rows of one unit: conflict free.
-// One 32-column block q of a stage feeds two MFMA k-steps s = 0, 1; MFMA slot
-// (half h of the wave, element j) stands for column 32q + 16h + 8s + j.
+// LDS stage layout (one of two buffers), unit u = (k % 64) / 8 = eight bf16 of one row,
+// paired (i, i + 4) per dword the way t12_decode8 / t12_pair_acts order them:
+//   act  [8 units][TB rows] x 16 B
+//   w    [8 units][TM rows] x 16 B     decoded weights
+// MFMA k-step t of a stage covers columns 16t .. 16t+15; the lanes of wave half h take
+// unit 2t + h of their row, for both operands.
 // ---------------------------------------------------------------------------
 // DBG (benchmark probes, 0 in production): bit 0 skips the MFMAs, bit 1 skips the global->LDS
-// staging inside the loop, bit 2 skips the barrier per stage.
-template <int WB, int WM, int FB, int FM, int DBG = 0>
-__global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
+// staging inside the loop, bit 3 skips the escapes.
+template <int WB, int WM, int FB, int FM, int DBG>
+__device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
 {
     constexpr int TB = WB * FB * 32;                  // batch rows per workgroup
     static_assert(WB * WM == 4, "four waves per workgroup");
     static_assert(WM * FM * 32 == TM, "row tile is 128");
     constexpr int ACT_UNITS = TB * 8;                 // 16-byte units per stage
     constexpr int ACT_LD = ACT_UNITS / 256;           // per thread
-    constexpr int STAGE_BYTES = ACT_UNITS * 16 + TM * 64 + TM * 32;
+    constexpr int STAGE_BYTES = ACT_UNITS * 16 + TM * 128;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -106,9 +110,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
     const uint32_t be2 = t12_opaque(((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23));
 
     // ---- this thread's share of the global -> LDS staging
-    //  acts: unit idx = tid + 256*i -> row idx / 8, unit idx % 8 (8 lanes = 128 contiguous bytes)
-    //  sm / gr: unit idx = tid + 256*i (i < 2) -> row idx / 4, unit idx % 4
-    // batch rows >= B are clamped to row B-1: their products are computed and never stored
+    //  acts:   item idx = tid + 256*i -> batch row idx / 8, unit idx % 8 (8 lanes = 128 contiguous bytes)
+    //  planes: item idx = tid + 256*i (i < 2) -> weight row idx / 4, 16 columns c = idx % 4
+    //          (16 sm bytes + 8 gr bytes -> two decoded units 2c, 2c + 1)
+    // rows past the end are clamped: their products are computed and never stored
     const uint16_t* a_src[ACT_LD];
     int a_dst[ACT_LD];
 #pragma unroll
@@ -116,25 +121,25 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
         const int idx = tid + 256 * i;
         const int r = idx >> 3, u = idx & 7;
         a_src[i] = p.act + (size_t)min(b0 + r, B - 1) * p.act_stride + k_begin + u * 8;
-        a_dst[i] = (u * TB + r) * 16;
+        a_dst[i] = lds_slot(u, r, TB) * 16;
     }
+    const int wc = tid & 3;                       // the same 16-column group for both items
     const uint8_t* s_src[2];
     const uint8_t* g_src[2];
-    int s_dst[2], g_dst[2];
+    int w_dst[2][2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-        const int idx = tid + 256 * i;
-        const int r = idx >> 2, c = idx & 3;
-        const size_t e = (size_t)min(m0 + r, M - 1) * K + k_begin;      // clamp: loads stay in bounds
-        s_src[i] = sg.sm + e + c * 16;
-        g_src[i] = sg.gr + (e >> 1) + c * 8;
-        s_dst[i] = ACT_UNITS * 16 + (c * TM + r) * 16;
-        g_dst[i] = ACT_UNITS * 16 + TM * 64 + (c * TM + r) * 8;
+        const int r = (tid + 256 * i) >> 2;
+        const size_t e = (size_t)min(m0 + r, M - 1) * K + k_begin;
+        s_src[i] = sg.sm + e + wc * 16;
+        g_src[i] = sg.gr + (e >> 1) + wc * 8;
+        w_dst[i][0] = ACT_UNITS * 16 + lds_slot(2 * wc, r, TM) * 16;
+        w_dst[i][1] = ACT_UNITS * 16 + lds_slot(2 * wc + 1, r, TM) * 16;
     }
 
     // Register ring: the global loads of stage st + D are issued while stage st is
-    // being multiplied (HBM latency is longer than one stage of MFMAs); a stage moves
-    // registers -> LDS one iteration before it is consumed (double-buffered LDS).
+    // being multiplied (HBM latency is longer than one stage of MFMAs); a stage is decoded
+    // and moved registers -> LDS one iteration before it is consumed (double-buffered LDS).
     constexpr int D = 3;
     uint4 ra[D][ACT_LD];
     uint4 rs[D][2];
@@ -154,8 +159,11 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
         _Pragma("unroll") for (int i = 0; i < ACT_LD; i++)                                          \
             *(uint4*)(base_ + a_dst[i]) = t12_pair_acts(ra[slot][i]);                               \
         _Pragma("unroll") for (int i = 0; i < 2; i++) {                                             \
-            *(uint4*)(base_ + s_dst[i]) = rs[slot][i];                                              \
-            *(uint2*)(base_ + g_dst[i]) = rg[slot][i];                                              \
+            uint32_t w_[2][4];                                                                      \
+            t12_decode8(rs[slot][i].x, rs[slot][i].y, rg[slot][i].x, be2, w_[0]);                   \
+            t12_decode8(rs[slot][i].z, rs[slot][i].w, rg[slot][i].y, be2, w_[1]);                   \
+            *(uint4*)(base_ + w_dst[i][0]) = make_uint4(w_[0][0], w_[0][1], w_[0][2], w_[0][3]);    \
+            *(uint4*)(base_ + w_dst[i][1]) = make_uint4(w_[1][0], w_[1][1], w_[1][2], w_[1][3]);    \
         }                                                                                           \
     }
 
@@ -169,12 +177,12 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
 
     // ---- escape list of this workgroup's rows -> LDS.  The rows are consecutive, so
     //      their entries are one contiguous slice [e0, e1) of cols[] / correct[].
-    //      esc_mode: 0 none, 1 staged (exact, in registers), 2 too many for LDS
-    //      (or K > 65536): streamed wrong values + correction in the epilogue.
+    //      esc_mode: 0 none, 1 staged (exact values written over the decoded ones in LDS),
+    //      2 too many for LDS (or K > 65536): wrong values multiplied, corrected in the epilogue.
     uint32_t* lpat = (uint32_t*)(lds + 2 * STAGE_BYTES);       // col | correct << 16
     int* lrow = (int*)(lpat + PCAP);                           // [TM + 1] offsets into lpat
     int esc_mode = 0;
-    if (sg.row_off) {
+    if (sg.row_off && !(DBG & 8)) {
         const int e0 = sg.row_off[min(m0, M)], e1 = sg.row_off[min(m0 + TM, M)];
         esc_mode = (e1 - e0 <= PCAP && K <= 65536) ? 1 : 2;
         if (esc_mode == 1) {
@@ -183,108 +191,82 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
             for (int t = tid; t <= TM; t += 256) lrow[t] = sg.row_off[min(m0 + t, M)] - e0;
         }
     }
-    // per lane: cursor into its rows' slices (FM rows), next escape column and its exact value
-    int pp[FM], pe[FM], nc[FM];
-    uint32_t cv[FM];
-#pragma unroll
-    for (int j = 0; j < FM; j++) { pp[j] = pe[j] = 0; nc[j] = NO_ESCAPE; cv[j] = 0; }
+    // Per staging item: cursor into its row's slice and the column of the next entry.  The
+    // thread that decoded 16 columns of a row into LDS also overwrites the escapes among them
+    // there (same wave, LDS executes its writes in order: no barrier needed in between).
+    int pp[2] = {0, 0}, pe[2] = {0, 0}, nc[2] = {NO_ESCAPE, NO_ESCAPE};
+#define T12_PATCH_STAGE(buf, kabs)                                                                  \
+    if (esc_mode == 1) {                                                                            \
+        uint8_t* base_ = lds + (buf) * STAGE_BYTES + ACT_UNITS * 16;                                \
+        _Pragma("unroll") for (int i = 0; i < 2; i++) {                                             \
+            while (nc[i] < (kabs) + KC) {                                                           \
+                const int e_ = nc[i] - (kabs) - 16 * wc;            /* 0..15: one of this item's */ \
+                if ((unsigned)e_ < 16u) {                                                           \
+                    const int r_ = (tid + 256 * i) >> 2;                                            \
+                    const int off_ = lds_slot(2 * wc + (e_ >> 3), r_, TM) * 16 + (e_ & 3) * 4 + ((e_ >> 2) & 1) * 2; \
+                    *(uint16_t*)(base_ + off_) = (uint16_t)(lpat[pp[i]] >> 16);                     \
+                }                                                                                   \
+                pp[i]++;                                                                            \
+                nc[i] = pp[i] < pe[i] ? (int)(lpat[pp[i]] & 0xFFFFu) : NO_ESCAPE;                   \
+            }                                                                                       \
+        }                                                                                           \
+    }
 
-    // One stage = 64 columns = 4 MFMA k-steps t = 0..3 (block q = t / 2, step ks = t % 2).
-    // Fragment loads run one k-step ahead of the MFMAs that use them, and the decode of
-    // block q = 1 is placed under the MFMAs of block q = 0.
-    auto load_w = [&](const uint4* lsm, const uint2* lgr, int q, uint4 (&S)[FM], uint2 (&G)[FM]) {
+    auto load_frags = [&](const uint4* lact, const uint4* lw, int t, uint4 (&A)[FB], uint4 (&W)[FM]) {
 #pragma unroll
-        for (int j = 0; j < FM; j++) {
-            const int row = (wm * FM + j) * 32 + ln;
-            S[j] = lsm[(2 * q + lh) * TM + row];
-            G[j] = lgr[(2 * q + lh) * TM + row];
-        }
+        for (int i = 0; i < FB; i++) A[i] = lact[lds_slot(2 * t + lh, (wb * FB + i) * 32 + ln, TB)];
+#pragma unroll
+        for (int j = 0; j < FM; j++) W[j] = lw[lds_slot(2 * t + lh, (wm * FM + j) * 32 + ln, TM)];
     };
-    auto decode_w = [&](const uint4 (&S)[FM], const uint2 (&G)[FM], int kq, uint32_t (&wf)[FM][2][4]) {
-#pragma unroll
-        for (int j = 0; j < FM; j++) {
-            t12_decode8(S[j].x, S[j].y, G[j].x, be2, wf[j][0]);
-            t12_decode8(S[j].z, S[j].w, G[j].y, be2, wf[j][1]);
-            // exact escapes: columns [kq, kq + 32) of this row; this lane owns the 16 of its half
-            while (nc[j] < kq + 32) {
-                const int e = nc[j] - kq;
-                if ((e >> 4) == lh) {
-                    const int i8 = e & 7, kst = (e >> 3) & 1;
-                    const uint32_t keep = (i8 >> 2) ? 0x0000FFFFu : 0xFFFF0000u;
-                    const uint32_t ins = (i8 >> 2) ? (cv[j] << 16) : cv[j];
-#pragma unroll
-                    for (int a = 0; a < 2; a++)
-#pragma unroll
-                        for (int r = 0; r < 4; r++)
-                            if (a == kst && r == (i8 & 3)) wf[j][a][r] = (wf[j][a][r] & keep) | ins;
-                }
-                pp[j]++;
-                const uint32_t ent = pp[j] < pe[j] ? lpat[pp[j]] : (uint32_t)NO_ESCAPE;
-                nc[j] = pp[j] < pe[j] ? (int)(ent & 0xFFFFu) : NO_ESCAPE;
-                cv[j] = ent >> 16;
-            }
-        }
-    };
-    auto load_a = [&](const uint4* lact, int t, uint4 (&A)[FB]) {
-#pragma unroll
-        for (int i = 0; i < FB; i++) A[i] = lact[(4 * (t >> 1) + 2 * lh + (t & 1)) * TB + (wb * FB + i) * 32 + ln];
-    };
-    auto mma = [&](const uint4 (&A)[FB], const uint32_t (&wf)[FM][2][4], int ks) {
+    auto mma = [&](const uint4 (&A)[FB], const uint4 (&W)[FM]) {
 #pragma unroll
         for (int i = 0; i < FB; i++) {
-            const t12_bf16x8 av = __builtin_bit_cast(t12_bf16x8, A[i]);
 #pragma unroll
             for (int j = 0; j < FM; j++) {
-                const uint4 Wv = make_uint4(wf[j][ks][0], wf[j][ks][1], wf[j][ks][2], wf[j][ks][3]);
-                if (DBG & 1) acc[i][j][0] += __builtin_bit_cast(float, A[i].x ^ Wv.x ^ Wv.y ^ Wv.z ^ Wv.w);
+                if (DBG & 1) acc[i][j][0] += __builtin_bit_cast(float, A[i].x ^ W[j].x ^ W[j].y ^ W[j].z ^ W[j].w);
                 else
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(t12_bf16x8, Wv),
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(t12_bf16x8, A[i]),
+                                                                        __builtin_bit_cast(t12_bf16x8, W[j]),
                                                                         acc[i][j], 0, 0, 0);
             }
         }
     };
-    auto compute_stage = [&](int buf, int kabs) {
+    // one stage = 64 columns = 4 MFMA k-steps; fragment loads run one k-step ahead
+    auto compute_stage = [&](int buf) {
         const uint8_t* base = lds + buf * STAGE_BYTES;
         const uint4* lact = (const uint4*)base;
-        const uint4* lsm = (const uint4*)(base + ACT_UNITS * 16);
-        const uint2* lgr = (const uint2*)(base + ACT_UNITS * 16 + TM * 64);
-        uint4 S0[FM], S1[FM], A0[FB], A1[FB];
-        uint2 G0[FM], G1[FM];
-        uint32_t w0[FM][2][4], w1[FM][2][4];
-        load_w(lsm, lgr, 0, S0, G0);
-        load_a(lact, 0, A0);
-        load_w(lsm, lgr, 1, S1, G1);
-        decode_w(S0, G0, kabs, w0);
-        load_a(lact, 1, A1);
-        mma(A0, w0, 0);                 // t = 0
-        decode_w(S1, G1, kabs + 32, w1);
-        load_a(lact, 2, A0);
-        mma(A1, w0, 1);                 // t = 1
-        load_a(lact, 3, A1);
-        mma(A0, w1, 0);                 // t = 2
-        mma(A1, w1, 1);                 // t = 3
+        const uint4* lw = (const uint4*)(base + ACT_UNITS * 16);
+        uint4 A0[FB], A1[FB], W0[FM], W1[FM];
+        load_frags(lact, lw, 0, A0, W0);
+        load_frags(lact, lw, 1, A1, W1);
+        mma(A0, W0);
+        load_frags(lact, lw, 2, A0, W0);
+        mma(A1, W1);
+        load_frags(lact, lw, 3, A1, W1);
+        mma(A0, W0);
+        mma(A1, W1);
     };
 
-    // prologue: stages 0..D-1 in flight, stage 0 into LDS
+    // prologue: stages 0..D-1 in flight, escape list visible, stage 0 into LDS
 #pragma unroll
     for (int d = 0; d < D; d++)
         if (d < nstage) T12_LOAD_STAGE(d, d)
-    if (nstage > 0) T12_STORE_STAGE(0, 0)
     __syncthreads();
     if (esc_mode == 1) {
 #pragma unroll
-        for (int j = 0; j < FM; j++) {
-            const int r = (wm * FM + j) * 32 + ln;
-            pp[j] = lrow[r];
-            pe[j] = lrow[r + 1];
-            while (pp[j] < pe[j] && (int)(lpat[pp[j]] & 0xFFFFu) < k_begin) pp[j]++;   // K split: skip earlier columns
-            if (pp[j] < pe[j]) {
-                const uint32_t ent = lpat[pp[j]];
-                nc[j] = (int)(ent & 0xFFFFu);
-                cv[j] = ent >> 16;
-            }
+        for (int i = 0; i < 2; i++) {
+            const int r = (tid + 256 * i) >> 2;
+            pp[i] = lrow[r];
+            pe[i] = lrow[r + 1];
+            while (pp[i] < pe[i] && (int)(lpat[pp[i]] & 0xFFFFu) < k_begin) pp[i]++;   // K split: skip earlier columns
+            if (pp[i] < pe[i]) nc[i] = (int)(lpat[pp[i]] & 0xFFFFu);
         }
     }
+    if (nstage > 0) {
+        T12_STORE_STAGE(0, 0)
+        T12_PATCH_STAGE(0, k_begin)
+    }
+    __syncthreads();
 
     int st = 0;
     // steady state, unrolled by D so that ring slots are compile-time; no guards inside
@@ -292,9 +274,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
 #pragma unroll
         for (int d = 0; d < D; d++) {
             if (!(DBG & 2)) T12_LOAD_STAGE(d, st + d + D)    // slot d held stage st + d: already in LDS
-            compute_stage((st + d) & 1, k_begin + (st + d) * KC);
+            compute_stage((st + d) & 1);
             if (!(DBG & 2)) T12_STORE_STAGE((d + 1) % D, (st + d + 1) & 1)
-            if (!(DBG & 4)) __syncthreads();
+            T12_PATCH_STAGE((st + d + 1) & 1, k_begin + (st + d + 1) * KC)
+            __syncthreads();
         }
     }
     // drain
@@ -303,14 +286,18 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
         for (int d = 0; d < D; d++) {
             if (st + d < nstage) {
                 if (st + d + D < nstage) T12_LOAD_STAGE(d, st + d + D)
-                compute_stage((st + d) & 1, k_begin + (st + d) * KC);
-                if (st + d + 1 < nstage) T12_STORE_STAGE((d + 1) % D, (st + d + 1) & 1)
+                compute_stage((st + d) & 1);
+                if (st + d + 1 < nstage) {
+                    T12_STORE_STAGE((d + 1) % D, (st + d + 1) & 1)
+                    T12_PATCH_STAGE((st + d + 1) & 1, k_begin + (st + d + 1) * KC)
+                }
                 __syncthreads();
             }
         }
     }
 #undef T12_LOAD_STAGE
 #undef T12_STORE_STAGE
+#undef T12_PATCH_STAGE
 
     // ---- overflow path only (more escapes than the LDS list holds): the streamed value of an
     //      escape was its "wrong" decode, so acc[b, m] += (correct - wrong) * X[b, col], added by
@@ -362,6 +349,20 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
                 if (m < M && b < B) dst[(size_t)b * ld + col_off + m] = acc[i][j][r];
             }
         }
+}
+
+// One workgroup per CU (batch tile 256: 128 accumulator registers + the load ring) ...
+template <int WB, int WM, int FB, int FM, int DBG = 0>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
+{
+    gemm_mfma_body<WB, WM, FB, FM, DBG>(p);
+}
+// ... or two (batch tiles <= 128): at most 256 registers per lane, so that two waves share a SIMD
+// and one wave's decode / LDS traffic runs under the other's MFMAs.
+template <int WB, int WM, int FB, int FM, int DBG = 0>
+__global__ __launch_bounds__(256, 2) void gemm_mfma_kernel_occ2(const GemmParams p)
+{
+    gemm_mfma_body<WB, WM, FB, FM, DBG>(p);
 }
 
 // ---------------------------------------------------------------------------
@@ -449,13 +450,13 @@ int g_gemm_ksplit = 0;   // 0 = choose by shape
 
 int g_gemm_dbg = 0;
 
-template <int WB, int WM, int FB, int FM, int DBG = 0>
+template <int WB, int WM, int FB, int FM, int DBG = 0, bool OCC2 = false>
 int launch_mfma(GemmParams& p, int tiles, hipStream_t st)
 {
     constexpr int TB = WB * FB * 32;
-    constexpr int STAGE_BYTES = TB * 8 * 16 + TM * 64 + TM * 32;
-    const dim3 grid(tiles, (p.B + TB - 1) / TB, p.ksplit);
-    auto kfn = gemm_mfma_kernel<WB, WM, FB, FM, DBG>;
+    constexpr int STAGE_BYTES = TB * 8 * 16 + TM * 128;
+    const dim3 grid(tiles, (p.B + TB - 1) / TB, p.ksplit);   // batch tiles of one row tile are neighbours in time
+    auto kfn = OCC2 ? gemm_mfma_kernel_occ2<WB, WM, FB, FM, DBG> : gemm_mfma_kernel<WB, WM, FB, FM, DBG>;
     static bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -544,8 +545,9 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
     p.blk_start[nseg] = tiles;
     // K split: fill the chip.  A 256-row batch tile needs a whole CU (LDS, accumulators);
     // smaller batch tiles fit 2-4 workgroups per CU.  Every split keeps >= 4 stages.
-    const int btiles = (B + 255) / 256;
-    const int per_cu = B > 128 ? 1 : (B > 64 ? 2 : 4);
+    const bool big = B > 128 && !(g_gemm_dbg & 64);
+    const int btiles = big ? (B + 255) / 256 : (B + 127) / 128;
+    const int per_cu = big ? 1 : (B > 64 ? 2 : 4);
     const int want = 256 * per_cu;
     int ks = 1;
     if (g_gemm_ksplit > 0) ks = g_gemm_ksplit;
@@ -564,13 +566,20 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
         }
     }
     int rc;
-    if (B <= 32) rc = launch_mfma<1, 4, 1, 1>(p, tiles, st);
-    else if (B <= 64) rc = launch_mfma<1, 4, 2, 1>(p, tiles, st);
-    else if (B <= 128) rc = launch_mfma<1, 4, 4, 1>(p, tiles, st);
+    if (B <= 32) rc = launch_mfma<1, 4, 1, 1, 0, true>(p, tiles, st);
+    else if (B <= 64) rc = launch_mfma<1, 4, 2, 1, 0, true>(p, tiles, st);
+    else if (B <= 128 || (g_gemm_dbg & 64)) {
+        if ((g_gemm_dbg & 63) == 0) rc = launch_mfma<1, 4, 4, 1, 0, true>(p, tiles, st);
+        else if ((g_gemm_dbg & 63) == 1) rc = launch_mfma<1, 4, 4, 1, 1, true>(p, tiles, st);
+        else if ((g_gemm_dbg & 63) == 2) rc = launch_mfma<1, 4, 4, 1, 2, true>(p, tiles, st);
+        else if ((g_gemm_dbg & 63) == 8) rc = launch_mfma<1, 4, 4, 1, 8, true>(p, tiles, st);
+        else if ((g_gemm_dbg & 63) == 16) rc = launch_mfma<1, 4, 4, 1, 0, false>(p, tiles, st);
+        else rc = launch_mfma<1, 4, 4, 1, 10, true>(p, tiles, st);
+    }
     else if (g_gemm_dbg == 1) rc = launch_mfma<2, 2, 4, 2, 1>(p, tiles, st);
     else if (g_gemm_dbg == 2) rc = launch_mfma<2, 2, 4, 2, 2>(p, tiles, st);
-    else if (g_gemm_dbg == 3) rc = launch_mfma<2, 2, 4, 2, 3>(p, tiles, st);
-    else if (g_gemm_dbg == 6) rc = launch_mfma<2, 2, 4, 2, 6>(p, tiles, st);
+    else if (g_gemm_dbg == 8) rc = launch_mfma<2, 2, 4, 2, 8>(p, tiles, st);
+    else if (g_gemm_dbg == 10) rc = launch_mfma<2, 2, 4, 2, 10>(p, tiles, st);
     else rc = launch_mfma<2, 2, 4, 2>(p, tiles, st);
     if (rc) return rc;
 
