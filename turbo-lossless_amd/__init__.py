@@ -52,7 +52,6 @@ _SIGS = {
     "t12_fill_f32": (_i, [_vp, C.c_size_t, C.c_float, _vp]),
     # glue launchers (reference names; void return)
     "t12_tune_attention": (_i, [_i]),
-    "t12_debug_gemm": (_i, [_i]),
     "launch_rope_init": (None, [_i, C.c_float]),
     "launch_embed_lookup": (None, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "launch_rms_norm_bf16_batch": (None, [_vp, _vp, _vp, _i, C.c_float, _i, _vp]),

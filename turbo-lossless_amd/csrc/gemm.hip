@@ -64,6 +64,17 @@ struct GemmParams {
 // the fragment reads (neighbouring lanes = consecutive rows of one unit).
 __device__ __forceinline__ int lds_slot(int u, int r, int rows) { return u * rows + (r & ~7) + ((r + u) & 7); }
 
+// Order in which a thread's staging units are stored: the ndec decode units (18 VALU each) evenly
+// among the nact activation units (4 VALU each).  Position pos -> unit index (activation units
+// 0 .. nact-1, decode units nact .. nact+ndec-1).
+__device__ __forceinline__ constexpr int stage_unit_order(int pos, int nact, int ndec)
+{
+    const int nu = nact + ndec;
+    const int dec_before = pos * ndec / nu;              // decode units placed before pos
+    const bool is_dec = (pos + 1) * ndec / nu > dec_before;
+    return is_dec ? nact + dec_before : pos - dec_before;
+}
+
 __device__ __forceinline__ int find_segment(const GemmParams& p, int tile)
 {
     int s = 0;
@@ -80,17 +91,31 @@ __device__ __forceinline__ int find_segment(const GemmParams& p, int tile)
 //   w    [8 units][TM rows] x 16 B     decoded weights
 // MFMA k-step t of a stage covers columns 16t .. 16t+15; the lanes of wave half h take
 // unit 2t + h of their row, for both operands.
+//
+// Global loads.  A stage is 64 columns: 128 B of an activation row (one cache line) but
+// only 64 B of a row's sm plane and 32 B of its gr plane.  Fetching those a stage at a
+// time asks HBM for every line twice or more (the rows of a tile are K bytes apart, a
+// power of two: they fall into a handful of L2 sets and are evicted before the next
+// stage comes back for the other half).  So weights are loaded per WINDOW of two stages
+// (128 columns), both halves of a line in back-to-back instructions:
+//   piece X (used by the even stage): lanes c8 < 4 take row rr, columns 16*c8 ..;
+//                                     lanes c8 >= 4 take row 64 + (rr^1), columns 16*(c8-4) ..
+//   piece Y (used by the odd stage) : the other halves of the same two lines, lanes swapped
+// where c8 = tid % 8, rr = item / 8 in 0..63.  Every lane decodes one piece per item and
+// stage (balanced), every sm line is requested whole within two instructions, and the
+// rr^1 keeps the LDS writes of the two lane groups on different banks.
 // ---------------------------------------------------------------------------
-// DBG (benchmark probes, 0 in production): bit 0 skips the MFMAs, bit 1 skips the global->LDS
-// staging inside the loop, bit 3 skips the escapes.
-template <int WB, int WM, int FB, int FM, int DBG>
+template <int WB, int WM, int FB, int FM>
 __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
 {
     constexpr int TB = WB * FB * 32;                  // batch rows per workgroup
-    static_assert(WB * WM == 4, "four waves per workgroup");
+    constexpr int NT = WB * WM * 64;                  // threads per workgroup
+    static_assert(NT == 256 || NT == 512, "four or eight waves per workgroup");
     static_assert(WM * FM * 32 == TM, "row tile is 128");
     constexpr int ACT_UNITS = TB * 8;                 // 16-byte units per stage
-    constexpr int ACT_LD = ACT_UNITS / 256;           // per thread
+    constexpr int ACT_LD = ACT_UNITS / NT;            // per thread
+    constexpr int W_LD = TM * 4 / NT;                 // 16-column weight pieces per thread and stage
+    static_assert(ACT_LD >= 1 && ACT_LD * NT == ACT_UNITS, "activation tile divides over the threads");
     constexpr int STAGE_BYTES = ACT_UNITS * 16 + TM * 128;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -110,62 +135,71 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
     const uint32_t be2 = t12_opaque(((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23));
 
     // ---- this thread's share of the global -> LDS staging
-    //  acts:   item idx = tid + 256*i -> batch row idx / 8, unit idx % 8 (8 lanes = 128 contiguous bytes)
-    //  planes: item idx = tid + 256*i (i < 2) -> weight row idx / 4, 16 columns c = idx % 4
-    //          (16 sm bytes + 8 gr bytes -> two decoded units 2c, 2c + 1)
+    //  acts: item idx = tid + NT*i -> batch row idx / 8, unit idx % 8 (8 lanes = 128 contiguous bytes)
     // rows past the end are clamped: their products are computed and never stored
     const uint16_t* a_src[ACT_LD];
     int a_dst[ACT_LD];
 #pragma unroll
     for (int i = 0; i < ACT_LD; i++) {
-        const int idx = tid + 256 * i;
+        const int idx = tid + NT * i;
         const int r = idx >> 3, u = idx & 7;
         a_src[i] = p.act + (size_t)min(b0 + r, B - 1) * p.act_stride + k_begin + u * 8;
         a_dst[i] = lds_slot(u, r, TB) * 16;
     }
-    const int wc = tid & 3;                       // the same 16-column group for both items
-    const uint8_t* s_src[2];
-    const uint8_t* g_src[2];
-    int w_dst[2][2];
+    //  weights: pieces X / Y of item i (see above); [0] = X, [1] = Y
+    const int c8 = tid & 7, hi = c8 >> 2, cc = c8 & 3;
+    const uint8_t* s_src[2][W_LD];
+    const uint8_t* g_src[2][W_LD];
+    int w_row[2][W_LD];
+    int w_dst[2][W_LD][2];
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int r = (tid + 256 * i) >> 2;
-        const size_t e = (size_t)min(m0 + r, M - 1) * K + k_begin;
-        s_src[i] = sg.sm + e + wc * 16;
-        g_src[i] = sg.gr + (e >> 1) + wc * 8;
-        w_dst[i][0] = ACT_UNITS * 16 + lds_slot(2 * wc, r, TM) * 16;
-        w_dst[i][1] = ACT_UNITS * 16 + lds_slot(2 * wc + 1, r, TM) * 16;
+    for (int i = 0; i < W_LD; i++) {
+        const int rr = (tid + NT * i) >> 3;                   // 0..63
+        const int r_lo = rr, r_hi = 64 + (rr ^ 1);
+#pragma unroll
+        for (int y = 0; y < 2; y++) {
+            const int r = (hi ^ y) ? r_hi : r_lo;
+            const size_t e = (size_t)min(m0 + r, M - 1) * K + k_begin + 64 * y + 16 * cc;
+            w_row[y][i] = r;
+            s_src[y][i] = sg.sm + e;
+            g_src[y][i] = sg.gr + (e >> 1);
+            w_dst[y][i][0] = ACT_UNITS * 16 + lds_slot(2 * cc, r, TM) * 16;
+            w_dst[y][i][1] = ACT_UNITS * 16 + lds_slot(2 * cc + 1, r, TM) * 16;
+        }
     }
 
-    // Register ring: the global loads of stage st + D are issued while stage st is
-    // being multiplied (HBM latency is longer than one stage of MFMAs); a stage is decoded
-    // and moved registers -> LDS one iteration before it is consumed (double-buffered LDS).
-    constexpr int D = 3;
-    uint4 ra[D][ACT_LD];
-    uint4 rs[D][2];
-    uint2 rg[D][2];
-#define T12_LOAD_STAGE(slot, st)                                                        \
-    {                                                                                   \
-        _Pragma("unroll") for (int i = 0; i < ACT_LD; i++)                              \
-            ra[slot][i] = *(const uint4*)(a_src[i] + (size_t)(st) * KC);                \
-        _Pragma("unroll") for (int i = 0; i < 2; i++) {                                 \
-            rs[slot][i] = t12_ldg_stream16(s_src[i] + (size_t)(st) * KC);               \
-            rg[slot][i] = t12_ldg_stream8(g_src[i] + (size_t)(st) * (KC / 2));          \
-        }                                                                               \
-    }
-#define T12_STORE_STAGE(slot, buf)                                                                  \
-    {                                                                                               \
-        uint8_t* base_ = lds + (buf) * STAGE_BYTES;                                                 \
-        _Pragma("unroll") for (int i = 0; i < ACT_LD; i++)                                          \
-            *(uint4*)(base_ + a_dst[i]) = t12_pair_acts(ra[slot][i]);                               \
-        _Pragma("unroll") for (int i = 0; i < 2; i++) {                                             \
-            uint32_t w_[2][4];                                                                      \
-            t12_decode8(rs[slot][i].x, rs[slot][i].y, rg[slot][i].x, be2, w_[0]);                   \
-            t12_decode8(rs[slot][i].z, rs[slot][i].w, rg[slot][i].y, be2, w_[1]);                   \
-            *(uint4*)(base_ + w_dst[i][0]) = make_uint4(w_[0][0], w_[0][1], w_[0][2], w_[0][3]);    \
-            *(uint4*)(base_ + w_dst[i][1]) = make_uint4(w_[1][0], w_[1][1], w_[1][2], w_[1][3]);    \
-        }                                                                                           \
-    }
+    // Register rings.  Activations: 4 slots, stage s + 4 is requested while stage s is
+    // multiplied.  Weights: 2 window slots, window w + 2 is requested during the odd stage of
+    // window w, when both of the slot's pieces have been decoded.  A stage is decoded and moved
+    // registers -> LDS one iteration before it is consumed (double-buffered LDS).
+    constexpr int DA = 4;
+    uint4 ra[DA][ACT_LD];
+    uint4 rs[2][2][W_LD];      // [window slot][X / Y][item]
+    uint2 rg[2][2][W_LD];
+    // The staging work of a thread is cut into units so that it can be spread between the
+    // MFMAs of a stage.  Load units: ACT_LD activation pieces, then (odd stages) 4 per item:
+    // sm X, sm Y, gr X, gr Y.  Store units: ACT_LD activation pieces, 2 decode units per item.
+    auto load_act = [&](int slot, int stg, int u) { ra[slot][u] = *(const uint4*)(a_src[u] + (size_t)stg * KC); };
+    auto load_w = [&](int slot, int win, int u, bool do_x, bool do_y) {
+        const int i = u >> 2, y = u & 1;
+        if (y == 0 ? !do_x : !do_y) return;
+        if ((u & 2) == 0) rs[slot][y][i] = *(const uint4*)(s_src[y][i] + (size_t)win * (2 * KC));
+        else rg[slot][y][i] = *(const uint2*)(g_src[y][i] + (size_t)win * KC);
+    };
+    auto store_unit = [&](int aslot, int wslot, int y, int buf, int u) {
+        uint8_t* base_ = lds + buf * STAGE_BYTES;
+        if (u < ACT_LD) {
+            *(uint4*)(base_ + a_dst[u]) = t12_pair_acts(ra[aslot][u]);
+        } else {
+            const int i = (u - ACT_LD) >> 1, h = (u - ACT_LD) & 1;
+            const uint4 sv = rs[wslot][y][i];
+            const uint2 gv = rg[wslot][y][i];
+            uint32_t w_[4];
+            if (h == 0) t12_decode8(sv.x, sv.y, gv.x, be2, w_);
+            else t12_decode8(sv.z, sv.w, gv.y, be2, w_);
+            *(uint4*)(base_ + w_dst[y][i][h]) = make_uint4(w_[0], w_[1], w_[2], w_[3]);
+        }
+    };
 
     t12_f32x16 acc[FB][FM];
 #pragma unroll
@@ -182,122 +216,164 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
     uint32_t* lpat = (uint32_t*)(lds + 2 * STAGE_BYTES);       // col | correct << 16
     int* lrow = (int*)(lpat + PCAP);                           // [TM + 1] offsets into lpat
     int esc_mode = 0;
-    if (sg.row_off && !(DBG & 8)) {
+    if (sg.row_off) {
         const int e0 = sg.row_off[min(m0, M)], e1 = sg.row_off[min(m0 + TM, M)];
         esc_mode = (e1 - e0 <= PCAP && K <= 65536) ? 1 : 2;
         if (esc_mode == 1) {
-            for (int t = tid; t < e1 - e0; t += 256)
+            for (int t = tid; t < e1 - e0; t += NT)
                 lpat[t] = (uint32_t)sg.cols[e0 + t] | ((uint32_t)(uint16_t)sg.correct[e0 + t] << 16);
-            for (int t = tid; t <= TM; t += 256) lrow[t] = sg.row_off[min(m0 + t, M)] - e0;
+            for (int t = tid; t <= TM; t += NT) lrow[t] = sg.row_off[min(m0 + t, M)] - e0;
         }
     }
-    // Per staging item: cursor into its row's slice and the column of the next entry.  The
+    // Per piece kind and item: cursor into its row's slice and the column of the next entry.  The
     // thread that decoded 16 columns of a row into LDS also overwrites the escapes among them
-    // there (same wave, LDS executes its writes in order: no barrier needed in between).
-    int pp[2] = {0, 0}, pe[2] = {0, 0}, nc[2] = {NO_ESCAPE, NO_ESCAPE};
-#define T12_PATCH_STAGE(buf, kabs)                                                                  \
-    if (esc_mode == 1) {                                                                            \
-        uint8_t* base_ = lds + (buf) * STAGE_BYTES + ACT_UNITS * 16;                                \
-        _Pragma("unroll") for (int i = 0; i < 2; i++) {                                             \
-            while (nc[i] < (kabs) + KC) {                                                           \
-                const int e_ = nc[i] - (kabs) - 16 * wc;            /* 0..15: one of this item's */ \
-                if ((unsigned)e_ < 16u) {                                                           \
-                    const int r_ = (tid + 256 * i) >> 2;                                            \
-                    const int off_ = lds_slot(2 * wc + (e_ >> 3), r_, TM) * 16 + (e_ & 3) * 4 + ((e_ >> 2) & 1) * 2; \
-                    *(uint16_t*)(base_ + off_) = (uint16_t)(lpat[pp[i]] >> 16);                     \
-                }                                                                                   \
-                pp[i]++;                                                                            \
-                nc[i] = pp[i] < pe[i] ? (int)(lpat[pp[i]] & 0xFFFFu) : NO_ESCAPE;                   \
-            }                                                                                       \
-        }                                                                                           \
-    }
-
-    auto load_frags = [&](const uint4* lact, const uint4* lw, int t, uint4 (&A)[FB], uint4 (&W)[FM]) {
+    // there (same wave, LDS executes its writes in order: no barrier needed in between).  A
+    // thread owns its X row in even stages and its Y row in odd ones; entries of the stages in
+    // between are stepped over.
+    int pp[2][W_LD], pe[2][W_LD], nc[2][W_LD];
 #pragma unroll
-        for (int i = 0; i < FB; i++) A[i] = lact[lds_slot(2 * t + lh, (wb * FB + i) * 32 + ln, TB)];
+    for (int y = 0; y < 2; y++)
 #pragma unroll
-        for (int j = 0; j < FM; j++) W[j] = lw[lds_slot(2 * t + lh, (wm * FM + j) * 32 + ln, TM)];
-    };
-    auto mma = [&](const uint4 (&A)[FB], const uint4 (&W)[FM]) {
+        for (int i = 0; i < W_LD; i++) { pp[y][i] = pe[y][i] = 0; nc[y][i] = NO_ESCAPE; }
+    auto patch_stage = [&](int y, int buf, int kabs) {
+        if (esc_mode != 1) return;
+        uint8_t* base_ = lds + buf * STAGE_BYTES + ACT_UNITS * 16;
 #pragma unroll
-        for (int i = 0; i < FB; i++) {
-#pragma unroll
-            for (int j = 0; j < FM; j++) {
-                if (DBG & 1) acc[i][j][0] += __builtin_bit_cast(float, A[i].x ^ W[j].x ^ W[j].y ^ W[j].z ^ W[j].w);
-                else
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(t12_bf16x8, A[i]),
-                                                                        __builtin_bit_cast(t12_bf16x8, W[j]),
-                                                                        acc[i][j], 0, 0, 0);
+        for (int i = 0; i < W_LD; i++) {
+            while (nc[y][i] < kabs + KC) {
+                const int e = nc[y][i] - kabs - 16 * cc;            // 0..15: one of this piece's
+                if ((unsigned)e < 16u) {
+                    const int off = lds_slot(2 * cc + (e >> 3), w_row[y][i], TM) * 16 + (e & 3) * 4 + ((e >> 2) & 1) * 2;
+                    *(uint16_t*)(base_ + off) = (uint16_t)(lpat[pp[y][i]] >> 16);
+                }
+                pp[y][i]++;
+                nc[y][i] = pp[y][i] < pe[y][i] ? (int)(lpat[pp[y][i]] & 0xFFFFu) : NO_ESCAPE;
             }
         }
     };
-    // one stage = 64 columns = 4 MFMA k-steps; fragment loads run one k-step ahead
-    auto compute_stage = [&](int buf) {
+
+    // One stage = 64 columns = 4 MFMA k-steps; the fragments of k-step t + 1 are read from LDS
+    // at the start of k-step t.  The staging work for later stages is placed between the MFMAs,
+    // a unit after every few of them, and pinned there with scheduling barriers: whatever is
+    // not issued under a running MFMA is serial time for the wave.
+    //   d = stage number modulo 4 (selects ring slots and LDS buffers at compile time)
+    constexpr int NMMA = 4 * FB * FM;
+    constexpr int NSU = ACT_LD + 2 * W_LD;               // store units per stage
+    constexpr int NLU_ODD = ACT_LD + 4 * W_LD;           // load units of an odd stage
+    constexpr int NCH = NMMA >= 2 * NSU ? NSU : NMMA;    // chunks of staging work per stage
+    auto run_stage = [&](int d, int stg, bool ld_act, bool ld_x, bool ld_y, bool do_store) {
+        const int buf = d & 1;
+        const bool odd = d & 1;
+        const int nlu = odd ? NLU_ODD : ACT_LD;
+        // stage stg + 1: activation slot, weight window slot, piece kind
+        const int n_aslot = (d + 1) & 3, n_wslot = ((d + 1) >> 1) & 1, n_y = (d + 1) & 1, n_buf = (d + 1) & 1;
+        // requests: activations of stage stg + 4 -> slot d; weights of window stg / 2 + 2 -> slot (d >> 1) & 1
+        const int l_wslot = (d >> 1) & 1, l_win = (stg >> 1) + 2;
         const uint8_t* base = lds + buf * STAGE_BYTES;
         const uint4* lact = (const uint4*)base;
         const uint4* lw = (const uint4*)(base + ACT_UNITS * 16);
-        uint4 A0[FB], A1[FB], W0[FM], W1[FM];
-        load_frags(lact, lw, 0, A0, W0);
-        load_frags(lact, lw, 1, A1, W1);
-        mma(A0, W0);
-        load_frags(lact, lw, 2, A0, W0);
-        mma(A1, W1);
-        load_frags(lact, lw, 3, A1, W1);
-        mma(A0, W0);
-        mma(A1, W1);
+        uint4 A[2][FB], W[2][FM];
+        auto load_frags = [&](int t) {
+#pragma unroll
+            for (int i = 0; i < FB; i++) A[t & 1][i] = lact[lds_slot(2 * t + lh, (wb * FB + i) * 32 + ln, TB)];
+#pragma unroll
+            for (int j = 0; j < FM; j++) W[t & 1][j] = lw[lds_slot(2 * t + lh, (wm * FM + j) * 32 + ln, TM)];
+        };
+        load_frags(0);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            if (t < 3) load_frags(t + 1);
+#pragma unroll
+            for (int i = 0; i < FB; i++) {
+#pragma unroll
+                for (int j = 0; j < FM; j++) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(t12_bf16x8, A[t & 1][i]), __builtin_bit_cast(t12_bf16x8, W[t & 1][j]),
+                        acc[i][j], 0, 0, 0);
+                    const int m = (t * FB + i) * FM + j;
+                    // chunk c of the staging work goes after MFMA number (c + 1) * NMMA / NCH - 1
+#pragma unroll
+                    for (int c = 0; c < NCH; c++) {
+                        if ((c + 1) * NMMA / NCH - 1 == m) {
+#pragma unroll
+                            for (int u = 0; u < NLU_ODD; u++) {
+                                if (u < nlu && u * NCH / nlu == c) {
+                                    if (u < ACT_LD) {
+                                        if (ld_act) load_act(d, stg + DA, u);
+                                    } else {
+                                        load_w(l_wslot, l_win, u - ACT_LD, ld_x, ld_y);
+                                    }
+                                }
+                            }
+#pragma unroll
+                            for (int u = 0; u < NSU; u++)
+                                if (do_store && u * NCH / NSU == c)
+                                    store_unit(n_aslot, n_wslot, n_y, n_buf, stage_unit_order(u, ACT_LD, 2 * W_LD));
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                }
+            }
+        }
+        if (do_store) patch_stage(n_y, n_buf, k_begin + (stg + 1) * KC);
+        __syncthreads();
     };
 
-    // prologue: stages 0..D-1 in flight, escape list visible, stage 0 into LDS
+    // prologue: activation stages 0..3 and weight windows 0, 1 in flight, escape list visible,
+    // stage 0 into LDS
 #pragma unroll
-    for (int d = 0; d < D; d++)
-        if (d < nstage) T12_LOAD_STAGE(d, d)
+    for (int d = 0; d < DA; d++)
+        if (d < nstage) {
+#pragma unroll
+            for (int u = 0; u < ACT_LD; u++) load_act(d, d, u);
+        }
+#pragma unroll
+    for (int w = 0; w < 2; w++)
+#pragma unroll
+        for (int u = 0; u < 4 * W_LD; u++) load_w(w, w, u, 2 * w < nstage, 2 * w + 1 < nstage);
     __syncthreads();
     if (esc_mode == 1) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int r = (tid + 256 * i) >> 2;
-            pp[i] = lrow[r];
-            pe[i] = lrow[r + 1];
-            while (pp[i] < pe[i] && (int)(lpat[pp[i]] & 0xFFFFu) < k_begin) pp[i]++;   // K split: skip earlier columns
-            if (pp[i] < pe[i]) nc[i] = (int)(lpat[pp[i]] & 0xFFFFu);
-        }
+        for (int y = 0; y < 2; y++)
+#pragma unroll
+            for (int i = 0; i < W_LD; i++) {
+                const int r = w_row[y][i];
+                int q = lrow[r];
+                const int qe = lrow[r + 1];
+                while (q < qe && (int)(lpat[q] & 0xFFFFu) < k_begin) q++;   // K split: skip earlier columns
+                pp[y][i] = q;
+                pe[y][i] = qe;
+                if (q < qe) nc[y][i] = (int)(lpat[q] & 0xFFFFu);
+            }
     }
+    // All prologue loads have landed before the loop is entered: the compiler's wait-count
+    // bookkeeping then sees only the loop's own loads at the loop head and waits for exactly
+    // the ring slot it needs (with loads pending across the entry edge it drains all of them
+    // once per trip).
+    __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0)
     if (nstage > 0) {
-        T12_STORE_STAGE(0, 0)
-        T12_PATCH_STAGE(0, k_begin)
+#pragma unroll
+        for (int u = 0; u < NSU; u++) store_unit(0, 0, 0, 0, u);
+        patch_stage(0, 0, k_begin);
     }
     __syncthreads();
 
     int st = 0;
-    // steady state, unrolled by D so that ring slots are compile-time; no guards inside
-    for (; st + 2 * D <= nstage; st += D) {
+    // steady state, unrolled by 4 so that ring slots and buffers are compile-time; no guards inside
+    for (; st + 2 * DA <= nstage; st += DA) {
 #pragma unroll
-        for (int d = 0; d < D; d++) {
-            if (!(DBG & 2)) T12_LOAD_STAGE(d, st + d + D)    // slot d held stage st + d: already in LDS
-            compute_stage((st + d) & 1);
-            if (!(DBG & 2)) T12_STORE_STAGE((d + 1) % D, (st + d + 1) & 1)
-            T12_PATCH_STAGE((st + d + 1) & 1, k_begin + (st + d + 1) * KC)
-            __syncthreads();
-        }
+        for (int d = 0; d < DA; d++) run_stage(d, st + d, true, true, true, true);
     }
     // drain
-    for (; st < nstage; st += D) {
+    for (; st < nstage; st += DA) {
 #pragma unroll
-        for (int d = 0; d < D; d++) {
-            if (st + d < nstage) {
-                if (st + d + D < nstage) T12_LOAD_STAGE(d, st + d + D)
-                compute_stage((st + d) & 1);
-                if (st + d + 1 < nstage) {
-                    T12_STORE_STAGE((d + 1) % D, (st + d + 1) & 1)
-                    T12_PATCH_STAGE((st + d + 1) & 1, k_begin + (st + d + 1) * KC)
-                }
-                __syncthreads();
-            }
+        for (int d = 0; d < DA; d++) {
+            const int sn = st + d;
+            if (sn < nstage)
+                run_stage(d, sn, sn + DA < nstage, 2 * ((sn >> 1) + 2) < nstage, 2 * ((sn >> 1) + 2) + 1 < nstage,
+                          sn + 1 < nstage);
         }
     }
-#undef T12_LOAD_STAGE
-#undef T12_STORE_STAGE
-#undef T12_PATCH_STAGE
 
     // ---- overflow path only (more escapes than the LDS list holds): the streamed value of an
     //      escape was its "wrong" decode, so acc[b, m] += (correct - wrong) * X[b, col], added by
@@ -352,17 +428,17 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
 }
 
 // One workgroup per CU (batch tile 256: 128 accumulator registers + the load ring) ...
-template <int WB, int WM, int FB, int FM, int DBG = 0>
-__global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmParams p)
+template <int WB, int WM, int FB, int FM>
+__global__ __launch_bounds__(WB * WM * 64) void gemm_mfma_kernel(const GemmParams p)
 {
-    gemm_mfma_body<WB, WM, FB, FM, DBG>(p);
+    gemm_mfma_body<WB, WM, FB, FM>(p);
 }
 // ... or two (batch tiles <= 128): at most 256 registers per lane, so that two waves share a SIMD
 // and one wave's decode / LDS traffic runs under the other's MFMAs.
-template <int WB, int WM, int FB, int FM, int DBG = 0>
+template <int WB, int WM, int FB, int FM>
 __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel_occ2(const GemmParams p)
 {
-    gemm_mfma_body<WB, WM, FB, FM, DBG>(p);
+    gemm_mfma_body<WB, WM, FB, FM>(p);
 }
 
 // ---------------------------------------------------------------------------
@@ -448,15 +524,13 @@ float* workspace(size_t bytes)
 
 int g_gemm_ksplit = 0;   // 0 = choose by shape
 
-int g_gemm_dbg = 0;
-
-template <int WB, int WM, int FB, int FM, int DBG = 0, bool OCC2 = false>
+template <int WB, int WM, int FB, int FM, bool OCC2 = false>
 int launch_mfma(GemmParams& p, int tiles, hipStream_t st)
 {
     constexpr int TB = WB * FB * 32;
     constexpr int STAGE_BYTES = TB * 8 * 16 + TM * 128;
     const dim3 grid(tiles, (p.B + TB - 1) / TB, p.ksplit);   // batch tiles of one row tile are neighbours in time
-    auto kfn = OCC2 ? gemm_mfma_kernel_occ2<WB, WM, FB, FM, DBG> : gemm_mfma_kernel<WB, WM, FB, FM, DBG>;
+    auto kfn = OCC2 ? gemm_mfma_kernel_occ2<WB, WM, FB, FM> : gemm_mfma_kernel<WB, WM, FB, FM>;
     static bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -467,7 +541,7 @@ int launch_mfma(GemmParams& p, int tiles, hipStream_t st)
         }
         attr_set = true;
     }
-    hipLaunchKernelGGL(kfn, grid, dim3(256), 2 * STAGE_BYTES + PATCH_BYTES, st, p);
+    hipLaunchKernelGGL(kfn, grid, dim3(WB * WM * 64), 2 * STAGE_BYTES + PATCH_BYTES, st, p);
     T12_CHECK_LAUNCH("t12_gemm");
     return T12_OK;
 }
@@ -480,13 +554,6 @@ extern "C" {
 int t12_tune_gemm(int ksplit)
 {
     g_gemm_ksplit = ksplit;
-    return T12_OK;
-}
-
-// Benchmark probe: runs the B > 128 kernel with parts of its loop removed (wrong results).
-int t12_debug_gemm(int mask)
-{
-    g_gemm_dbg = mask;
     return T12_OK;
 }
 
@@ -545,15 +612,14 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
     p.blk_start[nseg] = tiles;
     // K split: fill the chip.  A 256-row batch tile needs a whole CU (LDS, accumulators);
     // smaller batch tiles fit 2-4 workgroups per CU.  Every split keeps >= 4 stages.
-    const bool big = B > 128 && !(g_gemm_dbg & 64);
-    const int btiles = big ? (B + 255) / 256 : (B + 127) / 128;
-    const int per_cu = big ? 1 : (B > 64 ? 2 : 4);
+    const int btiles = B > 128 ? (B + 255) / 256 : 1;
+    const int per_cu = B > 64 ? 1 : 2;
     const int want = 256 * per_cu;
     int ks = 1;
     if (g_gemm_ksplit > 0) ks = g_gemm_ksplit;
     else
         while (tiles * btiles * ks * 4 < want * 3 && K / (ks * 2) >= 4 * KC && ks < 16) ks *= 2;
-    int kslice = ((K / KC + ks - 1) / ks) * KC;
+    int kslice = (((K + 2 * KC - 1) / (2 * KC) + ks - 1) / ks) * 2 * KC;      // whole windows of two stages
     ks = (K + kslice - 1) / kslice;
     p.ksplit = ks;
     p.kslice = kslice;
@@ -566,21 +632,10 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
         }
     }
     int rc;
-    if (B <= 32) rc = launch_mfma<1, 4, 1, 1, 0, true>(p, tiles, st);
-    else if (B <= 64) rc = launch_mfma<1, 4, 2, 1, 0, true>(p, tiles, st);
-    else if (B <= 128 || (g_gemm_dbg & 64)) {
-        if ((g_gemm_dbg & 63) == 0) rc = launch_mfma<1, 4, 4, 1, 0, true>(p, tiles, st);
-        else if ((g_gemm_dbg & 63) == 1) rc = launch_mfma<1, 4, 4, 1, 1, true>(p, tiles, st);
-        else if ((g_gemm_dbg & 63) == 2) rc = launch_mfma<1, 4, 4, 1, 2, true>(p, tiles, st);
-        else if ((g_gemm_dbg & 63) == 8) rc = launch_mfma<1, 4, 4, 1, 8, true>(p, tiles, st);
-        else if ((g_gemm_dbg & 63) == 16) rc = launch_mfma<1, 4, 4, 1, 0, false>(p, tiles, st);
-        else rc = launch_mfma<1, 4, 4, 1, 10, true>(p, tiles, st);
-    }
-    else if (g_gemm_dbg == 1) rc = launch_mfma<2, 2, 4, 2, 1>(p, tiles, st);
-    else if (g_gemm_dbg == 2) rc = launch_mfma<2, 2, 4, 2, 2>(p, tiles, st);
-    else if (g_gemm_dbg == 8) rc = launch_mfma<2, 2, 4, 2, 8>(p, tiles, st);
-    else if (g_gemm_dbg == 10) rc = launch_mfma<2, 2, 4, 2, 10>(p, tiles, st);
-    else rc = launch_mfma<2, 2, 4, 2>(p, tiles, st);
+    if (B <= 32) rc = launch_mfma<1, 4, 1, 1, true>(p, tiles, st);
+    else if (B <= 64) rc = launch_mfma<1, 4, 2, 1, true>(p, tiles, st);
+    else if (B <= 128) rc = launch_mfma<2, 4, 2, 1>(p, tiles, st);
+    else rc = launch_mfma<4, 2, 2, 2>(p, tiles, st);
     if (rc) return rc;
 
     if (ks > 1) {
