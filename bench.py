@@ -14,6 +14,9 @@ Workloads (synthetic, seeded, random-init weights of the Llama-3.1-8B shape:
                   `value`; B = 256 is measured in the same run and reported under "b256"; the
                   decode-GEMV launches of a step are also timed alone for `roofline`.
 
+  moe             one step = one Mixtral-8x7B-shaped MoE FFN layer (8 split-12 experts, top-2) over 256 tokens
+                  grouped per expert through the decode+GEMM (BASELINE config 5).
+
   gemv_stack_b1   one step = every linear layer of one decode step at B = 1 through
                   the fused split-12 decode-GEMV: per layer QKV (3 segments, one
                   launch), O, gate+up (2 segments, one launch), down; then lm_head.
@@ -208,6 +211,38 @@ def run_decode(args, t12, torch, dev):
     _, ms_gemv = timed(torch, cur, gemv_pass, max(args.steps, 10))
     achieved = alg_bytes / (ms_gemv * 1e-3) / 1e9
 
+    # ---- decode+GEMM per layer shape (BASELINE config 2): B in {16, 64, 256}, rotating over the
+    #      weights of up to three layers so that neither L2 nor the 256 MB last-level cache holds a tensor
+    gemm_layers = {}
+    n_rot = min(3, n_l)
+    names = ["qkv", "o", "gate_up", "down"]
+    for B in (16, 64, 256):
+        xs = {K: torch.randn((B, K), generator=g, device=dev).to(torch.bfloat16) for K in (cfg["n_embd"], cfg["n_ff"])}
+        obuf = torch.empty((B, 2 * cfg["n_ff"]), dtype=torch.float32, device=dev)
+        for name, grp in zip(names, groups):
+            calls, flops, wbytes = [], 0.0, 0.0
+            for layer in range(n_rot):
+                segs, off, K = [], 0, None
+                for which in grp:
+                    seg, K, P = eng.weight(layer, which)
+                    seg.out = obuf.data_ptr() + 4 * off
+                    off += seg.M
+                    segs.append(seg)
+                flops, wbytes = 2.0 * off * K * B, 1.5 * off * K
+                calls.append((t12._seg_array(segs), len(segs), xs[K].data_ptr(), K))
+
+            def gemm_pass():
+                for segs, n, act, K in calls:
+                    rc = t12.lib.t12_gemm(segs, n, act, K, 2 * cfg["n_ff"], K, B, cur.cuda_stream)
+                    if rc:
+                        t12.check(rc, "t12_gemm")
+            gemm_pass()
+            _, ms = timed(torch, cur, gemm_pass, 10)
+            us = ms * 1e3 / n_rot
+            gemm_layers["%s_b%d" % (name, B)] = {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
+                                                 "mfma_frac": round(flops / us / 1e6 / 2500.0, 4),
+                                                 "weight_GBps": round(wbytes / us / 1e3, 1)}
+
     # ---- B = 256
     b256 = None
     if args.batch256:
@@ -232,6 +267,7 @@ def run_decode(args, t12, torch, dev):
         "b256": b256,
         "gemv_compressed_GBps": plane_bytes / (ms_gemv * 1e-3) / 1e9,
         "gemv_only_ms_per_step": ms_gemv,
+        "gemm_layers": gemm_layers,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["gemv_stack_b1"] if n_l == LLAMA8B["n_layer"] else None,
@@ -271,12 +307,50 @@ def run_decode(args, t12, torch, dev):
     return result
 
 
+def run_moe(args, t12, torch, dev):
+    """Mixtral-8x7B-shaped MoE FFN layer (BASELINE config 5): 8 experts x (4096 -> 14336 -> 4096, SwiGLU),
+    256 tokens, top-2 routing from random router logits; one step = the whole layer."""
+    import importlib
+    moe = importlib.import_module("turbo_lossless_amd.moe")
+    E, n, ff, T = 8, 4096, 14336, 256
+    t0 = time.time()
+    experts = [moe.Expert(*[t12.pack_device(synth_weight(torch, M, K, 5000 + 3 * e + j, dev, p_out=5e-4))
+                            for j, (M, K) in enumerate([(ff, n), (ff, n), (n, ff)])]) for e in range(E)]
+    torch.cuda.synchronize()
+    t_build = time.time() - t0
+    g = torch.Generator(device=dev)
+    g.manual_seed(5100)
+    X = torch.randn((T, n), generator=g, device=dev).to(torch.bfloat16).view(torch.int16)
+    ids, w = moe.route_top_k(torch.randn((T, E), generator=g, device=dev), 2)
+    cur = torch.cuda.current_stream()
+
+    def step():
+        moe.moe_ffn(experts, X, ids, w, stream=cur.cuda_stream)
+    for _ in range(args.warmup):
+        step()
+    ms_step, ms = timed(torch, cur, step, args.steps)
+    flops = 2.0 * (T * 2) * 3 * n * ff
+    wbytes = 1.5 * E * 3 * n * ff
+    return {
+        "metric": "tokens/s through one Mixtral-8x7B-shaped split-12 MoE FFN layer (8 experts, top-2), 256 tokens",
+        "value": T * 1e3 / ms_step, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "moe_mixtral_b256", "experts": E, "top_k": 2, "tokens": T,
+                   "tokens_per_expert": torch.bincount(ids.reshape(-1), minlength=E).tolist()},
+        "TFLOPs": flops / ms / 1e9, "weight_GBps": wbytes / ms / 1e6,
+        "roofline": {"bound": "hbm", "achieved": wbytes / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": wbytes / ms / 1e6 / HBM_PEAK_GBS, "traffic": None, "kernel": "gemm_mfma_kernel"},
+        "setup_s": t_build,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="decode", choices=["decode", "gemv_stack_b1"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "gemv_stack_b1", "moe"])
     ap.add_argument("--prompt", type=int, default=128)
     ap.add_argument("--no-batch256", dest="batch256", action="store_false")
     ap.add_argument("--layers", type=int, default=LLAMA8B["n_layer"], help="debug: fewer layers (invalid as a result)")
@@ -297,6 +371,9 @@ def main():
     torch.cuda.set_device(dev)
     if args.workload == "decode":
         print(json.dumps(run_decode(args, t12, torch, dev)))
+        return
+    if args.workload == "moe":
+        print(json.dumps(run_moe(args, t12, torch, dev)))
         return
     cfg = dict(LLAMA8B, n_layer=args.layers)
 

@@ -1,0 +1,105 @@
+"""GPU parity: Mixtral-shaped MoE FFN (top-2 of 8 split-12 experts, tokens grouped per expert
+through the decode+GEMM) -- small layer against the CPU oracle, full-size layer against a
+decode-then-fp32 matmul of the same (bit-exact, separately tested) decoded weights.
+
+Tolerance: 1e-2 relative (north star); observed ~1e-5 (fp32 accumulation order only; the
+SwiGLU activation is rounded to bf16 on both sides, as the engine does between the two GEMMs).
+"""
+import importlib
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import dev, rel_err, to_dev_bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def synth(t12):
+    return importlib.import_module("turbo_lossless_amd.synth")
+
+
+@pytest.fixture(scope="module")
+def moe(t12):
+    return importlib.import_module("turbo_lossless_amd.moe")
+
+
+def bf16_to_f32(bits):
+    return (np.asarray(bits, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def test_moe_small_vs_oracle(t12, oracle, synth, moe):
+    E, n, n_ff, T = 8, 512, 1024, 64
+    packs = [[oracle.pack(synth.weights_llm(m, k, seed=5000 + 3 * e + j, p_outlier=5e-4))
+              for j, (m, k) in enumerate([(n_ff, n), (n_ff, n), (n, n_ff)])] for e in range(E)]
+    experts = [moe.Expert(*[t12.DeviceTensor12.from_packed(p, dev()) for p in ps]) for ps in packs]
+    X = synth.activations(T, n, seed=77)
+    rng = np.random.default_rng(5)
+    logits = torch.from_numpy(rng.standard_normal((T, E)).astype(np.float32)).to(dev())
+    ids, w = moe.route_top_k(logits, 2)
+    got = moe.moe_ffn(experts, to_dev_bits(X).reshape(T, n), ids, w).cpu().numpy()
+    ids_h, w_h = ids.cpu().numpy(), w.cpu().numpy()
+    assert sorted(np.bincount(ids_h.reshape(-1), minlength=E).tolist())[0] >= 0      # ragged groups, some may be empty
+    ref = np.zeros((T, n), np.float64)
+    for e in range(E):
+        rows, slots = np.nonzero(ids_h == e)
+        if len(rows) == 0:
+            continue
+        xe = X[rows]
+        g = oracle.gemm(packs[e][0], xe)
+        u = oracle.gemm(packs[e][1], xe)
+        a = oracle.silu_mul_bf16(g, u)
+        y = oracle.gemm(packs[e][2], a)
+        ref[rows] += w_h[rows, slots][:, None].astype(np.float64) * y
+    assert rel_err(got, ref) < 1e-4
+
+
+def test_moe_single_expert_gets_every_token(t12, oracle, synth, moe):
+    # all tokens routed to one expert (the other seven groups are empty): equals a plain FFN
+    E, n, n_ff, T = 4, 256, 512, 33
+    packs = [[oracle.pack(synth.weights_llm(m, k, seed=60 + 3 * e + j)) for j, (m, k) in
+              enumerate([(n_ff, n), (n_ff, n), (n, n_ff)])] for e in range(E)]
+    experts = [moe.Expert(*[t12.DeviceTensor12.from_packed(p, dev()) for p in ps]) for ps in packs]
+    X = synth.activations(T, n, seed=78)
+    ids = torch.full((T, 1), 2, dtype=torch.int64, device=dev())
+    w = torch.ones((T, 1), dtype=torch.float32, device=dev())
+    got = moe.moe_ffn(experts, to_dev_bits(X).reshape(T, n), ids, w).cpu().numpy()
+    a = oracle.silu_mul_bf16(oracle.gemm(packs[2][0], X), oracle.gemm(packs[2][1], X))
+    assert rel_err(got, oracle.gemm(packs[2][2], a)) < 1e-4
+
+
+def test_moe_mixtral_shape_b256(t12, synth, moe):
+    # full size: 8 experts x (4096 -> 14336 -> 4096), 256 tokens, top-2; weights N(0, 0.02) + 5e-4 outliers
+    E, n, n_ff, T = 8, 4096, 14336, 256
+    g = torch.Generator(device=dev())
+
+    def mk(M, K, seed):
+        g.manual_seed(seed)
+        wt = torch.randn((M, K), generator=g, device=dev()) * 0.02
+        m = torch.rand((M, K), generator=g, device=dev()) < 5e-4
+        wt = torch.where(m, torch.randn((M, K), generator=g, device=dev()) * 8, wt).to(torch.bfloat16)
+        return t12.pack_device(wt)
+
+    experts = [moe.Expert(mk(n_ff, n, 5000 + 3 * e), mk(n_ff, n, 5001 + 3 * e), mk(n, n_ff, 5002 + 3 * e))
+               for e in range(E)]
+    g.manual_seed(9)
+    Xf = torch.randn((T, n), generator=g, device=dev()).to(torch.bfloat16)
+    logits = torch.randn((T, E), generator=g, device=dev())
+    ids, w = moe.route_top_k(logits, 2)
+    got = moe.moe_ffn(experts, Xf.view(torch.int16), ids, w)
+    torch.cuda.synchronize()
+    ref = torch.zeros((T, n), dtype=torch.float32, device=dev())
+    for e in range(E):
+        rows, slots = torch.nonzero(ids == e, as_tuple=True)
+        if rows.numel() == 0:
+            continue
+        dec = [t12.decompress(t).view(torch.bfloat16).float() for t in (experts[e].w1, experts[e].w3, experts[e].w2)]
+        xe = Xf[rows].float()
+        gate, up = xe @ dec[0].t(), xe @ dec[1].t()
+        a = (torch.nn.functional.silu(gate) * up).to(torch.bfloat16).float()
+        ref[rows] += w[rows, slots][:, None] * (a @ dec[2].t())
+        del dec
+    err = float((got - ref).abs().max() / ref.abs().max())
+    assert err < 1e-2, err
