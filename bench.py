@@ -14,6 +14,10 @@ Workloads (synthetic, seeded, random-init weights of the Llama-3.1-8B shape:
                   `value`; B = 256 is measured in the same run and reported under "b256"; the
                   decode-GEMV launches of a step are also timed alone for `roofline`.
 
+  gemm_layers     the four linear-layer shapes through the fused decode+GEMM at B = 16, 64, 256 on three
+                  rotating weight copies (BASELINE config 2); `roofline` prices gate|up at B = 256 against
+                  the 2.5 PFLOP/s dense bf16 MFMA peak.
+
   moe             one step = one Mixtral-8x7B-shaped MoE FFN layer (8 split-12 experts, top-2) over 256 tokens
                   grouped per expert through the decode+GEMM (BASELINE config 5).
 
@@ -44,7 +48,9 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per gemv launch of the gemv_stack_b1 workload, from two rocprofv3 --pmc runs of this file
 # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from the --calibrate copy kernel; the summary is
 # profiles/gemv_stream_kernel_llama8b_stack_b1.md).  Valid for the full 32-layer stack only.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"gemv_stack_b1": 88.48e6}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"gemv_stack_b1": 88.48e6,
+                                     # gate|up at B = 256 (profiles/gemm_mfma_kernel_llama8b_layers.md)
+                                     "gemm_gate_up_b256": 226.8e6}
 
 
 def synth_weight(torch, M, K, seed, dev, sigma=0.02, p_out=3e-4, sigma_out=8.0):
@@ -211,37 +217,8 @@ def run_decode(args, t12, torch, dev):
     _, ms_gemv = timed(torch, cur, gemv_pass, max(args.steps, 10))
     achieved = alg_bytes / (ms_gemv * 1e-3) / 1e9
 
-    # ---- decode+GEMM per layer shape (BASELINE config 2): B in {16, 64, 256}, rotating over the
-    #      weights of up to three layers so that neither L2 nor the 256 MB last-level cache holds a tensor
-    gemm_layers = {}
-    n_rot = min(3, n_l)
-    names = ["qkv", "o", "gate_up", "down"]
-    for B in (16, 64, 256):
-        xs = {K: torch.randn((B, K), generator=g, device=dev).to(torch.bfloat16) for K in (cfg["n_embd"], cfg["n_ff"])}
-        obuf = torch.empty((B, 2 * cfg["n_ff"]), dtype=torch.float32, device=dev)
-        for name, grp in zip(names, groups):
-            calls, flops, wbytes = [], 0.0, 0.0
-            for layer in range(n_rot):
-                segs, off, K = [], 0, None
-                for which in grp:
-                    seg, K, P = eng.weight(layer, which)
-                    seg.out = obuf.data_ptr() + 4 * off
-                    off += seg.M
-                    segs.append(seg)
-                flops, wbytes = 2.0 * off * K * B, 1.5 * off * K
-                calls.append((t12._seg_array(segs), len(segs), xs[K].data_ptr(), K))
-
-            def gemm_pass():
-                for segs, n, act, K in calls:
-                    rc = t12.lib.t12_gemm(segs, n, act, K, 2 * cfg["n_ff"], K, B, cur.cuda_stream)
-                    if rc:
-                        t12.check(rc, "t12_gemm")
-            gemm_pass()
-            _, ms = timed(torch, cur, gemm_pass, 10)
-            us = ms * 1e3 / n_rot
-            gemm_layers["%s_b%d" % (name, B)] = {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
-                                                 "mfma_frac": round(flops / us / 1e6 / 2500.0, 4),
-                                                 "weight_GBps": round(wbytes / us / 1e3, 1)}
+    gemm_layers = gemm_layer_leg(t12, torch, dev, cfg, lambda layer, which: eng.weight(layer, which), min(3, n_l),
+                                 cur, g)
 
     # ---- B = 256
     b256 = None
@@ -345,12 +322,93 @@ def run_moe(args, t12, torch, dev):
     }
 
 
+def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(16, 64, 256), iters=10):
+    """decode+GEMM per layer shape (BASELINE config 2): for each B, each of QKV (3 segments), O, gate|up
+    (2 segments), down is timed over `n_rot` distinct weight copies in rotation, so that neither L2 nor
+    the 256 MB last-level cache holds a tensor between launches.  weight_of(copy, which) -> (segment, K, P)."""
+    out = {}
+    groups = [(0, 1, 2), (3,), (4, 5), (6,)]
+    names = ["qkv", "o", "gate_up", "down"]
+    for B in batches:
+        xs = {K: torch.randn((B, K), generator=g, device=dev).to(torch.bfloat16) for K in (cfg["n_embd"], cfg["n_ff"])}
+        obuf = torch.empty((B, 2 * cfg["n_ff"]), dtype=torch.float32, device=dev)
+        for name, grp in zip(names, groups):
+            calls, flops, wbytes = [], 0.0, 0.0
+            for copy in range(n_rot):
+                segs, off, K = [], 0, None
+                for which in grp:
+                    seg, K, P = weight_of(copy, which)
+                    seg.out = obuf.data_ptr() + 4 * off
+                    off += seg.M
+                    segs.append(seg)
+                flops, wbytes = 2.0 * off * K * B, 1.5 * off * K
+                calls.append((t12._seg_array(segs), len(segs), xs[K].data_ptr(), K))
+
+            def gemm_pass():
+                for segs, n, act, K in calls:
+                    rc = t12.lib.t12_gemm(segs, n, act, K, 2 * cfg["n_ff"], K, B, cur.cuda_stream)
+                    if rc:
+                        t12.check(rc, "t12_gemm")
+            gemm_pass()
+            _, ms = timed(torch, cur, gemm_pass, iters)
+            us = ms * 1e3 / n_rot
+            out["%s_b%d" % (name, B)] = {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
+                                         "mfma_frac": round(flops / us / 1e6 / 2500.0, 4),
+                                         "weight_GBps": round(wbytes / us / 1e3, 1), "flops": flops}
+    return out
+
+
+def run_gemm_layers(args, t12, torch, dev):
+    """The four Llama-3.1-8B linear-layer shapes through the fused decode+GEMM at B = 16, 64, 256 (BASELINE
+    config 2) on three rotating weight copies; one step = the four layer GEMMs of one decoder layer at B = 256."""
+    cfg = dict(LLAMA8B)
+    n, ff = cfg["n_embd"], cfg["n_ff"]
+    kv = cfg["n_head_kv"] * (n // cfg["n_head"])
+    shapes = [(n, n), (kv, n), (kv, n), (n, n), (ff, n), (ff, n), (n, ff)]       # wq wk wv wo gate up down
+    t0 = time.time()
+    copies = [[t12.pack_device(synth_weight(torch, M, K, 2000 + 10 * c + i, dev)) for i, (M, K) in enumerate(shapes)]
+              for c in range(3)]
+    torch.cuda.synchronize()
+    t_build = time.time() - t0
+
+    def weight_of(copy, which):
+        t = copies[copy][which]
+        return t.segment(None), t.K, t.P
+    g = torch.Generator(device=dev)
+    g.manual_seed(2100)
+    cur = torch.cuda.current_stream()
+    if args.calibrate:
+        src = torch.empty(2**30, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        t12.check(t12.lib.t12_util_copy(dst.data_ptr(), src.data_ptr(), src.numel(), 8192, cur.cuda_stream), "t12_util_copy")
+        torch.cuda.synchronize()
+        del src, dst
+    layers = gemm_layer_leg(t12, torch, dev, cfg, weight_of, 3, cur, g, iters=max(args.steps, 10))
+    us256 = sum(layers["%s_b256" % k]["us"] for k in ("qkv", "o", "gate_up", "down"))
+    fl256 = sum(layers["%s_b256" % k]["flops"] for k in ("qkv", "o", "gate_up", "down"))
+    gu = layers["gate_up_b256"]
+    return {
+        "metric": "decode+GEMM TFLOP/s at B=256 over the linear layers of one Llama-3.1-8B decoder layer (split-12 weights)",
+        "value": fl256 / us256 / 1e6, "unit": "TFLOP/s", "n_gpus": 1, "steps": max(args.steps, 10), "warmup": 1,
+        "ms_per_step": us256 / 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "gemm_layers: QKV 4096->6144 (3 segments), O 4096->4096, gate|up 4096->28672 (2 segments), "
+                               "down 14336->4096; N(0,0.02)+3e-4 outliers; B in {16,64,256}; 3 rotating weight copies"},
+        "layers": layers,
+        "roofline": {"bound": "mfma", "achieved": gu["TFLOPs"], "peak": 2500.0, "unit": "TFLOP/s",
+                     "frac": gu["TFLOPs"] / 2500.0, "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get("gemm_gate_up_b256"),
+                     "kernel": "gemm_mfma_kernel<4,2,2,2> on gate|up at B=256", "flops_per_launch": gu["flops"],
+                     "us_per_launch": gu["us"]},
+        "setup_s": t_build,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="decode", choices=["decode", "gemv_stack_b1", "moe"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "gemv_stack_b1", "moe", "gemm_layers"])
     ap.add_argument("--prompt", type=int, default=128)
     ap.add_argument("--no-batch256", dest="batch256", action="store_false")
     ap.add_argument("--layers", type=int, default=LLAMA8B["n_layer"], help="debug: fewer layers (invalid as a result)")
@@ -371,6 +429,9 @@ def main():
     torch.cuda.set_device(dev)
     if args.workload == "decode":
         print(json.dumps(run_decode(args, t12, torch, dev)))
+        return
+    if args.workload == "gemm_layers":
+        print(json.dumps(run_gemm_layers(args, t12, torch, dev)))
         return
     if args.workload == "moe":
         print(json.dumps(run_moe(args, t12, torch, dev)))
