@@ -1,0 +1,51 @@
+/* C face of the engine API (libturbo12.so) for callers that cannot include the C++ headers
+ * include/turbo/{model,inference,sampler}.h: ctypes, cgo, JNI.  Each function forwards to the C++
+ * function named beside it, which keeps the reference's name and meaning (engine/model.h:79-82,
+ * engine/inference.h:43-55, engine/sampler.h:5-11).  Handles are the C++ objects as void*.
+ */
+#ifndef T12_ENGINE_H
+#define T12_ENGINE_H
+
+#include <stddef.h>
+#include <stdint.h>
+#include "t12_abi.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+void* t12_engine_load(const char* model_dir, int device);            /* load_model; NULL on failure (model.cpp:165-328) */
+/* create_synthetic_model: a random-init model of the given shape, generated and packed on the GPU
+ * (weights N(0, 0.02) with outliers N(0, 8) at rate p_outlier; norm weights 1).  No reference counterpart:
+ * the reference loads converted checkpoints only. */
+void* t12_engine_create_synthetic(int n_vocab, int n_embd, int n_head, int n_head_kv, int n_layer, int n_ff, int n_ctx,
+                                  float rope_theta, float rms_eps, uint64_t seed, int max_seq, float p_outlier);
+int   t12_engine_save(void* model, const char* dir);                 /* save_model: the files of convert_model.py:127-152; 0 = ok */
+void  t12_engine_free_model(void* model);                            /* free_model */
+int   t12_engine_max_seq(void* model);                               /* Model::max_seq_len (TURBO_CTX, model.cpp:192-195) */
+/* which: 0 wq 1 wk 2 wv 3 wo 4 w_gate 5 w_up 6 w_down; layer -1 = output_proj.  Fills *seg (out = NULL), *K and the
+ * escape count; returns 0, or -1 for a tensor that does not exist. */
+int   t12_engine_weight(void* model, int layer, int which, T12Segment* seg, int* K, int* num_patches);
+
+void* t12_engine_create_state(void* model, int batch, int max_seq);  /* create_inference_state (inference.cpp:94-166) */
+void  t12_engine_free_state(void* state);                            /* free_inference_state */
+void  t12_engine_set_positions(void* state, const int* pos);         /* state->positions[0..batch) = pos (inference.cpp:722) */
+void  t12_engine_get_positions(void* state, int* pos);
+int   t12_engine_forward(void* state, const int* tokens_host);       /* forward: logits stay on the device */
+void* t12_engine_logits(void* state);                                /* state->logits, fp32 [batch, n_vocab] on the device */
+void* t12_engine_stream(void* state);                                /* state->stream (hipStream_t) */
+int   t12_engine_sync(void* state);                                  /* hipStreamSynchronize(state->stream); 0 = ok */
+int   t12_engine_sample(void* state, int* tokens_out_host);          /* sample_greedy_batch on state->logits (sampler.cpp:18-32) */
+/* generate: prompt, then up to max_tokens greedy tokens (stops on id 2, inference.cpp:727,742); writes them to out
+ * (room for max_tokens ints) and returns how many. */
+int   t12_engine_generate(void* state, const int* prompt, int n_prompt, int max_tokens, int* out);
+
+/* Synthetic tensors on the device (what create_synthetic_model is built from). */
+int   t12_synth_normal_bf16(void* out_bf16, size_t n, uint64_t seed, float sigma, float p_outlier, float sigma_outlier,
+                            void* stream);
+int   t12_fill_f32(void* out, size_t n, float value, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* T12_ENGINE_H */

@@ -26,6 +26,26 @@ def test_library_exports_declared_c_abi():
     assert not missing, missing
 
 
+def test_library_exports_every_declaration_of_every_header():
+    lib = ctypes.CDLL(LIB)
+    for header in ("t12_abi.h", "t12_glue.h", "t12_engine.h"):
+        names = declared_functions(os.path.join(ROOT, "include", header))
+        assert len(names) >= 15, (header, names)
+        missing = [n for n in sorted(names) if not hasattr(lib, n)]
+        assert not missing, (header, missing)
+
+
+def test_every_exported_c_symbol_is_declared_in_a_header():
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", LIB], capture_output=True, text=True).stdout
+    exported = {ln.split()[2] for ln in out.splitlines() if len(ln.split()) == 3 and ln.split()[1] == "T"
+                and not ln.split()[2].startswith("_")}
+    declared = set()
+    for header in ("t12_abi.h", "t12_glue.h", "t12_engine.h"):
+        declared |= declared_functions(os.path.join(ROOT, "include", header))
+    assert not sorted(exported - declared), sorted(exported - declared)
+
+
 def test_library_exports_glue_and_engine_c_face():
     lib = ctypes.CDLL(LIB)
     glue = ["launch_embed_lookup", "launch_rms_norm_bf16_batch", "launch_add_rms_norm_bf16_batch",
