@@ -169,14 +169,11 @@ def run_decode(args, t12, torch, dev):
         for i, t in enumerate(prompt):                      # prefill, one token per forward (inference.cpp:721-724)
             e.set_positions([i] * B)
             e.forward([t] * B)
-        state = {"tok": e.sample()}
-
-        def step():
-            e.forward(state["tok"])
-            state["tok"] = e.sample()                       # D2H + stream sync per token (sampler.cpp:18-32)
-        for _ in range(args.warmup):
-            step()
-        return timed(torch, st, step, args.steps)
+        # one step = sample (argmax on the device) + forward on the sampled ids, K of them inside
+        # decode_greedy: the host reads token t while the GPU computes step t + 1
+        e.decode(args.warmup)
+        ms, ev = timed(torch, st, lambda: e.decode(args.steps), 1)
+        return ms / args.steps, ev / args.steps
 
     ms1, _ = decode_loop(eng, 1)
 

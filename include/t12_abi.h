@@ -66,6 +66,8 @@ const char* t12_last_error(void);      /* text of the last failure on this threa
  * profiler's FETCH_SIZE / WRITE_SIZE counters.  `sink` holds blocks x u32. */
 int t12_util_read(const void* src, size_t bytes, void* sink, int blocks, void* stream);
 int t12_util_copy(void* dst, const void* src, size_t bytes, int blocks, void* stream);
+/* dst[0..n) = src[0..n) (32-bit words) by a kernel; dst may be pinned host memory. */
+int t12_util_copy_i32(void* dst, const void* src, int n, void* stream);
 /* Pins the B = 1 kernel variant (100*waves + 10*rows_per_wave + ring depth);
  * 0 restores the choice by shape.  For benchmark sweeps. */
 int t12_tune_gemv(int variant);

@@ -39,6 +39,9 @@ int   t12_engine_sample(void* state, int* tokens_out_host);          /* sample_g
 /* generate: prompt, then up to max_tokens greedy tokens (stops on id 2, inference.cpp:727,742); writes them to out
  * (room for max_tokens ints) and returns how many. */
 int   t12_engine_generate(void* state, const int* prompt, int n_prompt, int max_tokens, int* out);
+/* decode_greedy: the decode half of generate, from the logits the state holds: up to max_tokens steps of
+ * (sample, forward), the next step enqueued before the host has read the token.  out may be NULL. */
+int   t12_engine_decode(void* state, int max_tokens, int stop_on_eos, int* out);
 
 /* Synthetic tensors on the device (what create_synthetic_model is built from). */
 int   t12_synth_normal_bf16(void* out_bf16, size_t n, uint64_t seed, float sigma, float p_outlier, float sigma_outlier,

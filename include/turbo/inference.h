@@ -45,3 +45,9 @@ void forward(InferenceState* state, const int* token_ids);
 // Prompt one token per forward, then greedy decode; stops at token id 2 like the
 // reference (engine/inference.cpp:716-748).
 std::vector<int> generate(InferenceState* state, const std::vector<int>& prompt_tokens, int max_tokens);
+
+// The decode half of generate (extension): up to max_tokens greedy steps from the logits the state
+// holds, each a sample followed by a forward on the sampled ids; returns the ids of sequence 0.
+// forward(state, nullptr) runs on the ids already in state->d_tokens (device) -- what lets the loop
+// enqueue step t + 1 before the host has seen token t.
+std::vector<int> decode_greedy(InferenceState* state, int max_tokens, bool stop_on_eos);

@@ -183,3 +183,37 @@ def test_synthetic_model_save_load_roundtrip(t12, tmp_path):
             assert torch.equal(b.logits(cfg["n_vocab"]), ref)
     finally:
         b.close()
+
+
+@pytest.mark.parametrize("B", [1, 3])
+def test_pipelined_decode_equals_step_by_step(t12, small_model, B):
+    """decode_greedy enqueues step t + 1 on the device-resident ids before the host has read token t;
+    the stream, the stop at id 2 and the positions left behind must equal the reference's order
+    (sample, wait, forward), which TURBO_NO_PIPELINE=1 runs."""
+    path, _ = small_model
+    rng = np.random.default_rng(11)
+    prompts = [[int(t) for t in rng.integers(3, SMALL["n_vocab"], size=5)] for _ in range(12)]
+    eng = t12.Engine.load(path, batch=B)
+    try:
+        saw_eos = False
+        for prompt in prompts:
+            runs = []
+            for env in ("1", None):
+                if env:
+                    os.environ["TURBO_NO_PIPELINE"] = env
+                else:
+                    os.environ.pop("TURBO_NO_PIPELINE", None)
+                toks = eng.generate(prompt, 40)
+                runs.append((toks, eng.positions()))
+            assert runs[0] == runs[1]
+            saw_eos = saw_eos or len(runs[0][0]) < 40
+            assert runs[0][1] == [len(prompt) + len(runs[0][0])] * B
+        # decode() continues from the logits left behind, without the stop rule
+        os.environ["TURBO_NO_PIPELINE"] = "1"
+        a = eng.generate(prompts[0], 8) + eng.decode(8)
+        os.environ.pop("TURBO_NO_PIPELINE", None)
+        b = eng.generate(prompts[0], 8) + eng.decode(8)
+        assert a == b and (len(a) == 16 or 2 in a or saw_eos)
+    finally:
+        os.environ.pop("TURBO_NO_PIPELINE", None)
+        eng.close()

@@ -84,6 +84,7 @@ _SIGS = {
     "t12_engine_get_positions": (None, [_vp, C.POINTER(C.c_int)]),
     "t12_engine_sample": (_i, [_vp, C.POINTER(C.c_int)]),
     "t12_engine_generate": (_i, [_vp, C.POINTER(C.c_int), _i, _i, C.POINTER(C.c_int)]),
+    "t12_engine_decode": (_i, [_vp, _i, _i, C.POINTER(C.c_int)]),
     "t12_engine_sync": (_i, [_vp]),
     "t12_engine_weight": (_i, [_vp, _i, _i, C.POINTER(Segment), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "t12_gemv_swiglu": (_i, [C.POINTER(Segment), C.POINTER(Segment), _vp, _i, _vp, _vp]),
@@ -317,6 +318,12 @@ class Engine:
         p = (C.c_int * len(prompt))(*[int(t) for t in prompt])
         out = (C.c_int * max(max_tokens, 1))()
         n = lib.t12_engine_generate(self.state, p, len(prompt), max_tokens, out)
+        return list(out[:n])
+
+    def decode(self, max_tokens, stop_on_eos=False):
+        """Up to max_tokens greedy steps (sample, forward) from the current logits; ids of sequence 0."""
+        out = (C.c_int * max(max_tokens, 1))()
+        n = lib.t12_engine_decode(self.state, max_tokens, int(stop_on_eos), out)
         return list(out[:n])
 
     def weight(self, layer, which):

@@ -65,6 +65,14 @@ int t12_engine_generate(void* state, const int* prompt, int n_prompt, int max_to
     return (int)r.size();
 }
 
+int t12_engine_decode(void* state, int max_tokens, int stop_on_eos, int* out)
+{
+    std::vector<int> r = decode_greedy((InferenceState*)state, max_tokens, stop_on_eos != 0);
+    if (out)
+        for (size_t i = 0; i < r.size(); i++) out[i] = r[i];
+    return (int)r.size();
+}
+
 int t12_engine_sync(void* state)
 {
     return hipStreamSynchronize(((InferenceState*)state)->stream) == hipSuccess ? 0 : -1;

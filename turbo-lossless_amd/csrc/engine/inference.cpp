@@ -21,6 +21,7 @@
 
 extern "C" {
 void launch_embed_lookup(const int16_t*, const int*, float*, int, int, int, hipStream_t);
+void launch_argmax_batch(const float*, int*, int, int, hipStream_t);
 void launch_rms_norm_bf16_batch(const float*, const float*, int16_t*, int, float, int, hipStream_t);
 void launch_add_rms_norm_bf16_batch(float*, const float*, const float*, int16_t*, int, float, int, hipStream_t);
 void launch_silu_mul_bf16_batch(const float*, const float*, int16_t*, int, int, hipStream_t);
@@ -46,6 +47,9 @@ struct Impl {
     T12Segment head[1];
     bool fused_b1 = false;     // B = 1 takes the 5-launch-per-layer path
     bool checked = false;
+    // pipelined greedy decoding: sampled tokens land in pinned host memory, two slots in rotation
+    int* h_tokens[2] = {nullptr, nullptr};
+    hipEvent_t sampled[2] = {nullptr, nullptr};
 };
 
 void check_gpu(hipError_t e, const char* what)
@@ -150,7 +154,14 @@ void free_inference_state(InferenceState* state)
     if (state->stream) (void)hipStreamDestroy(state->stream);
     if (state->stream2) (void)hipStreamDestroy(state->stream2);
     if (state->sync_event) (void)hipEventDestroy(state->sync_event);
-    delete (Impl*)state->impl;
+    Impl* impl = (Impl*)state->impl;
+    if (impl) {
+        for (int i = 0; i < 2; i++) {
+            if (impl->h_tokens[i]) (void)hipHostFree(impl->h_tokens[i]);
+            if (impl->sampled[i]) (void)hipEventDestroy(impl->sampled[i]);
+        }
+    }
+    delete impl;
     delete state;
 }
 
@@ -198,7 +209,7 @@ void forward_b1_fused(InferenceState* state, const int* token_ids)
     Impl* impl = (Impl*)state->impl;
     const int pos = state->positions[0];
 
-    (void)hipMemcpyAsync(state->d_tokens, token_ids, sizeof(int), hipMemcpyHostToDevice, st);
+    if (token_ids) (void)hipMemcpyAsync(state->d_tokens, token_ids, sizeof(int), hipMemcpyHostToDevice, st);
     launch_embed_lookup(m->token_embd, state->d_tokens, state->hidden, n, 1, c.n_vocab, st);
 
     float* h = state->hidden;          // residual stream
@@ -281,7 +292,7 @@ void forward(InferenceState* state, const int* token_ids)
             return;
         }
     }
-    (void)hipMemcpyAsync(state->d_tokens, token_ids, B * sizeof(int), hipMemcpyHostToDevice, st);
+    if (token_ids) (void)hipMemcpyAsync(state->d_tokens, token_ids, B * sizeof(int), hipMemcpyHostToDevice, st);
     if (B > 1) (void)hipMemcpyAsync(state->d_positions, state->positions, B * sizeof(int), hipMemcpyHostToDevice, st);
     launch_embed_lookup(m->token_embd, state->d_tokens, state->hidden, n, B, c.n_vocab, st);
 
@@ -338,10 +349,62 @@ void forward(InferenceState* state, const int* token_ids)
     for (int b = 0; b < B; b++) state->positions[b]++;
 }
 
-std::vector<int> generate(InferenceState* state, const std::vector<int>& prompt_tokens, int max_tokens)
+// Greedy decoding from the logits the state holds, `max_tokens` steps of (sample, forward).
+// The reference's loop (inference.cpp:726-746) waits for every sampled token on the host before it
+// enqueues the next forward, so the GPU idles for a host round trip per token.  Here the argmax
+// writes the token ids straight into state->d_tokens and the next forward is enqueued on them at
+// once (forward(state, nullptr)); the ids also travel to pinned host memory, and the host reads
+// token t while the GPU already computes step t + 1.  Same tokens, same stop rule (id 2 of sequence
+// 0 ends the stream when stop_on_eos): the one forward issued past an end-of-stream token is undone
+// by stepping the positions back.  TURBO_NO_PIPELINE=1 restores the reference's order.
+std::vector<int> decode_greedy(InferenceState* state, int max_tokens, bool stop_on_eos)
 {
     std::vector<int> output;
     const int n_vocab = state->model->config.n_vocab;
+    const int bs = state->batch_size;
+    hipStream_t st = state->stream;
+    const bool no_pipeline = getenv("TURBO_NO_PIPELINE") != nullptr;
+    if (no_pipeline) {
+        std::vector<int> tokens(bs);
+        for (int t = 0; t < max_tokens; t++) {
+            if (bs == 1) tokens[0] = sample_greedy(state->logits, n_vocab, st);
+            else sample_greedy_batch(state->logits, tokens.data(), n_vocab, bs, st);
+            if (stop_on_eos && tokens[0] == 2) break;
+            output.push_back(tokens[0]);
+            forward(state, tokens.data());
+        }
+        return output;
+    }
+    Impl* impl = (Impl*)state->impl;
+    for (int i = 0; i < 2; i++) {
+        if (!impl->h_tokens[i]) check_gpu(hipHostMalloc((void**)&impl->h_tokens[i], bs * sizeof(int)), "hipHostMalloc");
+        if (!impl->sampled[i]) check_gpu(hipEventCreateWithFlags(&impl->sampled[i], hipEventDisableTiming), "hipEventCreate");
+    }
+    auto enqueue_sample = [&](int slot) {
+        launch_argmax_batch(state->logits, state->d_tokens, n_vocab, bs, st);
+        // ids -> pinned host memory by a kernel: a DMA-engine copy in the middle of the stream costs a
+        // queue hand-over each way (~0.2 ms per token measured)
+        must(t12_util_copy_i32(impl->h_tokens[slot], state->d_tokens, bs, st), "token copy");
+        (void)hipEventRecord(impl->sampled[slot], st);
+    };
+    if (max_tokens > 0) enqueue_sample(0);
+    for (int t = 0; t < max_tokens; t++) {
+        forward(state, nullptr);                                  // on the ids the argmax left in d_tokens
+        if (t + 1 < max_tokens) enqueue_sample((t + 1) & 1);
+        check_gpu(hipEventSynchronize(impl->sampled[t & 1]), "hipEventSynchronize");
+        const int tok = impl->h_tokens[t & 1][0];
+        if (stop_on_eos && tok == 2) {
+            for (int b = 0; b < bs; b++) state->positions[b]--;   // the forward on the end-of-stream id does not count
+            break;
+        }
+        output.push_back(tok);
+    }
+    check_gpu(hipStreamSynchronize(st), "hipStreamSynchronize");
+    return output;
+}
+
+std::vector<int> generate(InferenceState* state, const std::vector<int>& prompt_tokens, int max_tokens)
+{
     const int bs = state->batch_size;
     std::vector<int> tokens(bs);
     for (int i = 0; i < (int)prompt_tokens.size(); i++) {
@@ -351,12 +414,5 @@ std::vector<int> generate(InferenceState* state, const std::vector<int>& prompt_
         }
         forward(state, tokens.data());
     }
-    for (int t = 0; t < max_tokens; t++) {
-        if (bs == 1) tokens[0] = sample_greedy(state->logits, n_vocab, state->stream);
-        else sample_greedy_batch(state->logits, tokens.data(), n_vocab, bs, state->stream);
-        if (tokens[0] == 2) break;
-        output.push_back(tokens[0]);
-        forward(state, tokens.data());
-    }
-    return output;
+    return decode_greedy(state, max_tokens, true);
 }
