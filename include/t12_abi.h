@@ -33,6 +33,7 @@ extern "C" {
 #define T12_EINVAL     (-1)   /* bad shape / null pointer / unsupported size */
 #define T12_ELAUNCH    (-2)   /* HIP reported a launch or runtime error      */
 #define T12_MAX_SEGMENTS 8
+#define T12_MAX_KSPLIT 16      /* most K splits a decode+GEMM launch uses (T12GemmPartials.nsplit) */
 
 /* One weight tensor of a fused launch.  Several tensors that consume the same
  * activations (wq|wk|wv, gate|up, the experts of one token group) are passed as
@@ -114,6 +115,21 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
              int out_stride, int K, int B, void* stream);
 
 /* Pins the number of K splits of the MFMA path; 0 restores the choice by shape. */
+/* t12_gemm with the last step left to the caller: when the launch splits K across workgroups, the
+ * partial sums stay in the library's per-device workspace and *part describes them,
+ *   value[b, m] = sum over z < nsplit (ascending) of ws[z * split_stride + b * ld + (segment's first column) + m],
+ * so that the caller's next kernel (launch_sum_add_rms_norm_bf16_batch) adds them up while it reads
+ * them anyway.  nsplit == 1: nothing was split, the outputs are complete in segs[].out.  The workspace is
+ * reused by the next t12_gemm* call on the device: consume the partials first (same stream).  No
+ * counterpart in the reference (its GEMM never splits K). */
+typedef struct T12GemmPartials {
+    const float* ws;
+    int          nsplit;
+    int          ld;            /* floats between consecutive batch rows of one split (sum of M over segments) */
+    size_t       split_stride;  /* floats between consecutive splits */
+} T12GemmPartials;
+int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride,
+                      int out_stride, int K, int B, T12GemmPartials* part, void* stream);
 int t12_tune_gemm(int ksplit);
 
 /* ---- (c) standalone decompress --------------------------------------------

@@ -39,6 +39,12 @@ void launch_rms_norm_bf16_batch(const float* x, const float* weight, int16_t* y,
 /* kernels.hip:471-477.  x[b] += residual[b] (stored), then as above. */
 void launch_add_rms_norm_bf16_batch(float* x, const float* residual, const float* weight, int16_t* y, int n, float eps,
                                     int batch_size, hipStream_t stream);
+/* The same, with x[b] first rebuilt as the ascending sum of nsplit partial rows
+ * partials[z * split_stride + b * ld + i] (what t12_gemm_deferred leaves behind): the K-split reduction of
+ * a decode+GEMM folded into the residual add + RMSNorm that follows it.  No counterpart in the reference. */
+void launch_sum_add_rms_norm_bf16_batch(float* x, const float* partials, int nsplit, size_t split_stride, int ld,
+                                        const float* residual, const float* weight, int16_t* y, int n, float eps,
+                                        int batch_size, hipStream_t stream);
 /* kernels.hip:479-485.  out = bf16(silu(gate) * up), [batch, n] contiguous. */
 void launch_silu_mul_bf16_batch(const float* gate, const float* up, int16_t* out, int n, int batch_size,
                                 hipStream_t stream);

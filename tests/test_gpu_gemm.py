@@ -129,3 +129,37 @@ def test_gemm_rejects_bad_operands(t12):
     x = torch.zeros(64, dtype=torch.int16, device=dev())
     assert t12.lib.t12_gemm(segs, 1, x.data_ptr(), 64, 4, 64, 1, None) == -1
     assert t12.lib.t12_gemm(segs, 1, x.data_ptr(), 32, 4, 64, 1, None) == -1
+
+
+@pytest.mark.parametrize("M,K,B", [(512, 4096, 256), (256, 14336, 96), (300, 1024, 40), (4096, 4096, 16)])
+def test_deferred_reduction_into_add_rms_norm_is_bit_identical(t12, oracle, synth, M, K, B):
+    """t12_gemm_deferred leaves the K-split partial sums for launch_sum_add_rms_norm_bf16_batch; the pair must
+    give exactly what t12_gemm + launch_add_rms_norm_bf16_batch give (same summation order)."""
+    p = oracle.pack(synth.weights_llm(M, K, seed=M + B, p_outlier=1e-3))
+    dt = t12.DeviceTensor12.from_packed(p, dev())
+    X = to_dev_bits(synth.activations(B, K, seed=3)).reshape(B, K)
+    g = torch.Generator(device=dev()); g.manual_seed(4)
+    res = torch.randn((B, M), generator=g, device=dev())
+    w = 1 + 0.1 * torch.randn(M, generator=g, device=dev())
+    st = t12.current_stream()
+    # reference pair
+    out_a = torch.empty((B, M), dtype=torch.float32, device=dev())
+    t12.gemm([dt], X, outs=[out_a])
+    y_a = torch.empty((B, M), dtype=torch.int16, device=dev())
+    t12.lib.launch_add_rms_norm_bf16_batch(out_a.data_ptr(), res.data_ptr(), w.data_ptr(), y_a.data_ptr(), M, 1e-5, B, st)
+    # deferred pair
+    out_b = torch.full((B, M), float("nan"), dtype=torch.float32, device=dev())
+    y_b = torch.empty((B, M), dtype=torch.int16, device=dev())
+    part = t12.GemmPartials()
+    segs = t12._seg_array([dt.segment(out_b)])
+    t12.check(t12.lib.t12_gemm_deferred(segs, 1, X.data_ptr(), K, M, K, B, part, st), "t12_gemm_deferred")
+    if part.nsplit > 1:
+        t12.lib.launch_sum_add_rms_norm_bf16_batch(out_b.data_ptr(), part.ws, part.nsplit, part.split_stride, part.ld,
+                                                   res.data_ptr(), w.data_ptr(), y_b.data_ptr(), M, 1e-5, B, st)
+    else:
+        t12.lib.launch_add_rms_norm_bf16_batch(out_b.data_ptr(), res.data_ptr(), w.data_ptr(), y_b.data_ptr(), M, 1e-5, B, st)
+    torch.cuda.synchronize()
+    assert torch.equal(out_a, out_b)
+    assert torch.equal(y_a, y_b)
+    if (M, K, B) == (512, 4096, 256):
+        assert part.nsplit > 1          # this shape does split K: the fused path is the one compared

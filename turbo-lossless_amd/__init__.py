@@ -35,6 +35,11 @@ class PatchBatchDesc(C.Structure):
                 ("patch_wrong", C.c_void_p), ("activations", C.c_void_p), ("output", C.c_void_p), ("M", C.c_int)]
 
 
+class GemmPartials(C.Structure):
+    """Mirror of T12GemmPartials (include/t12_abi.h)."""
+    _fields_ = [("ws", C.c_void_p), ("nsplit", C.c_int), ("ld", C.c_int), ("split_stride", C.c_size_t)]
+
+
 _vp, _i = C.c_void_p, C.c_int
 _SIGS = {
     "t12_version": (C.c_char_p, []),
@@ -95,6 +100,9 @@ _SIGS = {
     "launch_split12_batch8_async": (_i, [_vp] * 2 + [_i] + [_vp] * 8 + [_vp] * 3 + [_vp] * 8 + [_i, _i, _vp]),
     "t12_gemm": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_tune_gemm": (_i, [_i]),
+    "t12_gemm_deferred": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, C.POINTER(GemmPartials), _vp]),
+    "launch_sum_add_rms_norm_bf16_batch": (None, [_vp, _vp, _i, C.c_size_t, _i, _vp, _vp, _vp, _i, C.c_float, _i, _vp]),
+    "t12_util_copy_i32": (_i, [_vp, _vp, _i, _vp]),
     "t12_decompress": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "launch_split12_v2_async": (_i, [_vp, _vp, _i, _vp, _vp, _i, _i, _vp]),
     "launch_split12_v2_dual_async": (_i, [_vp, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _vp]),

@@ -24,6 +24,8 @@ void launch_embed_lookup(const int16_t*, const int*, float*, int, int, int, hipS
 void launch_argmax_batch(const float*, int*, int, int, hipStream_t);
 void launch_rms_norm_bf16_batch(const float*, const float*, int16_t*, int, float, int, hipStream_t);
 void launch_add_rms_norm_bf16_batch(float*, const float*, const float*, int16_t*, int, float, int, hipStream_t);
+void launch_sum_add_rms_norm_bf16_batch(float*, const float*, int, size_t, int, const float*, const float*, int16_t*, int,
+                                        float, int, hipStream_t);
 void launch_silu_mul_bf16_batch(const float*, const float*, int16_t*, int, int, hipStream_t);
 void launch_rope_store_kv_batch(float*, float*, const float*, int8_t*, int8_t*, float*, float*, const int*, int, int,
                                 int, int, int, float, int, hipStream_t);
@@ -91,6 +93,23 @@ void run_linear(const T12Segment* segs, int nseg, const int16_t* act, int K, int
         fprintf(stderr, "ERROR: split-12 linear launch failed: %s\n", t12_last_error());
         exit(1);
     }
+}
+
+// out = W . act, then x = out + residual (stored in out) and y = bf16(RMSNorm(x) * norm_w): the K-split
+// partial sums of the GEMM are added up by the norm kernel itself (one launch less per linear).
+void run_linear_add_norm(const T12Segment* seg, const int16_t* act, int K, int B, const float* residual,
+                         const float* norm_w, float eps, int16_t* y, hipStream_t st)
+{
+    T12GemmPartials part;
+    if (t12_gemm_deferred(seg, 1, act, K, seg->out_stride, K, B, &part, st) != T12_OK) {
+        fprintf(stderr, "ERROR: split-12 linear launch failed: %s\n", t12_last_error());
+        exit(1);
+    }
+    if (part.nsplit > 1)
+        launch_sum_add_rms_norm_bf16_batch(seg->out, part.ws, part.nsplit, part.split_stride, part.ld, residual, norm_w,
+                                           y, seg->M, eps, B, st);
+    else
+        launch_add_rms_norm_bf16_batch(seg->out, residual, norm_w, y, seg->M, eps, B, st);
 }
 
 }  // namespace
@@ -320,8 +339,12 @@ void forward(InferenceState* state, const int* token_ids)
                                     head_dim, c.rope_theta, scale, B, 0, st);
 
         S.o[0] = seg_of(L.wo, res, n);
-        run_linear(S.o, 1, bf16_a, n, B, st);
-        launch_add_rms_norm_bf16_batch(res, cur, L.ffn_norm, bf16_a, n, c.rms_norm_eps, B, st);
+        if (B > 1) {
+            run_linear_add_norm(S.o, bf16_a, n, B, cur, L.ffn_norm, c.rms_norm_eps, bf16_a, st);
+        } else {
+            run_linear(S.o, 1, bf16_a, n, B, st);
+            launch_add_rms_norm_bf16_batch(res, cur, L.ffn_norm, bf16_a, n, c.rms_norm_eps, B, st);
+        }
 
         S.gateup[0] = seg_of(L.w_gate, state->ffn_gate, n_ff);
         S.gateup[1] = seg_of(L.w_up, state->ffn_up, n_ff);
@@ -338,9 +361,13 @@ void forward(InferenceState* state, const int* token_ids)
         }
 
         S.down[0] = seg_of(L.w_down, cur, n);
-        run_linear(S.down, 1, bf16_b, n_ff, B, st);
         const float* next_norm = layer + 1 < c.n_layer ? m->layers[layer + 1].attn_norm : m->output_norm;
-        launch_add_rms_norm_bf16_batch(cur, res, next_norm, bf16_a, n, c.rms_norm_eps, B, st);
+        if (B > 1) {
+            run_linear_add_norm(S.down, bf16_b, n_ff, B, res, next_norm, c.rms_norm_eps, bf16_a, st);
+        } else {
+            run_linear(S.down, 1, bf16_b, n_ff, B, st);
+            launch_add_rms_norm_bf16_batch(cur, res, next_norm, bf16_a, n, c.rms_norm_eps, B, st);
+        }
     }
     if (c.n_layer == 0) launch_rms_norm_bf16_batch(cur, m->output_norm, bf16_a, n, c.rms_norm_eps, B, st);
 

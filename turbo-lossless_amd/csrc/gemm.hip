@@ -560,6 +560,20 @@ int t12_tune_gemm(int ksplit)
 int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride, int out_stride, int K, int B,
              void* stream)
 {
+    return t12_gemm_deferred(segs, nseg, act_bf16, act_stride, out_stride, K, B, nullptr, stream);
+}
+
+// t12_gemm whose K-split partial sums may be left in the workspace for the caller's next kernel to add
+// up (part != NULL): part->nsplit == 1 means the outputs are complete in segs[].out.
+int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride, int out_stride, int K,
+                      int B, T12GemmPartials* part, void* stream)
+{
+    if (part) {
+        part->ws = nullptr;
+        part->nsplit = 1;
+        part->ld = 0;
+        part->split_stride = 0;
+    }
     T12_REQUIRE(segs && nseg >= 1 && nseg <= T12_MAX_SEGMENTS, "t12_gemm: nseg must be 1..%d (got %d)",
                 T12_MAX_SEGMENTS, nseg);
     T12_REQUIRE(act_bf16 && K >= 1 && B >= 1, "t12_gemm: activations null or K/B < 1 (K=%d B=%d)", K, B);
@@ -616,9 +630,9 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
     const int per_cu = B > 64 ? 1 : 2;
     const int want = 256 * per_cu;
     int ks = 1;
-    if (g_gemm_ksplit > 0) ks = g_gemm_ksplit;
+    if (g_gemm_ksplit > 0) ks = g_gemm_ksplit < T12_MAX_KSPLIT ? g_gemm_ksplit : T12_MAX_KSPLIT;
     else
-        while (tiles * btiles * ks * 4 < want * 3 && K / (ks * 2) >= 4 * KC && ks < 16) ks *= 2;
+        while (tiles * btiles * ks * 4 < want * 3 && K / (ks * 2) >= 4 * KC && ks < T12_MAX_KSPLIT) ks *= 2;
     int kslice = (((K + 2 * KC - 1) / (2 * KC) + ks - 1) / ks) * 2 * KC;      // whole windows of two stages
     ks = (K + kslice - 1) / kslice;
     p.ksplit = ks;
@@ -638,7 +652,12 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
     else rc = launch_mfma<4, 2, 2, 2>(p, tiles, st);
     if (rc) return rc;
 
-    if (ks > 1) {
+    if (ks > 1 && part) {
+        part->ws = p.ws;
+        part->nsplit = ks;
+        part->ld = m_total;
+        part->split_stride = (size_t)B * m_total;
+    } else if (ks > 1) {
         hipLaunchKernelGGL(gemm_reduce_kernel, dim3((m_total + 255) / 256, B), dim3(256), 0, st, p);
         T12_CHECK_LAUNCH("t12_gemm(reduce)");
     }

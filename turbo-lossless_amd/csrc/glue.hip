@@ -60,13 +60,35 @@ __global__ __launch_bounds__(256) void embed_kernel(const uint16_t* __restrict__
 // y = bf16(x * rsqrt(mean(x^2) + eps) * w); with ADD: x += residual first, written back
 // (kernels.hip:355-392 and :399-442).  One workgroup per row, values kept in registers
 // between the two passes.
-template <bool ADD>
+// PART: x[row] is first rebuilt as the sum of nsplit partial rows (ascending, the order of the GEMM's
+// own reduction kernel) -- the K-split decode+GEMM leaves them for this kernel to add up.
+template <bool ADD, bool PART = false>
 __global__ __launch_bounds__(1024) void rms_norm_kernel(float* __restrict__ x, const float* __restrict__ res,
                                                         const float* __restrict__ w, uint16_t* __restrict__ y,
-                                                        int n, float eps)
+                                                        int n, float eps, const float* __restrict__ part = nullptr,
+                                                        int nsplit = 0, size_t split_stride = 0, int ld = 0)
 {
     __shared__ float red[17];
     const size_t off = (size_t)blockIdx.x * n;
+    const float* prow = PART ? part + (size_t)blockIdx.x * ld : nullptr;
+    auto value = [&](int i) {
+        float t;
+        if (PART) {
+            // all partial loads of the element in flight together, then the sum in ascending order
+            float pz[T12_MAX_KSPLIT];
+#pragma unroll
+            for (int z = 0; z < T12_MAX_KSPLIT; z++) pz[z] = z < nsplit ? prow[(size_t)z * split_stride + i] : 0.0f;
+            t = 0.0f;
+#pragma unroll
+            for (int z = 0; z < T12_MAX_KSPLIT; z++)
+                if (z < nsplit) t += pz[z];
+        } else {
+            t = x[off + i];
+        }
+        if (ADD) t += res[off + i];
+        if (ADD || PART) x[off + i] = t;
+        return t;
+    };
     constexpr int MAXV = 8;                // up to 8 values per thread in registers (n <= 8 * blockDim)
     float v[MAXV];
     float ss = 0.0f;
@@ -75,21 +97,13 @@ __global__ __launch_bounds__(1024) void rms_norm_kernel(float* __restrict__ x, c
         const int i = threadIdx.x + j * blockDim.x;
         v[j] = 0.0f;
         if (i < n) {
-            float t = x[off + i];
-            if (ADD) {
-                t += res[off + i];
-                x[off + i] = t;
-            }
+            const float t = value(i);
             v[j] = t;
             ss += t * t;
         }
     }
     for (int i = threadIdx.x + MAXV * blockDim.x; i < n; i += blockDim.x) {   // very wide rows
-        float t = x[off + i];
-        if (ADD) {
-            t += res[off + i];
-            x[off + i] = t;
-        }
+        const float t = value(i);
         ss += t * t;
     }
     ss = block_reduce<false>(ss, red);
@@ -742,6 +756,22 @@ void launch_add_rms_norm_bf16_batch(float* x, const float* residual, const float
     hipLaunchKernelGGL(rms_norm_kernel<true>, dim3(batch_size), dim3(norm_threads(n)), 0, stream, x, residual, weight,
                        (uint16_t*)y, n, eps);
     report("add_rms_norm");
+}
+
+// x[b] = (sum of the nsplit partial rows) + residual[b] (stored), y[b] = bf16(RMSNorm(x[b]) * weight):
+// launch_add_rms_norm_bf16_batch fed by the K-split partial sums of t12_gemm_deferred.
+void launch_sum_add_rms_norm_bf16_batch(float* x, const float* partials, int nsplit, size_t split_stride, int ld,
+                                        const float* residual, const float* weight, int16_t* y, int n, float eps,
+                                        int batch_size, hipStream_t stream)
+{
+    if (nsplit < 1 || nsplit > T12_MAX_KSPLIT || !partials) {
+        t12_set_error("sum_add_rms_norm: nsplit %d outside 1..%d or null partials", nsplit, T12_MAX_KSPLIT);
+        fprintf(stderr, "turbo12: %s\n", t12_last_error());
+        return;
+    }
+    hipLaunchKernelGGL((rms_norm_kernel<true, true>), dim3(batch_size), dim3(norm_threads(n)), 0, stream, x, residual,
+                       weight, (uint16_t*)y, n, eps, partials, nsplit, split_stride, ld);
+    report("sum_add_rms_norm");
 }
 
 void launch_silu_mul_bf16_batch(const float* gate, const float* up, int16_t* out, int n, int batch_size,
