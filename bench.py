@@ -10,16 +10,16 @@ Workloads (synthetic, seeded, random-init weights of the Llama-3.1-8B shape:
   decode (default) one step = one greedy decode step of the full engine (embedding, 32 x [RMSNorm, fused
                   QKV decode-GEMV, RoPE + INT8 KV store, GQA attention, O, add+RMSNorm, fused gate|up,
                   SiLU*mul, down, add+RMSNorm], lm_head, argmax + D2H) on a model generated and packed on
-                  the GPU; prompt 128 random ids, 2048-token KV cache (BASELINE config 4).  B = 1 is
+                  the GPU; prompt 128 random ids, 2048-token KV cache.  B = 1 is
                   `value`; B = 256 is measured in the same run and reported under "b256"; the
                   decode-GEMV launches of a step are also timed alone for `roofline`.
 
   gemm_layers     the four linear-layer shapes through the fused decode+GEMM at B = 16, 64, 256 on three
-                  rotating weight copies (BASELINE config 2); `roofline` prices gate|up at B = 256 against
+                  rotating weight copies; `roofline` prices gate|up at B = 256 against
                   the 2.5 PFLOP/s dense bf16 MFMA peak.
 
   moe             one step = one Mixtral-8x7B-shaped MoE FFN layer (8 split-12 experts, top-2) over 256 tokens
-                  grouped per expert through the decode+GEMM (BASELINE config 5).
+                  grouped per expert through the decode+GEMM.
 
   gemv_stack_b1   one step = every linear layer of one decode step at B = 1 through
                   the fused split-12 decode-GEMV: per layer QKV (3 segments, one
@@ -152,7 +152,7 @@ def timed(torch, stream, fn, steps):
 
 def run_decode(args, t12, torch, dev):
     """Full greedy decode on a random-init Llama-3.1-8B-shaped model generated and packed on the GPU
-    (BASELINE config 4): prompt of 128 random ids, 2048-token KV cache, one forward + one greedy sample
+    prompt of 128 random ids, 2048-token KV cache, one forward + one greedy sample
     per step; B = 1 is `value`, B = 256 (256 lock-step copies sharing the cache, the reference's batched
     mode) is reported next to it."""
     import numpy as np
@@ -282,7 +282,7 @@ def run_decode(args, t12, torch, dev):
 
 
 def run_moe(args, t12, torch, dev):
-    """Mixtral-8x7B-shaped MoE FFN layer (BASELINE config 5): 8 experts x (4096 -> 14336 -> 4096, SwiGLU),
+    """Mixtral-8x7B-shaped MoE FFN layer: 8 experts x (4096 -> 14336 -> 4096, SwiGLU),
     256 tokens, top-2 routing from random router logits; one step = the whole layer."""
     import importlib
     moe = importlib.import_module("turbo_lossless_amd.moe")
@@ -320,7 +320,7 @@ def run_moe(args, t12, torch, dev):
 
 
 def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(16, 64, 256), iters=10):
-    """decode+GEMM per layer shape (BASELINE config 2): for each B, each of QKV (3 segments), O, gate|up
+    """decode+GEMM per layer shape: for each B, each of QKV (3 segments), O, gate|up
     (2 segments), down is timed over `n_rot` distinct weight copies in rotation, so that neither L2 nor
     the 256 MB last-level cache holds a tensor between launches.  weight_of(copy, which) -> (segment, K, P)."""
     out = {}
@@ -356,8 +356,8 @@ def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(16, 
 
 
 def run_gemm_layers(args, t12, torch, dev):
-    """The four Llama-3.1-8B linear-layer shapes through the fused decode+GEMM at B = 16, 64, 256 (BASELINE
-    config 2) on three rotating weight copies; one step = the four layer GEMMs of one decoder layer at B = 256."""
+    """The four Llama-3.1-8B linear-layer shapes through the fused decode+GEMM at B = 16, 64, 256 on three
+    rotating weight copies; one step = the four layer GEMMs of one decoder layer at B = 256."""
     cfg = dict(LLAMA8B)
     n, ff = cfg["n_embd"], cfg["n_ff"]
     kv = cfg["n_head_kv"] * (n // cfg["n_head"])

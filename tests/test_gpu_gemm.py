@@ -1,7 +1,7 @@
 """GPU parity: split-12 decode+GEMM (bf16 MFMA, fp32 accumulate) through the C ABI vs the
 CPU oracle's decode-then-fp32-accumulate GEMM.
 
-Tolerance: north star 1e-2 relative; both sides multiply bf16 x bf16 exactly and accumulate
+Tolerance: the target is 1e-2 relative; both sides multiply bf16 x bf16 exactly and accumulate
 in fp32, so the observed error is ~1e-6 and the assertions use 1e-4.
 """
 import importlib

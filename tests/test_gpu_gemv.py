@@ -1,6 +1,6 @@
 """GPU parity: split-12 decode-GEMV (B = 1) through the C ABI vs the CPU oracle.
 
-Tolerance: BASELINE north star -- outputs within 1e-2 relative of the
+Tolerance: the target is outputs within 1e-2 relative of the
 decode-then-fp32-accumulate reference.  The kernels accumulate in fp32 like the
 oracle, so the observed error is ~1e-6; the assertions use 1e-4 to catch a wrong
 pairing / dropped tile, which would show at 1e-2..1.
@@ -40,7 +40,7 @@ def test_gemv_llm_law(t12, oracle, synth, M, K):
 
 
 def test_gemv_config1_escape_statistics(t12, oracle, synth):
-    """BASELINE config 1: 4096x4096 N(0,.02) + 0.03 % N(0,8) outliers."""
+    """Single-tensor case: 4096x4096 N(0,.02) + 0.03 % N(0,8) outliers."""
     w = synth.weights_llm(4096, 4096, seed=1001)
     x = synth.activations(1, 4096, seed=1002)[0]
     p = oracle.pack(w)
@@ -55,7 +55,7 @@ def test_gemv_config1_escape_statistics(t12, oracle, synth):
 
 
 def test_gemv_escape_heavy(t12, oracle, synth):
-    """BASELINE config 3 law: every row holds several escapes."""
+    """Diffusion-UNet-like weight law: every row holds several escapes."""
     for (M, K) in [(1280, 5120), (640, 1280)]:
         w = synth.weights_diffusion(M, K, seed=3000 + M)
         x = synth.activations(1, K, seed=3001)[0]

@@ -2,7 +2,7 @@
 through the decode+GEMM) -- small layer against the CPU oracle, full-size layer against a
 decode-then-fp32 matmul of the same (bit-exact, separately tested) decoded weights.
 
-Tolerance: 1e-2 relative (north star); observed ~1e-5 (fp32 accumulation order only; the
+Tolerance: 1e-2 relative (the target); observed ~1e-5 (fp32 accumulation order only; the
 SwiGLU activation is rounded to bf16 on both sides, as the engine does between the two GEMMs).
 """
 import importlib
