@@ -163,3 +163,22 @@ def test_deferred_reduction_into_add_rms_norm_is_bit_identical(t12, oracle, synt
     assert torch.equal(y_a, y_b)
     if (M, K, B) == (512, 4096, 256):
         assert part.nsplit > 1          # this shape does split K: the fused path is the one compared
+
+
+@pytest.mark.parametrize("B", [16, 64, 128, 256])
+def test_gemm_more_escapes_than_the_lds_list_holds(t12, oracle, synth, B):
+    """A 128-row tile with ~10 k escapes overflows the in-LDS escape list (1536 / 2048 entries): the kernel then
+    multiplies the unpatched values and adds (correct - wrong) * x per entry in its epilogue -- still exact to
+    fp32 rounding, with and without a K split."""
+    M, K = 256, 4096
+    p = oracle.pack(synth.weights_llm(M, K, seed=77, p_outlier=3e-2))
+    assert p.P > 2 * 4096                       # > 2048 entries in every 128-row tile
+    X = synth.activations(B, K, seed=B + 1)
+    ref = oracle.gemm(p, X)
+    try:
+        for ks in (0, 1, 4):
+            t12.lib.t12_tune_gemm(ks)
+            (got,) = run_gemm(t12, [p], X)
+            assert rel_err(got, ref) < TOL, ks
+    finally:
+        t12.lib.t12_tune_gemm(0)
