@@ -385,6 +385,39 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
     const float* skb = sk + (size_t)b * sstride + kvh;
     const float* svb = sv + (size_t)b * sstride + kvh;
     const float* qb = q + (size_t)b * n_head * HD + (size_t)kvh * RATIO * HD;
+
+    // The cache rows of the first tile are requested before anything else, so that their HBM latency
+    // runs under the Q / new-K / new-V work instead of behind it: this lane's K row (phase 1) into
+    // registers and, in the FUSE variant, the V tile through registers into LDS (phase 3 reads it from
+    // there).  The row of the position being written (FUSE) is not in memory yet: it comes from LDS.
+    constexpr int VPRE = FUSE ? (ATT_TILE * CH) / 256 : 0;          // 16-byte V pieces per thread
+    __shared__ __attribute__((aligned(16))) int8_t vt[FUSE ? ATT_TILE * HD : 16];
+    __shared__ float vts[FUSE ? ATT_TILE : 1];
+    __shared__ __attribute__((aligned(16))) int8_t knew8[FUSE ? HD : 16];
+    __shared__ float knew_scale;
+    const int tl0 = min(ATT_TILE, seq_len);
+    const int newpos = FUSE ? seq_len - 1 : -1;
+    const bool kpre = tid < tl0 && tid != newpos;
+    uint4 kk_pre[CH];
+    float kscale_pre = 0.0f;
+    if (kpre) {
+        const uint4* kr = (const uint4*)(kbase + (size_t)tid * kv_dim);
+#pragma unroll
+        for (int u = 0; u < CH; u++) kk_pre[u] = kr[u];
+        kscale_pre = skb[(size_t)tid * n_head_kv] * scale;
+    }
+    uint4 v_pre[VPRE > 0 ? VPRE : 1];
+    float vs_pre = 0.0f;
+    if (FUSE) {
+#pragma unroll
+        for (int x = 0; x < VPRE; x++) {
+            const int idx = tid + 256 * x, t = idx / CH, u = idx % CH;
+            v_pre[x] = make_uint4(0, 0, 0, 0);
+            if (t < tl0 && t != newpos) v_pre[x] = *(const uint4*)(vbase + (size_t)t * kv_dim + u * 16);
+        }
+        if (tid < tl0 && tid != newpos) vs_pre = svb[(size_t)tid * n_head_kv];
+    }
+
     if (!FUSE) {
         for (int i = tid; i < RATIO * HD; i += 256) qs[i] = qb[i];
     } else {
@@ -416,14 +449,33 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
             const float amax = wave_max(fmaxf(fabsf(r0), fabsf(r1)));
             const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
             int8_t* row = (wave == 0 ? fz.ck_w : fz.cv_w) + (size_t)b * kv_stride + (size_t)pos * kv_dim + (size_t)kvh * HD;
+            const int8_t q0 = (int8_t)(int)fminf(fmaxf(rintf(r0 * inv), -127.0f), 127.0f);
+            const int8_t q1 = (int8_t)(int)fminf(fmaxf(rintf(r1 * inv), -127.0f), 127.0f);
+            // the new row: to the cache, and (first tile) to LDS where this launch reads it
+            int8_t* lrow = wave == 0 ? knew8 : vt + (size_t)(pos < ATT_TILE ? pos : 0) * HD;
+            const bool to_lds = wave == 0 || pos < ATT_TILE;
             if (own) {
-                row[lane] = (int8_t)(int)fminf(fmaxf(rintf(r0 * inv), -127.0f), 127.0f);
-                row[lane + HALF] = (int8_t)(int)fminf(fmaxf(rintf(r1 * inv), -127.0f), 127.0f);
+                row[lane] = q0;
+                row[lane + HALF] = q1;
+                if (to_lds) {
+                    lrow[lane] = q0;
+                    lrow[lane + HALF] = q1;
+                }
             }
-            if (lane == 0)
+            if (lane == 0) {
                 (wave == 0 ? fz.sk_w : fz.sv_w)[(size_t)b * sstride + (size_t)pos * n_head_kv + kvh] = amax / 127.0f;
+                if (wave == 0) knew_scale = amax / 127.0f;
+                else if (pos < ATT_TILE) vts[pos] = amax / 127.0f;
+            }
         }
-        __threadfence();      // the new row is read back through the cache pointers below
+        __threadfence();      // later tiles read the new row back through the cache pointers
+        // the prefetched V tile: registers -> LDS (row-major, 16-byte pieces)
+#pragma unroll
+        for (int x = 0; x < VPRE; x++) {
+            const int idx = tid + 256 * x, t = idx / CH;
+            if (t < tl0 && t != newpos) ((uint4*)vt)[idx] = v_pre[x];
+        }
+        if (tid < tl0 && tid != newpos) vts[tid] = vs_pre;
     }
     __syncthreads();
 
@@ -442,11 +494,22 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
         // ---- phase 1
         if (tid < tl) {
             const int t = t0 + tid;
-            const uint4* kr = (const uint4*)(kbase + (size_t)t * kv_dim);
             uint4 kk[CH];
+            float kscale;
+            if (t0 == 0 && kpre) {
 #pragma unroll
-            for (int u = 0; u < CH; u++) kk[u] = kr[u];
-            const float kscale = skb[(size_t)t * n_head_kv] * scale;
+                for (int u = 0; u < CH; u++) kk[u] = kk_pre[u];
+                kscale = kscale_pre;
+            } else if (FUSE && t == newpos && t0 == 0) {
+#pragma unroll
+                for (int u = 0; u < CH; u++) kk[u] = ((const uint4*)knew8)[u];
+                kscale = knew_scale * scale;
+            } else {
+                const uint4* kr = (const uint4*)(kbase + (size_t)t * kv_dim);
+#pragma unroll
+                for (int u = 0; u < CH; u++) kk[u] = kr[u];
+                kscale = skb[(size_t)t * n_head_kv] * scale;
+            }
             float dot[RATIO];
 #pragma unroll
             for (int h = 0; h < RATIO; h++) dot[h] = 0.0f;
@@ -503,8 +566,13 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
                         const int t = (it + x) * PG + g;
                         const bool ok = t < tl;
                         const int tc = ok ? t : 0;
-                        vv[x] = *(const uint4*)(vbase + (size_t)(t0 + tc) * kv_dim + c * 16);
-                        w[x] = ok ? ph[tc] * svb[(size_t)(t0 + tc) * n_head_kv] : 0.0f;
+                        if (FUSE && t0 == 0) {
+                            vv[x] = ((const uint4*)vt)[tc * CH + c];
+                            w[x] = ok ? ph[tc] * vts[tc] : 0.0f;
+                        } else {
+                            vv[x] = *(const uint4*)(vbase + (size_t)(t0 + tc) * kv_dim + c * 16);
+                            w[x] = ok ? ph[tc] * svb[(size_t)(t0 + tc) * n_head_kv] : 0.0f;
+                        }
                     }
 #pragma unroll
                     for (int x = 0; x < 4; x++) {
