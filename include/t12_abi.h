@@ -81,6 +81,11 @@ int t12_tune_gemv(int variant);
  * array (it travels as a kernel argument; no device copy is made). */
 int t12_gemv(const T12Segment* segs, int nseg, const void* act_bf16, int K, void* stream);
 
+/* out[m] = residual[m] + W[m,:] . act (one segment): the residual add that follows wo / w_down
+ * (first half of add_rms_norm_bf16_batch, engine/kernels.hip:399-442, inference.cpp:301,343) folded into
+ * the store of the decode-GEMV.  out and residual may not alias. */
+int t12_gemv_add(const T12Segment* seg, const void* act_bf16, int K, const float* residual, void* stream);
+
 /* SwiGLU front half in one launch: out_bf16[m] = bf16( silu(gate[m,:].x) * (up[m,:].x) ).
  * Replaces launch_split12_v2_dual_async (decompress_v2.hip:549) + its patch launch +
  * launch_silu_mul_bf16_batch (engine/kernels.hip:480); bit-identical to that sequence.

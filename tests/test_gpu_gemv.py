@@ -301,3 +301,22 @@ def test_gemv_norm_prologue(t12, oracle, synth, K, with_res):
     # aliasing is rejected
     if with_res:
         assert t12.lib.t12_gemv_norm(segs, 2, xd.data_ptr(), rd.data_ptr(), wd.data_ptr(), 1e-5, xd.data_ptr(), K, st) == -1
+
+
+@pytest.mark.parametrize("M,K", [(4096, 4096), (300, 14336), (77, 1040), (9, 15)])
+def test_gemv_add_is_bit_identical_to_gemv_plus_add(t12, oracle, synth, M, K):
+    """t12_gemv_add folds the residual add into the store: out = residual + W.x with the same single fp32 add
+    the separate kernel does (the odd-K case runs the general kernel)."""
+    p = oracle.pack(synth.weights_llm(M, K, seed=M * 3 + K, p_outlier=2e-3))
+    dt = t12.DeviceTensor12.from_packed(p, dev())
+    x = to_dev_bits(synth.activations(1, K, seed=9)[0])
+    g = torch.Generator(device=dev()); g.manual_seed(M)
+    res = torch.randn(M, generator=g, device=dev())
+    (plain,) = t12.gemv([dt], x)
+    want = plain + res
+    out = torch.full((M,), float("nan"), dtype=torch.float32, device=dev())
+    segs = t12._seg_array([dt.segment(out)])
+    t12.check(t12.lib.t12_gemv_add(segs, x.data_ptr(), K, res.data_ptr(), t12.current_stream()), "t12_gemv_add")
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    assert t12.lib.t12_gemv_add(segs, x.data_ptr(), K, None, t12.current_stream()) == -1

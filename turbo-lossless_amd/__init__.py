@@ -92,6 +92,7 @@ _SIGS = {
     "t12_engine_decode": (_i, [_vp, _i, _i, C.POINTER(C.c_int)]),
     "t12_engine_sync": (_i, [_vp]),
     "t12_engine_weight": (_i, [_vp, _i, _i, C.POINTER(Segment), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "t12_gemv_add": (_i, [C.POINTER(Segment), _vp, _i, _vp, _vp]),
     "t12_gemv_swiglu": (_i, [C.POINTER(Segment), C.POINTER(Segment), _vp, _i, _vp, _vp]),
     "t12_gemv_norm": (_i, [C.POINTER(Segment), _i, _vp, _vp, _vp, C.c_float, _vp, _i, _vp]),
     "t12_gemv_swiglu_norm": (_i, [C.POINTER(Segment), C.POINTER(Segment), _vp, _vp, _vp, C.c_float, _vp, _i, _vp, _vp]),

@@ -209,11 +209,11 @@ void must(int rc, const char* what)
 }
 
 // B = 1 decode step in 5 launches per layer:
-//   [RMSNorm (+ residual add)] + wq|wk|wv      t12_gemv_norm
+//   RMSNorm + wq|wk|wv                          t12_gemv_norm
 //   RoPE + INT8 KV store + GQA attention        launch_rope_store_attention
-//   wo                                          t12_gemv
-//   residual add + RMSNorm + gate|up + SiLU*mul t12_gemv_swiglu_norm
-//   w_down                                      t12_gemv
+//   wo + residual add                           t12_gemv_add
+//   RMSNorm + gate|up + SiLU*mul                t12_gemv_swiglu_norm
+//   w_down + residual add                       t12_gemv_add
 // The residual stream ping-pongs between hidden and hidden2 (a norm prologue reads one and
 // workgroup 0 writes the sum into the other); the additions the reference does in
 // add_rms_norm_bf16_batch (inference.cpp:301,341-346) happen in the prologue of the next linear.
@@ -231,13 +231,10 @@ void forward_b1_fused(InferenceState* state, const int* token_ids)
     if (token_ids) (void)hipMemcpyAsync(state->d_tokens, token_ids, sizeof(int), hipMemcpyHostToDevice, st);
     launch_embed_lookup(m->token_embd, state->d_tokens, state->hidden, n, 1, c.n_vocab, st);
 
-    float* h = state->hidden;          // residual stream
+    float* h = state->hidden;          // residual stream (always complete: wo / w_down add it in their store)
     float* h_alt = state->hidden2;
-    float* o_out = state->attn_out;    // output of wo
-    float* d_out = state->ffn_down;    // output of w_down (pending addition)
     int16_t* bf16_a = state->bf16_act;
     int16_t* bf16_b = state->bf16_act2;
-    const float* pending = nullptr;    // residual not yet added into h
 
     for (int layer = 0; layer < c.n_layer; layer++) {
         TransformerLayer& L = m->layers[layer];
@@ -245,9 +242,7 @@ void forward_b1_fused(InferenceState* state, const int* token_ids)
         S.qkv[0] = seg_of(L.wq, state->q_buf, n);
         S.qkv[1] = seg_of(L.wk, state->k_buf, kv_dim);
         S.qkv[2] = seg_of(L.wv, state->v_buf, kv_dim);
-        must(t12_gemv_norm(S.qkv, 3, h, pending, L.attn_norm, c.rms_norm_eps, pending ? h_alt : nullptr, n, st),
-             "qkv decode-GEMV");
-        if (pending) std::swap(h, h_alt);
+        must(t12_gemv_norm(S.qkv, 3, h, nullptr, L.attn_norm, c.rms_norm_eps, nullptr, n, st), "qkv decode-GEMV");
 
         const size_t kv_off = (size_t)layer * m->max_seq_len * kv_dim;
         const size_t sc_off = (size_t)layer * m->max_seq_len * c.n_head_kv;
@@ -255,28 +250,27 @@ void forward_b1_fused(InferenceState* state, const int* token_ids)
                                     m->kv_cache_v + kv_off, m->kv_scale_k + sc_off, m->kv_scale_v + sc_off, bf16_a,
                                     nullptr, pos, c.n_head, c.n_head_kv, head_dim, c.rope_theta, scale, 1, 0, st);
 
-        S.o[0] = seg_of(L.wo, o_out, n);
-        must(t12_gemv(S.o, 1, bf16_a, n, st), "wo decode-GEMV");
+        S.o[0] = seg_of(L.wo, h_alt, n);
+        must(t12_gemv_add(S.o, bf16_a, n, h, st), "wo decode-GEMV");                  // h_alt = h + wo . attn
+        std::swap(h, h_alt);
 
         S.gateup[0] = seg_of(L.w_gate, nullptr, n_ff);
         S.gateup[1] = seg_of(L.w_up, nullptr, n_ff);
-        must(t12_gemv_swiglu_norm(&S.gateup[0], &S.gateup[1], h, o_out, L.ffn_norm, c.rms_norm_eps, h_alt, n, bf16_b, st),
+        must(t12_gemv_swiglu_norm(&S.gateup[0], &S.gateup[1], h, nullptr, L.ffn_norm, c.rms_norm_eps, nullptr, n, bf16_b, st),
              "gate|up decode-GEMV");
-        std::swap(h, h_alt);
 
-        S.down[0] = seg_of(L.w_down, d_out, n);
-        must(t12_gemv(S.down, 1, bf16_b, n_ff, st), "w_down decode-GEMV");
-        pending = d_out;
+        S.down[0] = seg_of(L.w_down, h_alt, n);
+        must(t12_gemv_add(S.down, bf16_b, n_ff, h, st), "w_down decode-GEMV");         // h_alt = h + w_down . ffn
+        std::swap(h, h_alt);
     }
     impl->head[0] = seg_of(m->output_proj, state->logits, c.n_vocab);
     if (c.n_vocab >= 32768) {
         // thousands of workgroups would each rebuild the normalised activations: one small kernel
         // does it once instead (measured: 7 + 114 us against 139 us for the 128256-row head)
-        if (pending) launch_add_rms_norm_bf16_batch(h, pending, m->output_norm, bf16_a, n, c.rms_norm_eps, 1, st);
-        else launch_rms_norm_bf16_batch(h, m->output_norm, bf16_a, n, c.rms_norm_eps, 1, st);
+        launch_rms_norm_bf16_batch(h, m->output_norm, bf16_a, n, c.rms_norm_eps, 1, st);
         must(t12_gemv(impl->head, 1, bf16_a, n, st), "lm_head decode-GEMV");
     } else {
-        must(t12_gemv_norm(impl->head, 1, h, pending, m->output_norm, c.rms_norm_eps, nullptr, n, st),
+        must(t12_gemv_norm(impl->head, 1, h, nullptr, m->output_norm, c.rms_norm_eps, nullptr, n, st),
              "lm_head decode-GEMV");
     }
     state->positions[0] = pos + 1;

@@ -28,6 +28,7 @@ struct GemvParams {
     int K;
     const uint16_t* act;
     uint16_t* out_bf16;                    // SwiGLU mode only
+    const float* add;                      // out[m] = add[m] + sum (single segment), or null
     // RMSNorm prologue (NORM > 0): activations = bf16(rmsnorm(nx [+ nres]) * nw)
     const float* nx;
     const float* nres;
@@ -285,7 +286,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
                 v += (t12_bf16_to_f32((uint16_t)SEG(r).correct[q]) - t12_bf16_to_f32((uint16_t)SEG(r).wrong[q])) *
                      lds_act_at(lds_act, SEG(r).cols[q]);
             tot[r] = t12_wave_sum_lane63(v);
-            if (!SWIGLU && lane == 63) sg.out[row0 + r] = tot[r];
+            if (!SWIGLU && lane == 63) sg.out[row0 + r] = p.add ? tot[r] + p.add[row0 + r] : tot[r];
         }
     }
     if (SWIGLU && lane == 63) {
@@ -323,7 +324,7 @@ __global__ __launch_bounds__(256) void gemv_general_kernel(const GemvParams p)
     }
     acc += patch_partial<false>(sg, row, lane, p.act);
     acc = t12_wave_sum(acc);
-    if (lane == 0) sg.out[row] = acc;
+    if (lane == 0) sg.out[row] = p.add ? acc + p.add[row] : acc;
 }
 
 // Only the escape corrections (the reference's separate patch kernels).
@@ -425,6 +426,8 @@ int validate(const T12Segment* segs, int nseg, const void* act, int K, bool need
     return T12_OK;
 }
 
+int gemv_impl(const T12Segment* segs, int nseg, const void* act_bf16, int K, const float* add, void* stream);
+
 }  // namespace
 
 extern "C" {
@@ -438,6 +441,23 @@ int t12_tune_gemv(int variant)
 
 int t12_gemv(const T12Segment* segs, int nseg, const void* act_bf16, int K, void* stream)
 {
+    return gemv_impl(segs, nseg, act_bf16, K, nullptr, stream);
+}
+
+// out[m] = residual[m] + W[m,:] . act : the residual add that follows wo / w_down in a decoder layer
+// (the first half of add_rms_norm_bf16_batch, engine/kernels.hip:399-442) folded into the GEMV's store.
+int t12_gemv_add(const T12Segment* seg, const void* act_bf16, int K, const float* residual, void* stream)
+{
+    T12_REQUIRE(residual, "t12_gemv_add: residual is null");
+    return gemv_impl(seg, 1, act_bf16, K, residual, stream);
+}
+
+}  // extern "C"
+
+namespace {
+
+int gemv_impl(const T12Segment* segs, int nseg, const void* act_bf16, int K, const float* add, void* stream)
+{
     int rc = validate(segs, nseg, act_bf16, K, true);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
@@ -446,6 +466,7 @@ int t12_gemv(const T12Segment* segs, int nseg, const void* act_bf16, int K, void
     p.K = K;
     p.act = (const uint16_t*)act_bf16;
     p.out_bf16 = nullptr;
+    p.add = add;
     bool fast = (K % 16 == 0) && ((K + 1023) / 1024 * 2048 <= 160 * 1024);
     for (int i = 0; i < nseg; i++) {
         p.seg[i] = segs[i];
@@ -492,6 +513,10 @@ int t12_gemv(const T12Segment* segs, int nseg, const void* act_bf16, int K, void
     }
 }
 
+}  // namespace
+
+extern "C" {
+
 // out_bf16[m] = bf16( silu(gate[m,:].x) * (up[m,:].x) ), escapes exact, one launch.
 int t12_gemv_swiglu(const T12Segment* gate, const T12Segment* up, const void* act_bf16, int K, void* out_bf16,
                     void* stream)
@@ -511,6 +536,7 @@ int t12_gemv_swiglu(const T12Segment* gate, const T12Segment* up, const void* ac
     p.K = K;
     p.act = (const uint16_t*)act_bf16;
     p.out_bf16 = (uint16_t*)out_bf16;
+    p.add = nullptr;
     return launch_swiglu<0>(p, (hipStream_t)stream);
 }
 
@@ -528,6 +554,7 @@ int t12_gemv_norm(const T12Segment* segs, int nseg, const float* x, const float*
     p.K = K;
     p.act = nullptr;
     p.out_bf16 = nullptr;
+    p.add = nullptr;
     p.nx = x;
     p.nres = residual;
     p.nw = norm_w;
@@ -554,6 +581,7 @@ int t12_gemv_swiglu_norm(const T12Segment* gate, const T12Segment* up, const flo
     p.K = K;
     p.act = nullptr;
     p.out_bf16 = (uint16_t*)out_bf16;
+    p.add = nullptr;
     p.nx = x;
     p.nres = residual;
     p.nw = norm_w;
