@@ -115,18 +115,20 @@ def cpu_baseline(torch, launches, cfg, runs=3, n_weights_model=None):
     rng = np.random.default_rng(7)
     xs = {K: oracle.f32_to_bf16_bits(rng.standard_normal(K).astype(np.float32)) for K in {p.K for p in packs}}
     times = []
-    for _ in range(runs):
+    t_begin = time.perf_counter()
+    while len(times) < runs or (time.perf_counter() - t_begin < 10.0 and len(times) < 2000):   # ~10 s of CPU work
         t0 = time.perf_counter()
         for p in packs:
             oracle.gemv(p, xs[p.K])
         times.append(time.perf_counter() - t0)
+    runs = len(times)
     t_layer = sorted(times)[len(times) // 2]
     w_layer = sum(p.M * p.K for p in packs)
     w_model = n_weights_model or sum(t.M * t.K for tensors, _ in launches for t in tensors)
     t_model = t_layer * w_model / w_layer
     return {
         "value": 1.0 / t_model, "unit": "tok/s", "cores": oracle.num_threads(), "kind": "port",
-        "sample": "decoder layer 0 (wq,wk,wv,wo,gate,up,down = %d weights) x%d runs, median %.3f s, scaled by weight "
+        "sample": "decoder layer 0 (wq,wk,wv,wo,gate,up,down = %d weights) x%d runs (~10 s), median %.4f s, scaled by weight "
                   "count to the %d-weight model; %.2f GB/s compressed" % (w_layer, runs, t_layer, w_model,
                                                                           1.5 * w_layer / t_layer / 1e9),
     }

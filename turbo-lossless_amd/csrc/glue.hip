@@ -386,10 +386,9 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
     const float* svb = sv + (size_t)b * sstride + kvh;
     const float* qb = q + (size_t)b * n_head * HD + (size_t)kvh * RATIO * HD;
 
-    // The cache rows of the first tile are requested before anything else, so that their HBM latency
-    // runs under the Q / new-K / new-V work instead of behind it: this lane's K row (phase 1) into
-    // registers and, in the FUSE variant, the V tile through registers into LDS (phase 3 reads it from
-    // there).  The row of the position being written (FUSE) is not in memory yet: it comes from LDS.
+    // FUSE: the cache rows of the first tile are requested before anything else, so that their HBM
+    // latency runs under the Q / new-K / new-V work instead of behind it: this lane's K row (phase 1)
+    // into registers and the V tile through registers into LDS (phase 3 reads it from there).  The row of the position being written (FUSE) is not in memory yet: it comes from LDS.
     constexpr int VPRE = FUSE ? (ATT_TILE * CH) / 256 : 0;          // 16-byte V pieces per thread
     __shared__ __attribute__((aligned(16))) int8_t vt[FUSE ? ATT_TILE * HD : 16];
     __shared__ float vts[FUSE ? ATT_TILE : 1];
@@ -397,7 +396,7 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
     __shared__ float knew_scale;
     const int tl0 = min(ATT_TILE, seq_len);
     const int newpos = FUSE ? seq_len - 1 : -1;
-    const bool kpre = tid < tl0 && tid != newpos;
+    const bool kpre = FUSE && tid < tl0 && tid != newpos;    // (many small workgroups per CU without FUSE: the registers cost more than the latency)
     uint4 kk_pre[CH];
     float kscale_pre = 0.0f;
     if (kpre) {
