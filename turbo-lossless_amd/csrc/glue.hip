@@ -836,7 +836,11 @@ void launch_sum_add_rms_norm_bf16_batch(float* x, const float* partials, int nsp
         fprintf(stderr, "turbo12: %s\n", t12_last_error());
         return;
     }
-    hipLaunchKernelGGL((rms_norm_kernel<true, true>), dim3(batch_size), dim3(norm_threads(n)), 0, stream, x, residual,
+    // one workgroup per row has every partial of the row to fetch: as many lanes as the row allows
+    int threads = (n + 1) / 2;
+    threads = (threads + 63) / 64 * 64;
+    threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
+    hipLaunchKernelGGL((rms_norm_kernel<true, true>), dim3(batch_size), dim3(threads), 0, stream, x, residual,
                        weight, (uint16_t*)y, n, eps, partials, nsplit, split_stride, ld);
     report("sum_add_rms_norm");
 }
