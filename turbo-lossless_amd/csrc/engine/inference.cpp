@@ -35,6 +35,9 @@ void launch_attention_all_heads(const float*, const int8_t*, const int8_t*, cons
                                 int, int, int, int, float, hipStream_t);
 void launch_attention_all_heads_batch(const float*, const int8_t*, const int8_t*, const float*, const float*, int16_t*,
                                       const int*, int, int, int, int, float, int, int, hipStream_t);
+void launch_rope_store_attention_partials(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int16_t*,
+                                          const int*, int, int, int, int, float, float, int, const float*, int, size_t,
+                                          int, hipStream_t);
 void launch_rope_store_attention(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int16_t*, const int*,
                                  int, int, int, int, float, float, int, int, hipStream_t);
 }
@@ -322,15 +325,31 @@ void forward(InferenceState* state, const int* token_ids)
         S.qkv[0] = seg_of(L.wq, state->q_buf, n);
         S.qkv[1] = seg_of(L.wk, state->k_buf, kv_dim);
         S.qkv[2] = seg_of(L.wv, state->v_buf, kv_dim);
-        run_linear(S.qkv, 3, bf16_a, n, B, st);
+        T12GemmPartials qkv_part = {nullptr, 1, 0, 0};
+        if (B > 1) {
+            // a K-split q | k | v projection leaves its partial sums to the RoPE / KV-store kernel
+            if (t12_gemm_deferred(S.qkv, 3, bf16_a, n, n, n, B, &qkv_part, st) != T12_OK) {
+                fprintf(stderr, "ERROR: split-12 linear launch failed: %s\n", t12_last_error());
+                exit(1);
+            }
+        } else {
+            run_linear(S.qkv, 3, bf16_a, n, B, st);
+        }
 
         const size_t kv_off = (size_t)layer * m->max_seq_len * kv_dim;
         const size_t sc_off = (size_t)layer * m->max_seq_len * c.n_head_kv;
-        // RoPE (Q, K) + INT8 KV store + GQA attention: one launch
-        launch_rope_store_attention(state->q_buf, state->k_buf, state->v_buf, m->kv_cache_k + kv_off,
-                                    m->kv_cache_v + kv_off, m->kv_scale_k + sc_off, m->kv_scale_v + sc_off, bf16_a,
-                                    B == 1 ? nullptr : state->d_positions, state->positions[0], c.n_head, c.n_head_kv,
-                                    head_dim, c.rope_theta, scale, B, 0, st);
+        // RoPE (Q, K) + INT8 KV store + GQA attention
+        if (qkv_part.nsplit > 1)
+            launch_rope_store_attention_partials(state->q_buf, state->k_buf, state->v_buf, m->kv_cache_k + kv_off,
+                                                 m->kv_cache_v + kv_off, m->kv_scale_k + sc_off, m->kv_scale_v + sc_off,
+                                                 bf16_a, state->d_positions, state->positions[0], c.n_head, c.n_head_kv,
+                                                 head_dim, c.rope_theta, scale, B, qkv_part.ws, qkv_part.nsplit,
+                                                 qkv_part.split_stride, qkv_part.ld, st);
+        else
+            launch_rope_store_attention(state->q_buf, state->k_buf, state->v_buf, m->kv_cache_k + kv_off,
+                                        m->kv_cache_v + kv_off, m->kv_scale_k + sc_off, m->kv_scale_v + sc_off, bf16_a,
+                                        B == 1 ? nullptr : state->d_positions, state->positions[0], c.n_head,
+                                        c.n_head_kv, head_dim, c.rope_theta, scale, B, 0, st);
 
         S.o[0] = seg_of(L.wo, res, n);
         if (B > 1) {

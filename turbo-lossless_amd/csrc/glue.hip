@@ -154,6 +154,26 @@ __global__ __launch_bounds__(256) void add_kernel(float* __restrict__ y, const f
 //   blocks [n_head, n_head + nkv)          rotate a K head in place, then quantise + store it
 //   blocks [n_head + nkv, n_head + 2 nkv)  quantise + store a V head
 // MODE bit 0: do the rotations; bit 1: do the stores.
+// Rotate-half RoPE of one pair (kernels.hip:244-262): two products and one add / subtract each, never
+// contracted into fused multiply-adds, so that every kernel that rotates gives the same bits.
+__device__ __forceinline__ void rope_rotate(float x0, float x1, float sn, float cs, float& r0, float& r1)
+{
+#pragma clang fp contract(off)
+    const float a = x0 * cs, b = x1 * sn, c = x0 * sn, d = x1 * cs;
+    r0 = a - b;
+    r1 = c + d;
+}
+
+// Partial sums of a K-split q|k|v projection (t12_gemm_deferred): element (b, col) of the fused
+// [q | k | v] row is the ascending sum over z < nsplit of ws[z * split_stride + b * ld + col].
+// nsplit == 0: the values are complete in the q / k / v buffers.
+struct QkvPartials {
+    const float* ws;
+    int nsplit;
+    int ld;
+    size_t split_stride;
+};
+
 template <int MODE>
 __global__ __launch_bounds__(64) void rope_kv_kernel(float* __restrict__ q, float* __restrict__ k,
                                                      const float* __restrict__ v, int8_t* __restrict__ ck,
@@ -161,7 +181,7 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(float* __restrict__ q, floa
                                                      float* __restrict__ sv, const float* __restrict__ freqs,
                                                      const int* __restrict__ positions, int position,
                                                      int head_dim, int n_head, int n_head_kv, int q_stride,
-                                                     int k_stride)
+                                                     int k_stride, QkvPartials part = QkvPartials{nullptr, 0, 0, 0})
 {
     const int b = blockIdx.y;
     const int pos = positions ? positions[b] : position;
@@ -173,20 +193,37 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(float* __restrict__ q, floa
     int8_t* dst = nullptr;
     float* sdst = nullptr;
     int kvh = 0;
+    int pcol = 0;                       // first column of this head in the fused [q | k | v] row
     if (blk < n_head) {
         rot = q + (size_t)b * q_stride + (size_t)blk * head_dim;
+        pcol = blk * head_dim;
     } else if (blk < n_head + n_head_kv) {
         kvh = blk - n_head;
         rot = k + (size_t)b * k_stride + (size_t)kvh * head_dim;
         src = rot;
         dst = ck;
         sdst = sk;
+        pcol = (n_head + kvh) * head_dim;
     } else {
         kvh = blk - n_head - n_head_kv;
         src = v + (size_t)b * k_stride + (size_t)kvh * head_dim;
         dst = cv;
         sdst = sv;
+        pcol = (n_head + n_head_kv + kvh) * head_dim;
     }
+    // value i of this head: from its buffer, or rebuilt from the K-split partial sums
+    auto value = [&](const float* buf, int i) {
+        if (part.nsplit == 0) return buf[i];
+        const float* pr = part.ws + (size_t)b * part.ld + pcol + i;
+        float pz[T12_MAX_KSPLIT];
+#pragma unroll
+        for (int z = 0; z < T12_MAX_KSPLIT; z++) pz[z] = z < part.nsplit ? pr[(size_t)z * part.split_stride] : 0.0f;
+        float t = 0.0f;
+#pragma unroll
+        for (int z = 0; z < T12_MAX_KSPLIT; z++)
+            if (z < part.nsplit) t += pz[z];
+        return t;
+    };
     // lane owns the pair (lane, lane + half); head_dim <= 128 so one pair per lane
     const bool own = lane < half;
     float r0 = 0.0f, r1 = 0.0f;
@@ -195,15 +232,14 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(float* __restrict__ q, floa
             const float ang = (float)pos * freqs[lane];
             float sn, cs;
             sincosf(ang, &sn, &cs);
-            const float x0 = rot[lane], x1 = rot[lane + half];
-            r0 = x0 * cs - x1 * sn;
-            r1 = x0 * sn + x1 * cs;
+            const float x0 = value(rot, lane), x1 = value(rot, lane + half);
+            rope_rotate(x0, x1, sn, cs, r0, r1);
             rot[lane] = r0;
             rot[lane + half] = r1;
         }
     } else if (src && own) {
-        r0 = src[lane];
-        r1 = src[lane + half];
+        r0 = value(src, lane);
+        r1 = value(src, lane + half);
     }
     if ((MODE & 2) && dst) {
         const float amax = wave_max(fmaxf(fabsf(r0), fabsf(r1)));
@@ -427,8 +463,7 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
             float sn, cs;
             sincosf((float)pos * fz.freqs[d], &sn, &cs);
             const float x0 = qb[h * HD + d], x1 = qb[h * HD + d + HALF];
-            qs[h * HD + d] = x0 * cs - x1 * sn;
-            qs[h * HD + d + HALF] = x0 * sn + x1 * cs;
+            rope_rotate(x0, x1, sn, cs, qs[h * HD + d], qs[h * HD + d + HALF]);
         }
         if (wave < 2) {                                              // wave 0: K (rotated), wave 1: V
             const bool own = lane < HALF;
@@ -441,8 +476,7 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
                     float sn, cs;
                     sincosf((float)pos * fz.freqs[lane], &sn, &cs);
                     const float x0 = r0, x1 = r1;
-                    r0 = x0 * cs - x1 * sn;
-                    r1 = x0 * sn + x1 * cs;
+                    rope_rotate(x0, x1, sn, cs, r0, r1);
                 }
             }
             const float amax = wave_max(fmaxf(fabsf(r0), fabsf(r1)));
@@ -716,7 +750,7 @@ void report(const char* what)
 template <int MODE>
 void launch_rope_kv(float* q, float* k, const float* v, int8_t* ck, int8_t* cv, float* sk, float* sv,
                     const int* positions, int position, int head_dim, int n_head, int n_head_kv, int q_stride,
-                    int k_stride, float theta, int batch, hipStream_t st)
+                    int k_stride, float theta, int batch, hipStream_t st, QkvPartials part = QkvPartials{nullptr, 0, 0, 0})
 {
     const float* f = nullptr;
     if (MODE & 1) {
@@ -729,7 +763,7 @@ void launch_rope_kv(float* q, float* k, const float* v, int8_t* ck, int8_t* cv, 
         return;
     }
     hipLaunchKernelGGL(rope_kv_kernel<MODE>, dim3(n_head + 2 * n_head_kv, batch), dim3(64), 0, st, q, k, v, ck, cv, sk,
-                       sv, f, positions, position, head_dim, n_head, n_head_kv, q_stride, k_stride);
+                       sv, f, positions, position, head_dim, n_head, n_head_kv, q_stride, k_stride, part);
     report("rope/kv-store");
 }
 
@@ -924,6 +958,28 @@ void launch_rope_store_attention(float* q, float* k, const float* v, int8_t* kv_
                       n_head * head_dim, n_head_kv * head_dim, theta, batch_size, stream);
     launch_attn(q, kv_k, kv_v, scale_k, scale_v, output, positions, position + 1, n_head, n_head_kv, head_dim, scale,
                 batch_size, (size_t)kv_stride, stream);
+}
+
+// launch_rope_store_attention for a batch on one shared cache region whose q | k | v projection was split
+// along K (t12_gemm_deferred, one launch for the three tensors in this order): the RoPE / KV-store kernel adds
+// the partial sums up itself.  q and k receive the rotated values; the v buffer is not written.
+void launch_rope_store_attention_partials(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v,
+                                          float* scale_k, float* scale_v, int16_t* output, const int* positions,
+                                          int position, int n_head, int n_head_kv, int head_dim, float theta,
+                                          float scale, int batch_size, const float* partials, int nsplit,
+                                          size_t split_stride, int ld, hipStream_t stream)
+{
+    if (!partials || nsplit < 1 || nsplit > T12_MAX_KSPLIT || ld < (n_head + 2 * n_head_kv) * head_dim) {
+        t12_set_error("rope_store_attention_partials: nsplit %d outside 1..%d, null partials or ld %d too small", nsplit,
+                      T12_MAX_KSPLIT, ld);
+        fprintf(stderr, "turbo12: %s\n", t12_last_error());
+        return;
+    }
+    launch_rope_kv<3>(q, k, v, kv_k, kv_v, scale_k, scale_v, positions, position, head_dim, n_head, n_head_kv,
+                      n_head * head_dim, n_head_kv * head_dim, theta, batch_size, stream,
+                      QkvPartials{partials, nsplit, ld, split_stride});
+    launch_attn(q, kv_k, kv_v, scale_k, scale_v, output, positions, position + 1, n_head, n_head_kv, head_dim, scale,
+                batch_size, 0, stream);
 }
 
 void launch_attention_all_heads(const float* q, const int8_t* k_cache, const int8_t* v_cache, const float* scale_k,
