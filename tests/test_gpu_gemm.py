@@ -186,3 +186,46 @@ def test_gemm_more_escapes_than_the_lds_list_holds(t12, oracle, synth, B):
             assert rel_err(got, ref) < TOL, ks
     finally:
         t12.lib.t12_tune_gemm(0)
+
+
+@pytest.mark.parametrize("M,K,B,p_out", [(14336, 4096, 256, 3e-4), (12300, 512, 129, 2e-3), (12352, 256, 300, 5e-2),
+                                          (12288, 64, 512, 0.0)])
+def test_gemm_swiglu_epilogue_is_bit_identical_to_unfused(t12, synth, M, K, B, p_out):
+    """t12_gemm_swiglu == t12_gemm on (gate, up) + launch_silu_mul_bf16_batch, bit for bit (ragged last tile,
+    escape lists that fit the LDS staging and ones that overflow it, tensors without escapes)."""
+    g = torch.Generator(device=dev())
+
+    def mk(seed):
+        g.manual_seed(seed)
+        w = torch.randn((M, K), generator=g, device=dev()) * 0.02
+        if p_out > 0:
+            m = torch.rand((M, K), generator=g, device=dev()) < p_out
+            w = torch.where(m, torch.randn((M, K), generator=g, device=dev()) * 8, w)
+        return t12.pack_device(w.to(torch.bfloat16))
+
+    gate, up = mk(1), mk(2)
+    g.manual_seed(3)
+    X = torch.randn((B, K), generator=g, device=dev()).to(torch.bfloat16).view(torch.int16)
+    st = t12.current_stream()
+    og, ou = t12.gemm([gate, up], X)
+    want = torch.empty((B, M), dtype=torch.int16, device=dev())
+    t12.lib.launch_silu_mul_bf16_batch(og.data_ptr(), ou.data_ptr(), want.data_ptr(), M, B, st)
+    got = torch.full((B, M), -1, dtype=torch.int16, device=dev())
+    sg = t12._seg_array([gate.segment(None)])
+    su = t12._seg_array([up.segment(None)])
+    rc = t12.lib.t12_gemm_swiglu(sg, su, X.data_ptr(), K, K, B, got.data_ptr(), M, st)
+    torch.cuda.synchronize()
+    assert rc == 0, t12.lib.t12_last_error()
+    assert torch.equal(got, want)
+
+
+def test_gemm_swiglu_declines_shapes_without_a_fused_kernel(t12, oracle, synth):
+    p = oracle.pack(synth.weights_llm(512, 256, seed=1))
+    dt = t12.DeviceTensor12.from_packed(p, dev())
+    X = to_dev_bits(synth.activations(256, 256, seed=2)).reshape(256, 256)
+    out = torch.empty((256, 512), dtype=torch.int16, device=dev())
+    s1 = t12._seg_array([dt.segment(None)])
+    st = t12.current_stream()
+    assert t12.lib.t12_gemm_swiglu(s1, s1, X.data_ptr(), 256, 256, 256, out.data_ptr(), 512, st) == 1      # few rows
+    assert t12.lib.t12_gemm_swiglu(s1, s1, X.data_ptr(), 256, 256, 64, out.data_ptr(), 512, st) == 1       # small batch
+    assert t12.lib.t12_gemm_swiglu(s1, s1, X.data_ptr(), 256, 256, 256, out.data_ptr(), 100, st) == -1     # out_stride < M

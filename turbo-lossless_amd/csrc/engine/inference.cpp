@@ -369,8 +369,16 @@ void forward(InferenceState* state, const int* token_ids)
                 exit(1);
             }
         } else {
-            run_linear(S.gateup, 2, bf16_a, n, B, st);
-            launch_silu_mul_bf16_batch(state->ffn_gate, state->ffn_up, bf16_b, n_ff, B, st);
+            // gate|up decode+GEMM with the SiLU*mul in its epilogue where the shape has such a kernel
+            const int rc = B > 1 ? t12_gemm_swiglu(&S.gateup[0], &S.gateup[1], bf16_a, n, n, B, bf16_b, n_ff, st) : 1;
+            if (rc < 0) {
+                fprintf(stderr, "ERROR: fused gate|up launch failed: %s\n", t12_last_error());
+                exit(1);
+            }
+            if (rc == 1) {
+                run_linear(S.gateup, 2, bf16_a, n, B, st);
+                launch_silu_mul_bf16_batch(state->ffn_gate, state->ffn_up, bf16_b, n_ff, B, st);
+            }
         }
 
         S.down[0] = seg_of(L.w_down, cur, n);

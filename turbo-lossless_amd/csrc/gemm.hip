@@ -56,6 +56,8 @@ struct GemmParams {
     int m_total;                           // sum of M over segments (workspace row length)
     const uint16_t* act;
     float* ws;                             // [ksplit][B][m_total] partial sums when ksplit > 1
+    uint16_t* out_bf16;                    // SwiGLU mode: bf16 [B, out_bf16_ld], silu(seg 0) * seg 1
+    int out_bf16_ld;
 };
 
 // LDS slot of (unit, row) in a [units][rows] array of 16-byte units.  Rows are rotated
@@ -105,9 +107,15 @@ __device__ __forceinline__ int find_segment(const GemmParams& p, int tile)
 // stage (balanced), every sm line is requested whole within two instructions, and the
 // rr^1 keeps the LDS writes of the two lane groups on different banks.
 // ---------------------------------------------------------------------------
-template <int WB, int WM, int FB, int FM>
+// SWI (two segments of equal M, gate and up; FM == 2): a tile holds 64 rows of each, interleaved in
+// blocks of 32 -- local rows [0,32) gate rows 0..31, [32,64) up rows 0..31, [64,96) gate 32..63, [96,128) up
+// 32..63 -- so that the two accumulator tiles of a wave are gate and up of the SAME 32 rows and the epilogue
+// writes bf16( silu(gate) * up ) straight from registers: the reference's silu_mul_bf16 kernel
+// (engine/kernels.hip:447-459) and the fp32 round trip of both projections folded away.
+template <int WB, int WM, int FB, int FM, bool SWI = false>
 __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
 {
+    static_assert(!SWI || FM == 2, "the SwiGLU epilogue pairs the two row tiles of a wave");
     constexpr int TB = WB * FB * 32;                  // batch rows per workgroup
     constexpr int NT = WB * WM * 64;                  // threads per workgroup
     static_assert(NT == 256 || NT == 512, "four or eight waves per workgroup");
@@ -124,15 +132,23 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
     const int ln = lane & 31, lh = lane >> 5;
 
     const int tile = blockIdx.x;
-    const int s = find_segment(p, tile);
+    const int s = SWI ? 0 : find_segment(p, tile);
     const T12Segment& sg = p.seg[s];
     const int M = sg.M, K = p.K, B = p.B;
-    const int m0 = (tile - p.blk_start[s]) * TM;
+    const int m0 = SWI ? tile * (TM / 2) : (tile - p.blk_start[s]) * TM;
+    // local row r of the tile -> segment and matrix row
+    auto row_seg = [&](int r) { return SWI ? (r >> 5) & 1 : s; };
+    auto row_mat = [&](int r) { return SWI ? m0 + ((r >> 6) << 5) + (r & 31) : m0 + r; };
     const int b0 = blockIdx.y * TB;
     const int k_begin = blockIdx.z * p.kslice;
     const int k_end = min(K, k_begin + p.kslice);
     const int nstage = (k_end - k_begin) / KC;
-    const uint32_t be2 = t12_opaque(((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23));
+    uint32_t be2s[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int be = p.seg[SWI ? j : s].base_exp;
+        be2s[j] = t12_opaque(((uint32_t)be << 7) | ((uint32_t)be << 23));
+    }
 
     // ---- this thread's share of the global -> LDS staging
     //  acts: item idx = tid + NT*i -> batch row idx / 8, unit idx % 8 (8 lanes = 128 contiguous bytes)
@@ -152,6 +168,7 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
     const uint8_t* g_src[2][W_LD];
     int w_row[2][W_LD];
     int w_dst[2][W_LD][2];
+    uint32_t w_be2[2][W_LD];
 #pragma unroll
     for (int i = 0; i < W_LD; i++) {
         const int rr = (tid + NT * i) >> 3;                   // 0..63
@@ -159,10 +176,12 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
 #pragma unroll
         for (int y = 0; y < 2; y++) {
             const int r = (hi ^ y) ? r_hi : r_lo;
-            const size_t e = (size_t)min(m0 + r, M - 1) * K + k_begin + 64 * y + 16 * cc;
+            const T12Segment& g = p.seg[row_seg(r)];
+            const size_t e = (size_t)min(row_mat(r), M - 1) * K + k_begin + 64 * y + 16 * cc;
             w_row[y][i] = r;
-            s_src[y][i] = sg.sm + e;
-            g_src[y][i] = sg.gr + (e >> 1);
+            w_be2[y][i] = be2s[SWI ? (r >> 5) & 1 : 0];
+            s_src[y][i] = g.sm + e;
+            g_src[y][i] = g.gr + (e >> 1);
             w_dst[y][i][0] = ACT_UNITS * 16 + lds_slot(2 * cc, r, TM) * 16;
             w_dst[y][i][1] = ACT_UNITS * 16 + lds_slot(2 * cc + 1, r, TM) * 16;
         }
@@ -195,8 +214,8 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
             const uint4 sv = rs[wslot][y][i];
             const uint2 gv = rg[wslot][y][i];
             uint32_t w_[4];
-            if (h == 0) t12_decode8(sv.x, sv.y, gv.x, be2, w_);
-            else t12_decode8(sv.z, sv.w, gv.y, be2, w_);
+            if (h == 0) t12_decode8(sv.x, sv.y, gv.x, w_be2[y][i], w_);
+            else t12_decode8(sv.z, sv.w, gv.y, w_be2[y][i], w_);
             *(uint4*)(base_ + w_dst[y][i][h]) = make_uint4(w_[0], w_[1], w_[2], w_[3]);
         }
     };
@@ -214,9 +233,27 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
     //      esc_mode: 0 none, 1 staged (exact values written over the decoded ones in LDS),
     //      2 too many for LDS (or K > 65536): wrong values multiplied, corrected in the epilogue.
     uint32_t* lpat = (uint32_t*)(lds + 2 * STAGE_BYTES);       // col | correct << 16
-    int* lrow = (int*)(lpat + PCAP);                           // [TM + 1] offsets into lpat
+    int* lrow = (int*)(lpat + PCAP);                           // [TM + 1] offsets into lpat (SWI: [2][TM/2 + 1])
     int esc_mode = 0;
-    if (sg.row_off) {
+    if (SWI) {
+        // two slices: the 64 gate rows, then the 64 up rows
+        const T12Segment& g0 = p.seg[0];
+        const T12Segment& g1 = p.seg[1];
+        const int r_lo = min(m0, M), r_hi = min(m0 + TM / 2, M);
+        const int e00 = g0.row_off ? g0.row_off[r_lo] : 0, e10 = g1.row_off ? g1.row_off[r_lo] : 0;
+        const int n0 = g0.row_off ? g0.row_off[r_hi] - e00 : 0, n1 = g1.row_off ? g1.row_off[r_hi] - e10 : 0;
+        if (g0.row_off || g1.row_off) esc_mode = (n0 + n1 <= PCAP && K <= 65536) ? 1 : 2;
+        if (esc_mode == 1) {
+            for (int t = tid; t < n0; t += NT)
+                lpat[t] = (uint32_t)g0.cols[e00 + t] | ((uint32_t)(uint16_t)g0.correct[e00 + t] << 16);
+            for (int t = tid; t < n1; t += NT)
+                lpat[n0 + t] = (uint32_t)g1.cols[e10 + t] | ((uint32_t)(uint16_t)g1.correct[e10 + t] << 16);
+            for (int t = tid; t <= TM / 2; t += NT) {
+                lrow[t] = g0.row_off ? g0.row_off[min(m0 + t, M)] - e00 : 0;
+                lrow[TM / 2 + 1 + t] = n0 + (g1.row_off ? g1.row_off[min(m0 + t, M)] - e10 : 0);
+            }
+        }
+    } else if (sg.row_off) {
         const int e0 = sg.row_off[min(m0, M)], e1 = sg.row_off[min(m0 + TM, M)];
         esc_mode = (e1 - e0 <= PCAP && K <= 65536) ? 1 : 2;
         if (esc_mode == 1) {
@@ -338,8 +375,9 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
 #pragma unroll
             for (int i = 0; i < W_LD; i++) {
                 const int r = w_row[y][i];
-                int q = lrow[r];
-                const int qe = lrow[r + 1];
+                const int li = SWI ? ((r >> 5) & 1) * (TM / 2 + 1) + ((r >> 6) << 5) + (r & 31) : r;
+                int q = lrow[li];
+                const int qe = lrow[li + 1];
                 while (q < qe && (int)(lpat[q] & 0xFFFFu) < k_begin) q++;   // K split: skip earlier columns
                 pp[y][i] = q;
                 pe[y][i] = qe;
@@ -381,13 +419,14 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
     if (blockIdx.z == 0 && esc_mode == 2) {
 #pragma unroll
         for (int j = 0; j < FM; j++) {
-            const int m = m0 + (wm * FM + j) * 32 + ln;
-            if (m < M) {
-                const int beg = sg.row_off[m], end = sg.row_off[m + 1];
+            const T12Segment& g = p.seg[SWI ? j : s];
+            const int m = SWI ? m0 + wm * 32 + ln : m0 + (wm * FM + j) * 32 + ln;
+            if (m < M && g.row_off) {
+                const int beg = g.row_off[m], end = g.row_off[m + 1];
                 for (int pp = beg; pp < end; pp++) {
-                    const float delta = t12_bf16_to_f32((uint16_t)sg.correct[pp]) -
-                                        t12_bf16_to_f32((uint16_t)sg.wrong[pp]);
-                    const uint16_t* xc = p.act + sg.cols[pp];
+                    const float delta = t12_bf16_to_f32((uint16_t)g.correct[pp]) -
+                                        t12_bf16_to_f32((uint16_t)g.wrong[pp]);
+                    const uint16_t* xc = p.act + g.cols[pp];
 #pragma unroll
                     for (int i = 0; i < FB; i++)
 #pragma unroll
@@ -402,6 +441,19 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
 
     // ---- store: accumulator register r of lane (ln, lh) is
     //      D[row = 8*(r/4) + 4*lh + r%4][col = ln]   (row = batch, col = m)
+    if (SWI) {
+        const int m = m0 + wm * 32 + ln;
+#pragma unroll
+        for (int i = 0; i < FB; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int b = b0 + (wb * FB + i) * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                const float g = acc[i][0][r];
+                if (m < M && b < B)
+                    p.out_bf16[(size_t)b * p.out_bf16_ld + m] = t12_f32_to_bf16(g / (1.0f + expf(-g)) * acc[i][FM - 1][r]);
+            }
+        return;
+    }
     float* dst;
     size_t ld;
     int col_off;
@@ -428,10 +480,10 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
 }
 
 // One workgroup per CU (batch tile 256: 128 accumulator registers + the load ring) ...
-template <int WB, int WM, int FB, int FM>
+template <int WB, int WM, int FB, int FM, bool SWI = false>
 __global__ __launch_bounds__(WB * WM * 64) void gemm_mfma_kernel(const GemmParams p)
 {
-    gemm_mfma_body<WB, WM, FB, FM>(p);
+    gemm_mfma_body<WB, WM, FB, FM, SWI>(p);
 }
 // ... or two (batch tiles <= 128): at most 256 registers per lane, so that two waves share a SIMD
 // and one wave's decode / LDS traffic runs under the other's MFMAs.
@@ -524,13 +576,14 @@ float* workspace(size_t bytes)
 
 int g_gemm_ksplit = 0;   // 0 = choose by shape
 
-template <int WB, int WM, int FB, int FM, bool OCC2 = false>
+template <int WB, int WM, int FB, int FM, bool OCC2 = false, bool SWI = false>
 int launch_mfma(GemmParams& p, int tiles, hipStream_t st)
 {
+    static_assert(!(OCC2 && SWI), "the SwiGLU epilogue exists for the one-workgroup-per-CU kernels");
     constexpr int TB = WB * FB * 32;
     constexpr int STAGE_BYTES = TB * 8 * 16 + TM * 128;
     const dim3 grid(tiles, (p.B + TB - 1) / TB, p.ksplit);   // batch tiles of one row tile are neighbours in time
-    auto kfn = OCC2 ? gemm_mfma_kernel_occ2<WB, WM, FB, FM> : gemm_mfma_kernel<WB, WM, FB, FM>;
+    auto kfn = OCC2 ? gemm_mfma_kernel_occ2<WB, WM, FB, FM> : gemm_mfma_kernel<WB, WM, FB, FM, SWI>;
     static bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -563,6 +616,47 @@ int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_str
     return t12_gemm_deferred(segs, nseg, act_bf16, act_stride, out_stride, K, B, nullptr, stream);
 }
 
+// out_bf16[b, m] = bf16( silu(gate[m,:] . X[b,:]) * (up[m,:] . X[b,:]) ): gate|up projection with the SwiGLU
+// in the GEMM's epilogue.  Returns T12_OK when launched, 1 when this shape has no fused kernel (the caller
+// then runs t12_gemm on the two segments and launch_silu_mul_bf16_batch), negative on bad operands.
+int t12_gemm_swiglu(const T12Segment* gate, const T12Segment* up, const void* act_bf16, int act_stride, int K, int B,
+                    void* out_bf16, int out_stride, void* stream)
+{
+    T12_REQUIRE(gate && up && act_bf16 && out_bf16, "t12_gemm_swiglu: null operand");
+    T12_REQUIRE(K >= 1 && B >= 1 && act_stride >= K, "t12_gemm_swiglu: K %d, B %d or act_stride %d invalid", K, B, act_stride);
+    T12_REQUIRE(gate->M >= 1 && gate->M == up->M, "t12_gemm_swiglu: gate has %d rows, up has %d", gate->M, up->M);
+    T12_REQUIRE(out_stride >= gate->M, "t12_gemm_swiglu: out_stride %d < M %d", out_stride, gate->M);
+    const T12Segment* two[2] = {gate, up};
+    bool fast = (K % KC == 0) && (act_stride % 8 == 0) && ((uintptr_t)act_bf16 % 16 == 0) && B > 128;
+    for (const T12Segment* g : two) {
+        T12_REQUIRE(g->sm && g->gr, "t12_gemm_swiglu: a plane is null");
+        T12_REQUIRE(!g->row_off || (g->cols && g->correct && g->wrong), "t12_gemm_swiglu: row_off without lists");
+        T12_REQUIRE(g->base_exp >= -1 && g->base_exp <= 254, "t12_gemm_swiglu: base_exp %d out of range", g->base_exp);
+        if (g->base_exp < 0 || g->base_exp > 240) fast = false;
+    }
+    const int tiles = (gate->M + TM / 2 - 1) / (TM / 2);
+    const int btiles = (B + 255) / 256;
+    if (!fast || tiles * btiles * 4 < 256 * 3) return 1;      // would need a K split: partial sums cannot be gated
+    GemmParams p;
+    p.seg[0] = *gate;
+    p.seg[1] = *up;
+    p.nseg = 2;
+    p.K = K;
+    p.B = B;
+    p.act_stride = act_stride;
+    p.act = (const uint16_t*)act_bf16;
+    p.ws = nullptr;
+    p.ksplit = 1;
+    p.kslice = ((K + 2 * KC - 1) / (2 * KC)) * 2 * KC;
+    p.m_total = gate->M;
+    p.blk_start[0] = 0;
+    p.blk_start[1] = p.blk_start[2] = tiles;
+    p.seg_row0[0] = p.seg_row0[1] = 0;
+    p.out_bf16 = (uint16_t*)out_bf16;
+    p.out_bf16_ld = out_stride;
+    return launch_mfma<4, 2, 2, 2, false, true>(p, tiles, (hipStream_t)stream);
+}
+
 // t12_gemm whose K-split partial sums may be left in the workspace for the caller's next kernel to add
 // up (part != NULL): part->nsplit == 1 means the outputs are complete in segs[].out.
 int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride, int out_stride, int K,
@@ -586,6 +680,8 @@ int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, in
     p.act_stride = act_stride;
     p.act = (const uint16_t*)act_bf16;
     p.ws = nullptr;
+    p.out_bf16 = nullptr;
+    p.out_bf16_ld = 0;
     bool fast = (K % KC == 0) && (act_stride % 8 == 0) && ((uintptr_t)act_bf16 % 16 == 0);
     int m_total = 0;
     for (int i = 0; i < nseg; i++) {

@@ -6,7 +6,7 @@ entry point (`nv_launch_split12_fused_gemm_async`, nvidia_kernels.cu:444) would 
 for a Mixtral-shaped layer: one call per expert with that expert's variable token count as B.
 torch is used for the routing bookkeeping only (top-k, sort, gather, weighted scatter-add).
 """
-from . import DeviceTensor12, gemm, lib, current_stream, _torch
+from . import DeviceTensor12, gemm, lib, check, current_stream, _seg_array, _torch
 
 
 class Expert:
@@ -48,8 +48,13 @@ def moe_ffn(experts, X, expert_ids, weights, stream=None):
             continue
         ex = experts[e]
         xs = Xg[pos:pos + cnt]
-        gemm([ex.w1, ex.w3], xs, outs=[gate[:cnt], up[:cnt]], stream=st)
-        lib.launch_silu_mul_bf16_batch(gate.data_ptr(), up.data_ptr(), act.data_ptr(), n_ff, cnt, st)
+        # SiLU*mul in the GEMM's epilogue where the group is large enough to have such a kernel
+        rc = lib.t12_gemm_swiglu(_seg_array([ex.w1.segment(None)]), _seg_array([ex.w3.segment(None)]), xs.data_ptr(),
+                                 xs.stride(0), n, cnt, act.data_ptr(), n_ff, st)
+        check(min(rc, 0), "t12_gemm_swiglu")
+        if rc == 1:
+            gemm([ex.w1, ex.w3], xs, outs=[gate[:cnt], up[:cnt]], stream=st)
+            lib.launch_silu_mul_bf16_batch(gate.data_ptr(), up.data_ptr(), act.data_ptr(), n_ff, cnt, st)
         gemm([ex.w2], act[:cnt], outs=[yd[:cnt]], stream=st)
         out.index_add_(0, tok[pos:pos + cnt], yd[:cnt] * wg[pos:pos + cnt, None])
         pos += cnt
