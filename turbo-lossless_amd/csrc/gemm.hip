@@ -14,21 +14,23 @@
 //   * The whole batch tile (up to 256 rows) lives in one workgroup: every
 //     weight byte is fetched once per launch (the reference re-decodes per
 //     batch tile, nvidia_kernels.cu:456).
-//   * The compressed planes are staged global -> LDS as they are (1.5 B per
-//     weight) and rebuilt to bf16 in registers, two weights per VGPR
-//     (t12_decode8), straight into the MFMA B operand: no bf16 copy of W ever
-//     exists in LDS or HBM.  The activations are staged already paired the way
-//     t12_decode8 orders its outputs, so no operand shuffling is needed.
-//   * Waves are laid out WB x WM; a wave owns FB x FM 32x32 accumulator tiles.
-//     B <= 128 uses 1 x 4 waves (each weight decoded once per workgroup);
-//     B <= 256 uses 2 x 2 waves with 4 x 2 tiles (128 accumulator VGPRs).
+//   * The compressed planes are loaded into registers, rebuilt to bf16 there, two
+//     weights per VGPR (t12_decode8), and written once per workgroup into a bf16 tile
+//     in LDS from which the waves read their MFMA B fragments: every weight is
+//     decoded once per workgroup, no bf16 copy of W ever exists in HBM.  The
+//     activations are staged already paired the way t12_decode8 orders its
+//     outputs, so no operand shuffling is needed.
+//   * Eight waves per workgroup (two per SIMD), laid out WB x WM; a wave owns FB x FM 32x32
+//     accumulator tiles: batch tiles of 64 (2 x 4 waves, 1 x 1), 128 (2 x 4, 2 x 1) and
+//     256 rows (4 x 2, 2 x 2).
 //   * Few row tiles (small M) are split along K across workgroups; the partial
 //     sums go to a workspace and a second kernel adds them in a fixed order
-//     (deterministic) together with the escape corrections.
+//     (deterministic) -- or the caller's next kernel does (t12_gemm_deferred).
 //   * Escapes are EXACT and cost no extra pass: the (column, exact bf16) pairs of
 //     the workgroup's 128 rows -- one contiguous slice of the CSR list -- are
-//     staged in LDS once; every lane walks its own row's slice in step with the
-//     K loop and overwrites the decoded half-word in its MFMA operand register.
+//     staged in LDS once; the thread that decoded 16 columns of a row walks that
+//     row's slice in step with the K loop and overwrites the decoded half-words
+//     in the LDS tile.
 //
 // Fast path requirements: K % 64 == 0, 0 <= base_exp <= 240, 16-byte aligned
 // activation rows.  Everything else goes to the general kernel below.
@@ -118,7 +120,7 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
     static_assert(!SWI || FM == 2, "the SwiGLU epilogue pairs the two row tiles of a wave");
     constexpr int TB = WB * FB * 32;                  // batch rows per workgroup
     constexpr int NT = WB * WM * 64;                  // threads per workgroup
-    static_assert(NT == 256 || NT == 512, "four or eight waves per workgroup");
+    static_assert(NT == 512, "eight waves per workgroup");
     static_assert(WM * FM * 32 == TM, "row tile is 128");
     constexpr int ACT_UNITS = TB * 8;                 // 16-byte units per stage
     constexpr int ACT_LD = ACT_UNITS / NT;            // per thread
@@ -479,18 +481,11 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
         }
 }
 
-// One workgroup per CU (batch tile 256: 128 accumulator registers + the load ring) ...
+// Eight waves per workgroup, two per SIMD: one wave's decode / LDS traffic runs under the other's MFMAs.
 template <int WB, int WM, int FB, int FM, bool SWI = false>
 __global__ __launch_bounds__(WB * WM * 64) void gemm_mfma_kernel(const GemmParams p)
 {
     gemm_mfma_body<WB, WM, FB, FM, SWI>(p);
-}
-// ... or two (batch tiles <= 128): at most 256 registers per lane, so that two waves share a SIMD
-// and one wave's decode / LDS traffic runs under the other's MFMAs.
-template <int WB, int WM, int FB, int FM>
-__global__ __launch_bounds__(256, 2) void gemm_mfma_kernel_occ2(const GemmParams p)
-{
-    gemm_mfma_body<WB, WM, FB, FM>(p);
 }
 
 // ---------------------------------------------------------------------------
@@ -576,14 +571,13 @@ float* workspace(size_t bytes)
 
 int g_gemm_ksplit = 0;   // 0 = choose by shape
 
-template <int WB, int WM, int FB, int FM, bool OCC2 = false, bool SWI = false>
+template <int WB, int WM, int FB, int FM, bool SWI = false>
 int launch_mfma(GemmParams& p, int tiles, hipStream_t st)
 {
-    static_assert(!(OCC2 && SWI), "the SwiGLU epilogue exists for the one-workgroup-per-CU kernels");
     constexpr int TB = WB * FB * 32;
     constexpr int STAGE_BYTES = TB * 8 * 16 + TM * 128;
     const dim3 grid(tiles, (p.B + TB - 1) / TB, p.ksplit);   // batch tiles of one row tile are neighbours in time
-    auto kfn = OCC2 ? gemm_mfma_kernel_occ2<WB, WM, FB, FM> : gemm_mfma_kernel<WB, WM, FB, FM, SWI>;
+    auto kfn = gemm_mfma_kernel<WB, WM, FB, FM, SWI>;
     static bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -654,7 +648,7 @@ int t12_gemm_swiglu(const T12Segment* gate, const T12Segment* up, const void* ac
     p.seg_row0[0] = p.seg_row0[1] = 0;
     p.out_bf16 = (uint16_t*)out_bf16;
     p.out_bf16_ld = out_stride;
-    return launch_mfma<4, 2, 2, 2, false, true>(p, tiles, (hipStream_t)stream);
+    return launch_mfma<4, 2, 2, 2, true>(p, tiles, (hipStream_t)stream);
 }
 
 // t12_gemm whose K-split partial sums may be left in the workspace for the caller's next kernel to add
@@ -728,7 +722,7 @@ int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, in
     int ks = 1;
     if (g_gemm_ksplit > 0) ks = g_gemm_ksplit < T12_MAX_KSPLIT ? g_gemm_ksplit : T12_MAX_KSPLIT;
     else
-        while (tiles * btiles * ks * 4 < want * 3 && K / (ks * 2) >= 4 * KC && ks < T12_MAX_KSPLIT) ks *= 2;
+        while (tiles * btiles * ks * 4 < want * 3 && K / (ks * 2) >= 8 * KC && ks < T12_MAX_KSPLIT) ks *= 2;
     int kslice = (((K + 2 * KC - 1) / (2 * KC) + ks - 1) / ks) * 2 * KC;      // whole windows of two stages
     ks = (K + kslice - 1) / kslice;
     p.ksplit = ks;
@@ -742,8 +736,7 @@ int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, in
         }
     }
     int rc;
-    if (B <= 32) rc = launch_mfma<1, 4, 1, 1, true>(p, tiles, st);
-    else if (B <= 64) rc = launch_mfma<1, 4, 2, 1, true>(p, tiles, st);
+    if (B <= 64) rc = launch_mfma<2, 4, 1, 1>(p, tiles, st);
     else if (B <= 128) rc = launch_mfma<2, 4, 2, 1>(p, tiles, st);
     else rc = launch_mfma<4, 2, 2, 2>(p, tiles, st);
     if (rc) return rc;
