@@ -578,7 +578,10 @@ int launch_mfma(GemmParams& p, int tiles, hipStream_t st)
     constexpr int STAGE_BYTES = TB * 8 * 16 + TM * 128;
     const dim3 grid(tiles, (p.B + TB - 1) / TB, p.ksplit);   // batch tiles of one row tile are neighbours in time
     auto kfn = gemm_mfma_kernel<WB, WM, FB, FM, SWI>;
-    static bool attr_set = false;
+    static bool attr_done[16] = {};                    // the attribute is per device
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) dev = 0;
+    bool& attr_set = attr_done[dev];
     if (!attr_set) {
         if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 2 * STAGE_BYTES + PATCH_BYTES) !=
