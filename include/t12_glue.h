@@ -25,6 +25,17 @@ extern "C" {
  * the RoPE launchers build (and cache per (head_dim, theta)) the table on first use. */
 void launch_rope_init(int head_dim, float theta_base);
 
+/* No counterpart in the reference, whose converter drops the checkpoint's rope_scaling entry
+ * (engine/convert_model.py:54) and whose table is always theta^(-2d/head_dim) (kernels.hip:133-134).
+ * t12_rope_freqs writes head_dim / 2 inverse frequencies on the host: that table, and for factor > 0 the
+ * "llama3" rule on top of it -- wavelengths (2 pi / freq) above original_ctx / low_freq_factor are divided
+ * by factor, those below original_ctx / high_freq_factor are kept, the band between is blended linearly in
+ * original_ctx / wavelength.  launch_rope_scaling makes every RoPE launcher of this library use that rule from
+ * then on (process-wide, like the table itself; factor <= 0 switches it off). */
+void t12_rope_freqs(int head_dim, float theta, float factor, float low_freq_factor, float high_freq_factor,
+                    float original_ctx, float* out);
+void launch_rope_scaling(float factor, float low_freq_factor, float high_freq_factor, float original_ctx);
+
 /* kernels.hip:142-147.  output[b, :] = f32(embd_table[token_ids[b], :]); ids outside [0, n_vocab) give zeros. */
 void launch_embed_lookup(const int16_t* embd_table, const int* token_ids, float* output, int n_embd, int batch_size,
                          int n_vocab, hipStream_t stream);

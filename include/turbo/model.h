@@ -20,6 +20,11 @@ struct ModelConfig {
     int n_ctx;
     float rope_theta;
     float rms_norm_eps;
+    // Not in the reference's struct or in config.bin: the checkpoint's rope_scaling entry of the "llama3"
+    // kind (factor, low_freq_factor, high_freq_factor, original_max_position_embeddings), read from the
+    // optional file rope_scaling.bin (4 x float32); factor 0 = plain RoPE, as the reference always does
+    // (engine/convert_model.py:54).
+    float rope_scaling[4];
 };
 
 // One split-12 tensor on the GPU (engine/model.h:21-40).

@@ -207,16 +207,27 @@ def silu_mul_bf16(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
     return f32_to_bf16_bits(s * up.astype(np.float32))
 
 
-def rope_freqs(head_dim: int, theta: float) -> np.ndarray:
-    """freq[d] = 1 / theta^(2d/head_dim), fp32 powf on the host (kernels.hip:129-140)."""
+def rope_freqs(head_dim: int, theta: float, scaling=None) -> np.ndarray:
+    """freq[d] = 1 / theta^(2d/head_dim), fp32 powf on the host (kernels.hip:129-140).
+
+    scaling = (factor, low_freq_factor, high_freq_factor, original_ctx): the "llama3" rule of a checkpoint's
+    rope_scaling entry, which the reference drops (engine/convert_model.py:54).  Not reference behaviour; pinned
+    against transformers' implementation of the published rule in tests/test_convert.py."""
     d = np.arange(head_dim // 2, dtype=np.float32)
-    return (np.float32(1.0) / np.power(np.float32(theta), (2 * d) / np.float32(head_dim), dtype=np.float32)).astype(np.float32)
+    f = (np.float32(1.0) / np.power(np.float32(theta), (2 * d) / np.float32(head_dim), dtype=np.float32)).astype(np.float32)
+    if scaling:
+        factor, low, high, orig = (np.float32(x) for x in scaling)
+        wavelen = np.float32(2 * np.pi) / f
+        smooth = (orig / wavelen - low) / (high - low)
+        mid = (np.float32(1) - smooth) * f / factor + smooth * f
+        f = np.where(wavelen > orig / low, f / factor, np.where(wavelen < orig / high, f, mid)).astype(np.float32)
+    return f
 
 
-def rope(x: np.ndarray, pos: int, n_head: int, head_dim: int, theta: float) -> np.ndarray:
+def rope(x: np.ndarray, pos: int, n_head: int, head_dim: int, theta: float, scaling=None) -> np.ndarray:
     """Rotate-half RoPE: pairs (d, d+hd/2), angle = pos*freq[d] (kernels.hip:174-213)."""
     h = head_dim // 2
-    f = rope_freqs(head_dim, theta).astype(np.float64)
+    f = rope_freqs(head_dim, theta, scaling).astype(np.float64)
     ang = pos * f
     c, s = np.cos(ang), np.sin(ang)
     v = x.astype(np.float64).reshape(n_head, head_dim).copy()
@@ -291,8 +302,8 @@ class RefModel:
             q = gemv(L["wq"], a)
             k = gemv(L["wk"], a)
             v = gemv(L["wv"], a)
-            q = rope(q, pos, nh, hd, theta)
-            k = rope(k, pos, nkv, hd, theta)
+            q = rope(q, pos, nh, hd, theta, c.get("rope_scaling"))
+            k = rope(k, pos, nkv, hd, theta, c.get("rope_scaling"))
             self.kc[li, pos], self.ks[li, pos] = quant_kv_int8(k, nkv, hd)
             self.vc[li, pos], self.vs[li, pos] = quant_kv_int8(v, nkv, hd)
             att = attention_int8(q, self.kc[li], self.vc[li], self.ks[li], self.vs[li], pos + 1, nh, nkv, hd)

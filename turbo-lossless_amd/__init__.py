@@ -58,6 +58,8 @@ _SIGS = {
     # glue launchers (reference names; void return)
     "t12_tune_attention": (_i, [_i]),
     "launch_rope_init": (None, [_i, C.c_float]),
+    "launch_rope_scaling": (None, [C.c_float] * 4),
+    "t12_rope_freqs": (None, [_i] + [C.c_float] * 5 + [_vp]),
     "launch_embed_lookup": (None, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "launch_rms_norm_bf16_batch": (None, [_vp, _vp, _vp, _i, C.c_float, _i, _vp]),
     "launch_add_rms_norm_bf16_batch": (None, [_vp, _vp, _vp, _vp, _i, C.c_float, _i, _vp]),

@@ -38,6 +38,7 @@ void launch_attention_all_heads_batch(const float*, const int8_t*, const int8_t*
 void launch_rope_store_attention_partials(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int16_t*,
                                           const int*, int, int, int, int, float, float, int, const float*, int, size_t,
                                           int, hipStream_t);
+void launch_rope_scaling(float, float, float, float);
 void launch_rope_store_attention(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int16_t*, const int*,
                                  int, int, int, int, float, float, int, int, hipStream_t);
 }
@@ -291,6 +292,9 @@ void forward(InferenceState* state, const int* token_ids)
     const int kv_dim = c.n_head_kv * head_dim;
     const float scale = 1.0f / sqrtf((float)head_dim);
     Impl* impl = (Impl*)state->impl;
+
+    // the RoPE table is library state shared by every model of the process: name this model's rule
+    launch_rope_scaling(c.rope_scaling[0], c.rope_scaling[1], c.rope_scaling[2], c.rope_scaling[3]);
 
     int max_pos = 0;
     for (int b = 0; b < B; b++) max_pos = std::max(max_pos, state->positions[b]);

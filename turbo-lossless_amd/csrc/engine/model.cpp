@@ -208,6 +208,23 @@ Model* load_model(const std::string& model_path, int device_id)
     c.n_vocab = raw.v[0]; c.n_embd = raw.v[1]; c.n_head = raw.v[2]; c.n_head_kv = raw.v[3];
     c.n_layer = raw.v[4]; c.n_ff = raw.v[5]; c.n_ctx = raw.v[6];
     c.rope_theta = raw.theta; c.rms_norm_eps = raw.eps;
+    c.rope_scaling[0] = c.rope_scaling[1] = c.rope_scaling[2] = c.rope_scaling[3] = 0.0f;
+    {
+        std::vector<uint8_t> rs;
+        if (read_file(model_path + "/rope_scaling.bin", rs, true)) {
+            if (rs.size() != 16) {
+                fprintf(stderr, "rope_scaling.bin in %s is not 4 floats\n", model_path.c_str());
+                delete m;
+                return nullptr;
+            }
+            memcpy(c.rope_scaling, rs.data(), 16);
+            if (!(c.rope_scaling[0] > 0.0f) || !(c.rope_scaling[2] > c.rope_scaling[1]) || !(c.rope_scaling[3] > 0.0f)) {
+                fprintf(stderr, "rope_scaling.bin in %s holds impossible values\n", model_path.c_str());
+                delete m;
+                return nullptr;
+            }
+        }
+    }
     if (c.n_vocab <= 0 || c.n_embd <= 0 || c.n_head <= 0 || c.n_head_kv <= 0 || c.n_layer < 0 || c.n_ff <= 0 ||
         c.n_embd % c.n_head || c.n_head % c.n_head_kv) {
         fprintf(stderr, "config.bin in %s holds an impossible shape\n", model_path.c_str());
@@ -413,6 +430,11 @@ bool save_model(const Model* m, const std::string& dir)
         std::ofstream f(dir + "/config.bin", std::ios::binary);
         if (!f) return false;
         f.write((const char*)&raw, sizeof raw);
+    }
+    if (c.rope_scaling[0] > 0.0f) {
+        std::ofstream f(dir + "/rope_scaling.bin", std::ios::binary);
+        if (!f) return false;
+        f.write((const char*)c.rope_scaling, sizeof c.rope_scaling);
     }
     bool ok = dump<int16_t>(dir + "/tok_embd.bin", m->token_embd, (size_t)c.n_vocab * c.n_embd) &&
               dump<float>(dir + "/output_norm.bin", m->output_norm, c.n_embd) &&

@@ -14,11 +14,15 @@
 // float_to_bf16 (kernels.hip:21-27).
 
 #include <cmath>
+#include <cstring>
 #include <mutex>
 #include <vector>
 
 #include "t12_device.h"
 #include "t12_host.h"
+
+extern "C" void t12_rope_freqs(int head_dim, float theta, float factor, float low_freq_factor, float high_freq_factor,
+                               float original_ctx, float* out);
 
 namespace {
 
@@ -708,19 +712,26 @@ float g_freqs_theta = 0.0f;
 ArgPair* g_part = nullptr;
 int g_part_rows = 0;
 
+// Frequency scaling of the "llama3" kind (factor <= 0: none); set by launch_rope_scaling
+float g_rope_scale[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+float g_freqs_scale[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+
 const float* rope_table(int head_dim, float theta)
 {
     std::lock_guard<std::mutex> lock(g_mu);
-    if (g_freqs && g_freqs_dim == head_dim && g_freqs_theta == theta) return g_freqs;
+    if (g_freqs && g_freqs_dim == head_dim && g_freqs_theta == theta &&
+        memcmp(g_freqs_scale, g_rope_scale, sizeof g_rope_scale) == 0)
+        return g_freqs;
     const int half = head_dim / 2;
     std::vector<float> h(half);
-    for (int d = 0; d < half; d++) h[d] = 1.0f / powf(theta, (float)(2 * d) / (float)head_dim);   // kernels.hip:133-134
+    t12_rope_freqs(head_dim, theta, g_rope_scale[0], g_rope_scale[1], g_rope_scale[2], g_rope_scale[3], h.data());
     if (g_freqs) (void)hipFree(g_freqs);
     g_freqs = nullptr;
     if (hipMalloc((void**)&g_freqs, half * sizeof(float)) != hipSuccess) return nullptr;
     if (hipMemcpy(g_freqs, h.data(), half * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) return nullptr;
     g_freqs_dim = head_dim;
     g_freqs_theta = theta;
+    memcpy(g_freqs_scale, g_rope_scale, sizeof g_rope_scale);
     return g_freqs;
 }
 
@@ -820,6 +831,40 @@ void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float
 extern "C" {
 
 void launch_rope_init(int head_dim, float theta_base) { (void)rope_table(head_dim, theta_base); }
+
+// freq[d] = theta^(-2d / head_dim) (kernels.hip:133-134), then, for factor > 0, the "llama3" rule
+// of the checkpoints' rope_scaling entry: wavelengths above original_ctx / low_freq_factor are
+// stretched by factor, those below original_ctx / high_freq_factor are kept, the band between is
+// blended linearly in original_ctx / wavelength.  Host arithmetic only.
+void t12_rope_freqs(int head_dim, float theta, float factor, float low_freq_factor, float high_freq_factor,
+                    float original_ctx, float* out)
+{
+    const int half = head_dim / 2;
+    const float two_pi = 6.283185307179586f;
+    for (int d = 0; d < half; d++) {
+        float f = 1.0f / powf(theta, (float)(2 * d) / (float)head_dim);
+        if (factor > 0.0f) {
+            const float wavelen = two_pi / f;
+            if (wavelen > original_ctx / low_freq_factor) {
+                f = f / factor;
+            } else if (!(wavelen < original_ctx / high_freq_factor)) {
+                const float smooth = (original_ctx / wavelen - low_freq_factor) / (high_freq_factor - low_freq_factor);
+                f = (1.0f - smooth) * f / factor + smooth * f;
+            }
+        }
+        out[d] = f;
+    }
+}
+
+void launch_rope_scaling(float factor, float low_freq_factor, float high_freq_factor, float original_ctx)
+{
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (!(factor > 0.0f)) factor = low_freq_factor = high_freq_factor = original_ctx = 0.0f;
+    g_rope_scale[0] = factor;
+    g_rope_scale[1] = low_freq_factor;
+    g_rope_scale[2] = high_freq_factor;
+    g_rope_scale[3] = original_ctx;
+}
 
 // 1 (default): shapes with a specialised attention kernel use it; 0: always the general kernel.
 int t12_tune_attention(int fast)

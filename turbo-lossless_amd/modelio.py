@@ -12,9 +12,14 @@ TENSORS = ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down")
 
 
 def write_config(path, cfg):
+    """config.bin, and rope_scaling.bin (factor, low_freq_factor, high_freq_factor, original context: four
+    float32; an addition to the reference's layout) when cfg carries a "rope_scaling" tuple."""
     with open(os.path.join(path, "config.bin"), "wb") as f:
         f.write(struct.pack("<iiiiiiiff", cfg["n_vocab"], cfg["n_embd"], cfg["n_head"], cfg["n_head_kv"],
                             cfg["n_layer"], cfg["n_ff"], cfg["n_ctx"], cfg["rope_theta"], cfg["rms_norm_eps"]))
+    if cfg.get("rope_scaling"):
+        with open(os.path.join(path, "rope_scaling.bin"), "wb") as f:
+            f.write(struct.pack("<ffff", *cfg["rope_scaling"]))
 
 
 def write_tensor(path, prefix, p):
