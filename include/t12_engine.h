@@ -28,7 +28,15 @@ int   t12_engine_max_seq(void* model);                               /* Model::m
 int   t12_engine_weight(void* model, int layer, int which, T12Segment* seg, int* K, int* num_patches);
 
 void* t12_engine_create_state(void* model, int batch, int max_seq);  /* create_inference_state (inference.cpp:94-166) */
+/* create_inference_state_per_sequence: batch INDEPENDENT sequences, each with its own KV-cache region of max_seq
+ * positions owned by the state.  No counterpart in the reference, whose batch shares one region (kv_stride = 0,
+ * inference.cpp:427-435).  NULL when the caches do not fit in free device memory. */
+void* t12_engine_create_state_per_sequence(void* model, int batch, int max_seq);
 void  t12_engine_free_state(void* state);                            /* free_inference_state */
+/* prefill: the n_tokens prompt ids (host) of sequence seq go through the layer stack as the rows of a batch
+ * (decode+GEMM kernels, causal), up to batch at a time; leaves the last token's logits in row seq and advances
+ * positions[seq].  The reference prompts one token per forward (inference.cpp:721-724). */
+int   t12_engine_prefill(void* state, int seq, const int* tokens_host, int n_tokens);
 void  t12_engine_set_positions(void* state, const int* pos);         /* state->positions[0..batch) = pos (inference.cpp:722) */
 void  t12_engine_get_positions(void* state, int* pos);
 int   t12_engine_forward(void* state, const int* tokens_host);       /* forward: logits stay on the device */
@@ -42,6 +50,9 @@ int   t12_engine_generate(void* state, const int* prompt, int n_prompt, int max_
 /* decode_greedy: the decode half of generate, from the logits the state holds: up to max_tokens steps of
  * (sample, forward), the next step enqueued before the host has read the token.  out may be NULL. */
 int   t12_engine_decode(void* state, int max_tokens, int stop_on_eos, int* out);
+/* decode_greedy_all: the same loop without the stop rule, every sequence's ids: out[t * batch + b] (host, room
+ * for max_tokens * batch ints, may be NULL); returns the number of steps. */
+int   t12_engine_decode_all(void* state, int max_tokens, int* out);
 
 /* Synthetic tensors on the device (what create_synthetic_model is built from). */
 int   t12_synth_normal_bf16(void* out_bf16, size_t n, uint64_t seed, float sigma, float p_outlier, float sigma_outlier,

@@ -108,16 +108,19 @@ void launch_rope_store_attention(float* q, float* k, const float* v, int8_t* kv_
                                  int n_head_kv, int head_dim, float theta, float scale, int batch_size, int kv_stride,
                                  hipStream_t stream);
 
-/* launch_rope_store_attention for a batch on one shared cache region (kv_stride 0) whose q | k | v projection
- * was one K-split launch of three segments in this order (t12_gemm_deferred): the RoPE / KV-store kernel
- * adds the partial sums up itself (element (b, col) of the fused row = ascending sum over z < nsplit of
- * partials[z * split_stride + b * ld + col]).  q and k receive the rotated values; the v buffer is not
- * written.  No counterpart in the reference. */
+/* launch_rope_store_attention for a batch whose q | k | v projection was one K-split launch of three segments
+ * in this order (t12_gemm_deferred): the RoPE / KV-store kernel adds the partial sums up itself (element
+ * (b, col) of the fused row = ascending sum over z < nsplit of partials[z * split_stride + b * ld + col]).  q and
+ * k receive the rotated values; the v buffer is not written.  kv_stride as in launch_attention_all_heads_batch
+ * (inference.cpp:430,435 pass 0): 0 = one cache region for all rows -- lock-step copies, or the rows of ONE
+ * sequence's prompt at consecutive positions: all rows are stored before any row attends, so row t attends to
+ * rows <= t (a causal prefill); otherwise the element distance between the regions of consecutive sequences
+ * (scale arrays: kv_stride / head_dim).  No counterpart in the reference. */
 void launch_rope_store_attention_partials(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v,
                                           float* scale_k, float* scale_v, int16_t* output, const int* positions,
                                           int position, int n_head, int n_head_kv, int head_dim, float theta,
                                           float scale, int batch_size, const float* partials, int nsplit,
-                                          size_t split_stride, int ld, hipStream_t stream);
+                                          size_t split_stride, int ld, int kv_stride, hipStream_t stream);
 
 /* Benchmark switch: 1 (default) lets shapes with a specialised attention kernel (head_dim 128 with GQA ratio
  * 1/2/4/8, head_dim 64 with ratio 1/4) use it; 0 forces the general kernel. */

@@ -237,3 +237,58 @@ def test_fused_rope_store_attention_equals_separate_launches(t12, oracle, nh, nk
         assert torch.equal(f[3], a[3]) and torch.equal(f[4], a[4])      # caches
         assert torch.equal(f[5], a[5]) and torch.equal(f[6], a[6])      # scales
         assert torch.equal(of, oa)
+
+
+@pytest.mark.parametrize("nh,nkv,hd", [(32, 8, 128), (8, 2, 32), (4, 4, 64)])
+def test_per_sequence_caches_fused_and_from_partial_sums(t12, oracle, nh, nkv, hd):
+    """Independent sequences, each with its own cache region (kv_stride != 0) and its own position: the fused
+    launch and the launch that first adds up K-split partial sums of q | k | v both equal one separate
+    RoPE/store + attention launch per sequence on that sequence's region."""
+    rng = np.random.default_rng(hd)
+    B, theta, max_seq = 3, 500000.0, 96
+    pos = [70, 5, 33]
+    q, k, v = make_qkv(rng, B, nh, nkv, hd)
+    kc = rng.integers(-127, 128, size=(B, max_seq, nkv, hd)).astype(np.int8)
+    vc = rng.integers(-127, 128, size=(B, max_seq, nkv, hd)).astype(np.int8)
+    ks = (rng.random((B, max_seq, nkv)).astype(np.float32) + 0.5) / 127
+    vs = (rng.random((B, max_seq, nkv)).astype(np.float32) + 0.5) / 127
+    pd = torch.tensor(pos, dtype=torch.int32, device=dev())
+    sc = 1.0 / np.sqrt(hd)
+    kv_stride = max_seq * nkv * hd
+    # partial sums of the fused [q | k | v] row: two splits whose fp32 sum is the value itself
+    row = np.concatenate([q.reshape(B, -1), k.reshape(B, -1), v.reshape(B, -1)], axis=1).astype(np.float32)
+    p0 = (rng.standard_normal(row.shape) * 0.5).astype(np.float32)
+    p1 = (row - p0).astype(np.float32)
+    row = (p0 + p1).astype(np.float32)
+    nq, nk = nh * hd, nkv * hd
+    q, k, v = row[:, :nq].copy(), row[:, nq:nq + nk].copy(), row[:, nq + nk:].copy()
+
+    def fresh():
+        return [torch.from_numpy(a.copy()).to(dev()) for a in (q, k, v, kc, vc, ks, vs)]
+
+    a = fresh(); oa = torch.zeros((B, nq), dtype=torch.int16, device=dev())
+    for b in range(B):                      # one sequence at a time on its own region
+        t12.lib.launch_rope_store_kv_batch(a[0][b].data_ptr(), a[1][b].data_ptr(), a[2][b].data_ptr(), a[3][b].data_ptr(),
+                                           a[4][b].data_ptr(), a[5][b].data_ptr(), a[6][b].data_ptr(), pd[b:].data_ptr(),
+                                           hd, nh, nkv, nq, nk, theta, 1, st(t12))
+        t12.lib.launch_attention_all_heads_batch(a[0][b].data_ptr(), a[3][b].data_ptr(), a[4][b].data_ptr(),
+                                                 a[5][b].data_ptr(), a[6][b].data_ptr(), oa[b].data_ptr(), pd[b:].data_ptr(),
+                                                 nh, nkv, hd, max_seq, sc, 1, 0, st(t12))
+    f = fresh(); of = torch.zeros_like(oa)
+    t12.lib.launch_rope_store_attention(f[0].data_ptr(), f[1].data_ptr(), f[2].data_ptr(), f[3].data_ptr(), f[4].data_ptr(),
+                                        f[5].data_ptr(), f[6].data_ptr(), of.data_ptr(), pd.data_ptr(), 0, nh, nkv, hd,
+                                        theta, sc, B, kv_stride, st(t12))
+    g = fresh(); og = torch.zeros_like(oa)
+    g[0].zero_(); g[1].zero_(); g[2].zero_()                  # the values come from the partial sums only
+    ws = torch.from_numpy(np.stack([p0, p1])).to(dev())
+    t12.lib.launch_rope_store_attention_partials(g[0].data_ptr(), g[1].data_ptr(), g[2].data_ptr(), g[3].data_ptr(),
+                                                 g[4].data_ptr(), g[5].data_ptr(), g[6].data_ptr(), og.data_ptr(),
+                                                 pd.data_ptr(), 0, nh, nkv, hd, theta, sc, B, ws.data_ptr(), 2,
+                                                 B * row.shape[1], row.shape[1], kv_stride, st(t12))
+    torch.cuda.synchronize()
+    assert not torch.equal(a[3], torch.from_numpy(kc).to(dev()))         # the stores happened
+    for x in (f, g):
+        assert torch.equal(x[3], a[3]) and torch.equal(x[4], a[4])      # caches: only each sequence's own slot changed
+        assert torch.equal(x[5], a[5]) and torch.equal(x[6], a[6])      # scales
+    assert torch.equal(of, oa) and torch.equal(og, oa)
+    assert not torch.equal(oa[0], oa[1])

@@ -70,6 +70,8 @@ _SIGS = {
     "launch_rope_store_kv": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _vp]),
     "launch_rope_store_kv_batch": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _i, _vp]),
     "launch_rope_store_attention": (None, [_vp] * 9 + [_i, _i, _i, _i, C.c_float, C.c_float, _i, _i, _vp]),
+    "launch_rope_store_attention_partials": (None, [_vp] * 9 + [_i, _i, _i, _i, C.c_float, C.c_float, _i, _vp, _i,
+                                                    C.c_size_t, _i, _i, _vp]),
     "launch_attention_all_heads": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _vp]),
     "launch_flash_attention": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _vp]),
     "launch_attention_all_heads_batch": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, C.c_float, _i, _i, _vp]),
@@ -82,6 +84,9 @@ _SIGS = {
     "t12_engine_save": (_i, [_vp, C.c_char_p]),
     "t12_engine_free_model": (None, [_vp]),
     "t12_engine_create_state": (_vp, [_vp, _i, _i]),
+    "t12_engine_create_state_per_sequence": (_vp, [_vp, _i, _i]),
+    "t12_engine_prefill": (_i, [_vp, _i, C.POINTER(C.c_int), _i]),
+    "t12_engine_decode_all": (_i, [_vp, _i, C.POINTER(C.c_int)]),
     "t12_engine_free_state": (None, [_vp]),
     "t12_engine_forward": (_i, [_vp, C.POINTER(C.c_int)]),
     "t12_engine_logits": (_vp, [_vp]),
@@ -263,32 +268,53 @@ def pack_device(w, base_exp=None, stream=None) -> DeviceTensor12:
 class Engine:
     """The engine's load / forward / sample / generate API (include/turbo/*.h) through its C face."""
 
-    def __init__(self, model_handle, batch=1):
+    def __init__(self, model_handle, batch=1, per_sequence=0):
+        """per_sequence = N > 0: batch independent sequences, each with its own KV cache of N positions
+        (create_inference_state_per_sequence); 0: the reference's one shared cache region."""
         if not model_handle:
             raise T12Error("model could not be loaded/created")
         self.model = model_handle
         self.batch = batch
-        self.state = lib.t12_engine_create_state(self.model, batch, 0)
+        self.state = self._make_state(batch, per_sequence)
+
+    def _make_state(self, batch, per_sequence):
+        if per_sequence:
+            st = lib.t12_engine_create_state_per_sequence(self.model, batch, int(per_sequence))
+            if not st:
+                raise T12Error("per-sequence KV cache could not be created")
+            return st
+        return lib.t12_engine_create_state(self.model, batch, 0)
 
     @classmethod
-    def load(cls, path, batch=1, device=0):
-        return cls(lib.t12_engine_load(os.fsencode(path), device), batch)
+    def load(cls, path, batch=1, device=0, per_sequence=0):
+        return cls(lib.t12_engine_load(os.fsencode(path), device), batch, per_sequence)
 
     @classmethod
-    def synthetic(cls, cfg, seed=4000, max_seq=2048, batch=1, p_outlier=3e-4):
+    def synthetic(cls, cfg, seed=4000, max_seq=2048, batch=1, p_outlier=3e-4, per_sequence=0):
         h = lib.t12_engine_create_synthetic(cfg["n_vocab"], cfg["n_embd"], cfg["n_head"], cfg["n_head_kv"],
                                             cfg["n_layer"], cfg["n_ff"], cfg.get("n_ctx", max_seq),
                                             cfg.get("rope_theta", 500000.0), cfg.get("rms_norm_eps", 1e-5), seed,
                                             max_seq, p_outlier)
-        return cls(h, batch)
+        return cls(h, batch, per_sequence)
 
-    def new_state(self, batch):
-        """A second InferenceState on the same model (they share the model's KV cache)."""
+    def new_state(self, batch, per_sequence=0):
+        """A second InferenceState on the same model (shared-region states share the model's KV cache)."""
         e = Engine.__new__(Engine)
         e.model, e.batch = self.model, batch
-        e.state = lib.t12_engine_create_state(self.model, batch, 0)
+        e.state = e._make_state(batch, per_sequence)
         e._borrowed = True
         return e
+
+    def prefill(self, seq, tokens):
+        """Batched prompt pass of sequence seq (rows = prompt tokens, up to batch at a time)."""
+        arr = (C.c_int * max(len(tokens), 1))(*[int(t) for t in tokens])
+        check(lib.t12_engine_prefill(self.state, int(seq), arr, len(tokens)), "prefill")
+
+    def decode_all(self, max_tokens):
+        """max_tokens greedy steps from the current logits; ids of every sequence as [steps][batch]."""
+        out = (C.c_int * max(max_tokens * self.batch, 1))()
+        n = lib.t12_engine_decode_all(self.state, max_tokens, out)
+        return [list(out[t * self.batch:(t + 1) * self.batch]) for t in range(n)]
 
     def save(self, path):
         check(lib.t12_engine_save(self.model, os.fsencode(path)), "save_model")

@@ -26,7 +26,17 @@ void* t12_engine_create_state(void* model, int batch, int max_seq)
 {
     return create_inference_state((Model*)model, batch, max_seq);
 }
+void* t12_engine_create_state_per_sequence(void* model, int batch, int max_seq)
+{
+    return create_inference_state_per_sequence((Model*)model, batch, max_seq);
+}
 void t12_engine_free_state(void* state) { free_inference_state((InferenceState*)state); }
+
+int t12_engine_prefill(void* state, int seq, const int* tokens_host, int n_tokens)
+{
+    prefill((InferenceState*)state, seq, tokens_host, n_tokens);
+    return 0;
+}
 
 int t12_engine_forward(void* state, const int* tokens_host)
 {
@@ -71,6 +81,16 @@ int t12_engine_decode(void* state, int max_tokens, int stop_on_eos, int* out)
     if (out)
         for (size_t i = 0; i < r.size(); i++) out[i] = r[i];
     return (int)r.size();
+}
+
+// decode_greedy_all(); out is a host array [max_tokens][batch]; returns the number of steps.
+int t12_engine_decode_all(void* state, int max_tokens, int* out)
+{
+    auto* s = (InferenceState*)state;
+    std::vector<int> r = decode_greedy_all(s, max_tokens);
+    if (out)
+        for (size_t i = 0; i < r.size(); i++) out[i] = r[i];
+    return (int)(r.size() / (size_t)s->batch_size);
 }
 
 int t12_engine_sync(void* state)

@@ -37,7 +37,7 @@ void launch_attention_all_heads_batch(const float*, const int8_t*, const int8_t*
                                       const int*, int, int, int, int, float, int, int, hipStream_t);
 void launch_rope_store_attention_partials(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int16_t*,
                                           const int*, int, int, int, int, float, float, int, const float*, int, size_t,
-                                          int, hipStream_t);
+                                          int, int, hipStream_t);
 void launch_rope_scaling(float, float, float, float);
 void launch_rope_store_attention(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int16_t*, const int*,
                                  int, int, int, int, float, float, int, int, hipStream_t);
@@ -56,7 +56,29 @@ struct Impl {
     // pipelined greedy decoding: sampled tokens land in pinned host memory, two slots in rotation
     int* h_tokens[2] = {nullptr, nullptr};
     hipEvent_t sampled[2] = {nullptr, nullptr};
+    // per-sequence KV caches owned by the state (create_inference_state_per_sequence):
+    // int8 [n_layer][batch][max_seq][kv_dim] twice, scales fp32 [n_layer][batch][max_seq][n_head_kv] twice
+    bool per_seq = false;
+    int seq_len = 0;
+    int8_t* pk = nullptr;
+    int8_t* pv = nullptr;
+    float* psk = nullptr;
+    float* psv = nullptr;
 };
+
+// Where a forward reads and writes the KV cache: layer l of sequence b starts at
+// k + l * layer_kv + b * kv_stride (scales: sk + l * layer_sc + b * kv_stride / head_dim).
+struct KvView {
+    int8_t* k;
+    int8_t* v;
+    float* sk;
+    float* sv;
+    size_t layer_kv, layer_sc;
+    int kv_stride;      // 0: every row of the batch works on one region
+    int max_seq;
+};
+
+enum LogitsMode { LOGITS_ALL, LOGITS_LAST_ROW, LOGITS_NONE };
 
 void check_gpu(hipError_t e, const char* what)
 {
@@ -164,6 +186,38 @@ InferenceState* create_inference_state(Model* model, int batch_size, int max_seq
     return s;
 }
 
+// Extension (the reference shares one cache region across the batch, inference.cpp:427-435): a state whose
+// sequences are independent -- own KV cache region each, own tokens, own positions.
+InferenceState* create_inference_state_per_sequence(Model* model, int batch_size, int max_seq_len)
+{
+    const ModelConfig& c = model->config;
+    const int head_dim = c.n_embd / c.n_head;
+    const size_t kv_dim = (size_t)c.n_head_kv * head_dim;
+    if (batch_size < 1 || max_seq_len < 1 || (size_t)max_seq_len * kv_dim > 0x7FFFFFFFu) {
+        fprintf(stderr, "ERROR: per-sequence KV cache: batch %d x %d positions is not a usable shape\n", batch_size,
+                max_seq_len);
+        return nullptr;
+    }
+    const size_t rows = (size_t)c.n_layer * batch_size * max_seq_len;
+    size_t free_b = 0, total_b = 0;
+    (void)hipMemGetInfo(&free_b, &total_b);
+    const size_t need = 2 * rows * kv_dim + 2 * rows * c.n_head_kv * sizeof(float);
+    if (need > free_b) {
+        fprintf(stderr, "ERROR: per-sequence KV cache needs %.1f GB, %.1f GB free\n", need / 1e9, free_b / 1e9);
+        return nullptr;
+    }
+    InferenceState* s = create_inference_state(model, batch_size, max_seq_len);
+    Impl* impl = (Impl*)s->impl;
+    impl->per_seq = true;
+    impl->seq_len = max_seq_len;
+    check_gpu(hipMalloc((void**)&impl->pk, rows * kv_dim), "hipMalloc");
+    check_gpu(hipMalloc((void**)&impl->pv, rows * kv_dim), "hipMalloc");
+    check_gpu(hipMalloc((void**)&impl->psk, rows * c.n_head_kv * sizeof(float)), "hipMalloc");
+    check_gpu(hipMalloc((void**)&impl->psv, rows * c.n_head_kv * sizeof(float)), "hipMalloc");
+    printf("  Per-sequence KV cache: %d x %d positions, %.2f GB\n", batch_size, max_seq_len, need / 1e9);
+    return s;
+}
+
 void free_inference_state(InferenceState* state)
 {
     if (!state) return;
@@ -183,6 +237,8 @@ void free_inference_state(InferenceState* state)
             if (impl->h_tokens[i]) (void)hipHostFree(impl->h_tokens[i]);
             if (impl->sampled[i]) (void)hipEventDestroy(impl->sampled[i]);
         }
+        for (void* p : {(void*)impl->pk, (void*)impl->pv, (void*)impl->psk, (void*)impl->psv})
+            if (p) (void)hipFree(p);
     }
     delete impl;
     delete state;
@@ -221,7 +277,7 @@ void must(int rc, const char* what)
 // The residual stream ping-pongs between hidden and hidden2 (a norm prologue reads one and
 // workgroup 0 writes the sum into the other); the additions the reference does in
 // add_rms_norm_bf16_batch (inference.cpp:301,341-346) happen in the prologue of the next linear.
-void forward_b1_fused(InferenceState* state, const int* token_ids)
+void forward_b1_fused(InferenceState* state, const int* token_ids, const KvView& kv)
 {
     Model* m = state->model;
     const ModelConfig& c = m->config;
@@ -248,11 +304,11 @@ void forward_b1_fused(InferenceState* state, const int* token_ids)
         S.qkv[2] = seg_of(L.wv, state->v_buf, kv_dim);
         must(t12_gemv_norm(S.qkv, 3, h, nullptr, L.attn_norm, c.rms_norm_eps, nullptr, n, st), "qkv decode-GEMV");
 
-        const size_t kv_off = (size_t)layer * m->max_seq_len * kv_dim;
-        const size_t sc_off = (size_t)layer * m->max_seq_len * c.n_head_kv;
-        launch_rope_store_attention(state->q_buf, state->k_buf, state->v_buf, m->kv_cache_k + kv_off,
-                                    m->kv_cache_v + kv_off, m->kv_scale_k + sc_off, m->kv_scale_v + sc_off, bf16_a,
-                                    nullptr, pos, c.n_head, c.n_head_kv, head_dim, c.rope_theta, scale, 1, 0, st);
+        const size_t kv_off = (size_t)layer * kv.layer_kv;
+        const size_t sc_off = (size_t)layer * kv.layer_sc;
+        launch_rope_store_attention(state->q_buf, state->k_buf, state->v_buf, kv.k + kv_off, kv.v + kv_off,
+                                    kv.sk + sc_off, kv.sv + sc_off, bf16_a, nullptr, pos, c.n_head, c.n_head_kv,
+                                    head_dim, c.rope_theta, scale, 1, 0, st);
 
         S.o[0] = seg_of(L.wo, h_alt, n);
         must(t12_gemv_add(S.o, bf16_a, n, h, st), "wo decode-GEMV");                  // h_alt = h + wo . attn
@@ -280,40 +336,40 @@ void forward_b1_fused(InferenceState* state, const int* token_ids)
     state->positions[0] = pos + 1;
 }
 
-}  // namespace
 
-void forward(InferenceState* state, const int* token_ids)
+// The KV cache a state works on: its own per-sequence regions, or the model's one region.
+KvView kv_view(const InferenceState* state)
+{
+    const Model* m = state->model;
+    const ModelConfig& c = m->config;
+    const Impl* impl = (const Impl*)state->impl;
+    const int kv_dim = c.n_head_kv * (c.n_embd / c.n_head);
+    KvView kv;
+    if (impl->per_seq) {
+        const size_t S = (size_t)impl->seq_len, B = (size_t)state->batch_size;
+        kv = KvView{impl->pk, impl->pv, impl->psk, impl->psv, B * S * kv_dim, B * S * c.n_head_kv, (int)(S * kv_dim),
+                    impl->seq_len};
+    } else {
+        kv = KvView{m->kv_cache_k, m->kv_cache_v, m->kv_scale_k, m->kv_scale_v, (size_t)m->max_seq_len * kv_dim,
+                    (size_t)m->max_seq_len * c.n_head_kv, 0, m->max_seq_len};
+    }
+    return kv;
+}
+
+// One pass of the layer stack over R rows (R <= batch_size) whose token ids are in state->d_tokens and, for
+// R > 1, whose positions are in state->d_positions; pos0 = position of row 0.  Logits: for every row into
+// state->logits (LOGITS_ALL), for the last row only into logits_last (LOGITS_LAST_ROW), or not at all.
+void forward_rows(InferenceState* state, int R, const KvView& kv, int pos0, LogitsMode lm, float* logits_last)
 {
     Model* m = state->model;
     const ModelConfig& c = m->config;
     hipStream_t st = state->stream;
-    const int B = state->batch_size;
+    const int B = R;
     const int n = c.n_embd, n_ff = c.n_ff, head_dim = n / c.n_head;
     const int kv_dim = c.n_head_kv * head_dim;
     const float scale = 1.0f / sqrtf((float)head_dim);
     Impl* impl = (Impl*)state->impl;
 
-    // the RoPE table is library state shared by every model of the process: name this model's rule
-    launch_rope_scaling(c.rope_scaling[0], c.rope_scaling[1], c.rope_scaling[2], c.rope_scaling[3]);
-
-    int max_pos = 0;
-    for (int b = 0; b < B; b++) max_pos = std::max(max_pos, state->positions[b]);
-    if (max_pos >= m->max_seq_len) {
-        fprintf(stderr, "ERROR: position %d exceeds the KV cache (%d)\n", max_pos, m->max_seq_len);
-        exit(1);
-    }
-    if (B == 1 && impl->fused_b1) {
-        if (!impl->checked) {
-            impl->checked = true;
-            impl->fused_b1 = fused_b1_eligible(m);
-        }
-        if (impl->fused_b1) {
-            forward_b1_fused(state, token_ids);
-            return;
-        }
-    }
-    if (token_ids) (void)hipMemcpyAsync(state->d_tokens, token_ids, B * sizeof(int), hipMemcpyHostToDevice, st);
-    if (B > 1) (void)hipMemcpyAsync(state->d_positions, state->positions, B * sizeof(int), hipMemcpyHostToDevice, st);
     launch_embed_lookup(m->token_embd, state->d_tokens, state->hidden, n, B, c.n_vocab, st);
 
     float* cur = state->hidden;    // residual stream
@@ -340,20 +396,18 @@ void forward(InferenceState* state, const int* token_ids)
             run_linear(S.qkv, 3, bf16_a, n, B, st);
         }
 
-        const size_t kv_off = (size_t)layer * m->max_seq_len * kv_dim;
-        const size_t sc_off = (size_t)layer * m->max_seq_len * c.n_head_kv;
+        const size_t kv_off = (size_t)layer * kv.layer_kv;
+        const size_t sc_off = (size_t)layer * kv.layer_sc;
         // RoPE (Q, K) + INT8 KV store + GQA attention
         if (qkv_part.nsplit > 1)
-            launch_rope_store_attention_partials(state->q_buf, state->k_buf, state->v_buf, m->kv_cache_k + kv_off,
-                                                 m->kv_cache_v + kv_off, m->kv_scale_k + sc_off, m->kv_scale_v + sc_off,
-                                                 bf16_a, state->d_positions, state->positions[0], c.n_head, c.n_head_kv,
-                                                 head_dim, c.rope_theta, scale, B, qkv_part.ws, qkv_part.nsplit,
-                                                 qkv_part.split_stride, qkv_part.ld, st);
+            launch_rope_store_attention_partials(state->q_buf, state->k_buf, state->v_buf, kv.k + kv_off, kv.v + kv_off,
+                                                 kv.sk + sc_off, kv.sv + sc_off, bf16_a, state->d_positions, pos0,
+                                                 c.n_head, c.n_head_kv, head_dim, c.rope_theta, scale, B, qkv_part.ws,
+                                                 qkv_part.nsplit, qkv_part.split_stride, qkv_part.ld, kv.kv_stride, st);
         else
-            launch_rope_store_attention(state->q_buf, state->k_buf, state->v_buf, m->kv_cache_k + kv_off,
-                                        m->kv_cache_v + kv_off, m->kv_scale_k + sc_off, m->kv_scale_v + sc_off, bf16_a,
-                                        B == 1 ? nullptr : state->d_positions, state->positions[0], c.n_head,
-                                        c.n_head_kv, head_dim, c.rope_theta, scale, B, 0, st);
+            launch_rope_store_attention(state->q_buf, state->k_buf, state->v_buf, kv.k + kv_off, kv.v + kv_off,
+                                        kv.sk + sc_off, kv.sv + sc_off, bf16_a, B == 1 ? nullptr : state->d_positions,
+                                        pos0, c.n_head, c.n_head_kv, head_dim, c.rope_theta, scale, B, kv.kv_stride, st);
 
         S.o[0] = seg_of(L.wo, res, n);
         if (B > 1) {
@@ -396,9 +450,107 @@ void forward(InferenceState* state, const int* token_ids)
     }
     if (c.n_layer == 0) launch_rms_norm_bf16_batch(cur, m->output_norm, bf16_a, n, c.rms_norm_eps, B, st);
 
-    impl->head[0] = seg_of(m->output_proj, state->logits, c.n_vocab);
-    run_linear(impl->head, 1, bf16_a, n, B, st);
+    if (lm == LOGITS_ALL) {
+        impl->head[0] = seg_of(m->output_proj, state->logits, c.n_vocab);
+        run_linear(impl->head, 1, bf16_a, n, B, st);
+    } else if (lm == LOGITS_LAST_ROW) {
+        impl->head[0] = seg_of(m->output_proj, logits_last, c.n_vocab);
+        run_linear(impl->head, 1, bf16_a + (size_t)(B - 1) * n, n, 1, st);
+    }
+}
+
+}  // namespace
+
+void forward(InferenceState* state, const int* token_ids)
+{
+    Model* m = state->model;
+    const ModelConfig& c = m->config;
+    hipStream_t st = state->stream;
+    const int B = state->batch_size;
+    Impl* impl = (Impl*)state->impl;
+
+    // the RoPE table is library state shared by every model of the process: name this model's rule
+    launch_rope_scaling(c.rope_scaling[0], c.rope_scaling[1], c.rope_scaling[2], c.rope_scaling[3]);
+
+    const KvView kv = kv_view(state);
+    int max_pos = 0;
+    for (int b = 0; b < B; b++) max_pos = std::max(max_pos, state->positions[b]);
+    if (max_pos >= kv.max_seq) {
+        fprintf(stderr, "ERROR: position %d exceeds the KV cache (%d)\n", max_pos, kv.max_seq);
+        exit(1);
+    }
+    if (B == 1 && impl->fused_b1) {
+        if (!impl->checked) {
+            impl->checked = true;
+            impl->fused_b1 = fused_b1_eligible(m);
+        }
+        if (impl->fused_b1) {
+            forward_b1_fused(state, token_ids, kv);
+            return;
+        }
+    }
+    if (token_ids) (void)hipMemcpyAsync(state->d_tokens, token_ids, B * sizeof(int), hipMemcpyHostToDevice, st);
+    if (B > 1) (void)hipMemcpyAsync(state->d_positions, state->positions, B * sizeof(int), hipMemcpyHostToDevice, st);
+    forward_rows(state, B, kv, state->positions[0], LOGITS_ALL, nullptr);
     for (int b = 0; b < B; b++) state->positions[b]++;
+}
+
+// Batched prefill (extension; the reference prompts one token per forward, inference.cpp:721-724): the n
+// prompt tokens of ONE sequence go through the layer stack as the rows of a batch, up to batch_size at a
+// time, at consecutive positions on that sequence's cache region.  Every row's K / V is stored before any
+// row attends, and row t attends to positions <= its own, so this is the causal prompt pass; the linears
+// run on the decode+GEMM kernels.  Only the last token's logits are computed (row `seq` of state->logits).
+// A state on the model's shared region (lock-step copies) advances every row and gets the logits in every row.
+void prefill(InferenceState* state, int seq, const int* token_ids, int n_tokens)
+{
+    Model* m = state->model;
+    const ModelConfig& c = m->config;
+    hipStream_t st = state->stream;
+    const int B = state->batch_size;
+    Impl* impl = (Impl*)state->impl;
+    if (seq < 0 || seq >= B || n_tokens < 0) {
+        fprintf(stderr, "ERROR: prefill: sequence %d outside the batch of %d, or negative length\n", seq, B);
+        exit(1);
+    }
+    if (n_tokens == 0) return;
+    if (B == 1) {                                   // nothing to batch over: the decode path, token by token
+        for (int i = 0; i < n_tokens; i++) forward(state, token_ids + i);
+        return;
+    }
+    launch_rope_scaling(c.rope_scaling[0], c.rope_scaling[1], c.rope_scaling[2], c.rope_scaling[3]);
+    KvView kv = kv_view(state);
+    const int head_dim = c.n_embd / c.n_head;
+    const int p0 = state->positions[seq];
+    if (p0 + n_tokens > kv.max_seq) {
+        fprintf(stderr, "ERROR: position %d exceeds the KV cache (%d)\n", p0 + n_tokens - 1, kv.max_seq);
+        exit(1);
+    }
+    // the rows of a chunk share this sequence's region
+    kv.k += (size_t)seq * kv.kv_stride;
+    kv.v += (size_t)seq * kv.kv_stride;
+    kv.sk += (size_t)seq * (kv.kv_stride / head_dim);
+    kv.sv += (size_t)seq * (kv.kv_stride / head_dim);
+    kv.kv_stride = 0;
+    float* row_logits = state->logits + (size_t)(impl->per_seq ? seq : 0) * c.n_vocab;
+    std::vector<int> pos(B);
+    for (int done = 0; done < n_tokens;) {
+        const int R = std::min(B, n_tokens - done);
+        const bool last = done + R == n_tokens;
+        for (int r = 0; r < R; r++) pos[r] = p0 + done + r;
+        (void)hipMemcpyAsync(state->d_tokens, token_ids + done, R * sizeof(int), hipMemcpyHostToDevice, st);
+        (void)hipMemcpyAsync(state->d_positions, pos.data(), R * sizeof(int), hipMemcpyHostToDevice, st);
+        forward_rows(state, R, kv, p0 + done, last ? LOGITS_LAST_ROW : LOGITS_NONE, row_logits);
+        // pos[] is reused by the next chunk: the copies above read it when they are issued (pageable memory)
+        done += R;
+    }
+    if (impl->per_seq) {
+        state->positions[seq] = p0 + n_tokens;
+    } else {
+        for (int b = 1; b < B; b++)
+            (void)hipMemcpyAsync(state->logits + (size_t)b * c.n_vocab, row_logits, (size_t)c.n_vocab * sizeof(float),
+                                 hipMemcpyDeviceToDevice, st);
+        for (int b = 0; b < B; b++) state->positions[b] = p0 + n_tokens;
+    }
 }
 
 // Greedy decoding from the logits the state holds, `max_tokens` steps of (sample, forward).
@@ -409,7 +561,8 @@ void forward(InferenceState* state, const int* token_ids)
 // token t while the GPU already computes step t + 1.  Same tokens, same stop rule (id 2 of sequence
 // 0 ends the stream when stop_on_eos): the one forward issued past an end-of-stream token is undone
 // by stepping the positions back.  TURBO_NO_PIPELINE=1 restores the reference's order.
-std::vector<int> decode_greedy(InferenceState* state, int max_tokens, bool stop_on_eos)
+namespace {
+std::vector<int> decode_loop(InferenceState* state, int max_tokens, bool stop_on_eos, bool all_rows)
 {
     std::vector<int> output;
     const int n_vocab = state->model->config.n_vocab;
@@ -422,7 +575,8 @@ std::vector<int> decode_greedy(InferenceState* state, int max_tokens, bool stop_
             if (bs == 1) tokens[0] = sample_greedy(state->logits, n_vocab, st);
             else sample_greedy_batch(state->logits, tokens.data(), n_vocab, bs, st);
             if (stop_on_eos && tokens[0] == 2) break;
-            output.push_back(tokens[0]);
+            if (all_rows) output.insert(output.end(), tokens.begin(), tokens.end());
+            else output.push_back(tokens[0]);
             forward(state, tokens.data());
         }
         return output;
@@ -449,10 +603,22 @@ std::vector<int> decode_greedy(InferenceState* state, int max_tokens, bool stop_
             for (int b = 0; b < bs; b++) state->positions[b]--;   // the forward on the end-of-stream id does not count
             break;
         }
-        output.push_back(tok);
+        if (all_rows) output.insert(output.end(), impl->h_tokens[t & 1], impl->h_tokens[t & 1] + bs);
+        else output.push_back(tok);
     }
     check_gpu(hipStreamSynchronize(st), "hipStreamSynchronize");
     return output;
+}
+}  // namespace
+
+std::vector<int> decode_greedy(InferenceState* state, int max_tokens, bool stop_on_eos)
+{
+    return decode_loop(state, max_tokens, stop_on_eos, false);
+}
+
+std::vector<int> decode_greedy_all(InferenceState* state, int max_tokens)
+{
+    return decode_loop(state, max_tokens, false, true);
 }
 
 std::vector<int> generate(InferenceState* state, const std::vector<int>& prompt_tokens, int max_tokens)

@@ -185,7 +185,8 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(float* __restrict__ q, floa
                                                      float* __restrict__ sv, const float* __restrict__ freqs,
                                                      const int* __restrict__ positions, int position,
                                                      int head_dim, int n_head, int n_head_kv, int q_stride,
-                                                     int k_stride, QkvPartials part = QkvPartials{nullptr, 0, 0, 0})
+                                                     int k_stride, QkvPartials part = QkvPartials{nullptr, 0, 0, 0},
+                                                     size_t kv_stride = 0)
 {
     const int b = blockIdx.y;
     const int pos = positions ? positions[b] : position;
@@ -249,12 +250,13 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(float* __restrict__ q, floa
         const float amax = wave_max(fmaxf(fabsf(r0), fabsf(r1)));
         const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
         const size_t kv_dim = (size_t)n_head_kv * head_dim;
-        int8_t* row = dst + (size_t)pos * kv_dim + (size_t)kvh * head_dim;
+        // per-sequence caches: sequence b's region starts kv_stride elements (kv_stride / head_dim scales) further on
+        int8_t* row = dst + (size_t)b * kv_stride + (size_t)pos * kv_dim + (size_t)kvh * head_dim;
         if (own) {
             row[lane] = (int8_t)(int)fminf(fmaxf(rintf(r0 * inv), -127.0f), 127.0f);
             row[lane + half] = (int8_t)(int)fminf(fmaxf(rintf(r1 * inv), -127.0f), 127.0f);
         }
-        if (lane == 0) sdst[(size_t)pos * n_head_kv + kvh] = amax / 127.0f;
+        if (lane == 0) sdst[(size_t)b * (kv_stride / head_dim) + (size_t)pos * n_head_kv + kvh] = amax / 127.0f;
     }
 }
 
@@ -761,7 +763,8 @@ void report(const char* what)
 template <int MODE>
 void launch_rope_kv(float* q, float* k, const float* v, int8_t* ck, int8_t* cv, float* sk, float* sv,
                     const int* positions, int position, int head_dim, int n_head, int n_head_kv, int q_stride,
-                    int k_stride, float theta, int batch, hipStream_t st, QkvPartials part = QkvPartials{nullptr, 0, 0, 0})
+                    int k_stride, float theta, int batch, hipStream_t st, QkvPartials part = QkvPartials{nullptr, 0, 0, 0},
+                    size_t kv_stride = 0)
 {
     const float* f = nullptr;
     if (MODE & 1) {
@@ -774,7 +777,7 @@ void launch_rope_kv(float* q, float* k, const float* v, int8_t* ck, int8_t* cv, 
         return;
     }
     hipLaunchKernelGGL(rope_kv_kernel<MODE>, dim3(n_head + 2 * n_head_kv, batch), dim3(64), 0, st, q, k, v, ck, cv, sk,
-                       sv, f, positions, position, head_dim, n_head, n_head_kv, q_stride, k_stride, part);
+                       sv, f, positions, position, head_dim, n_head, n_head_kv, q_stride, k_stride, part, kv_stride);
     report("rope/kv-store");
 }
 
@@ -1000,19 +1003,23 @@ void launch_rope_store_attention(float* q, float* k, const float* v, int8_t* kv_
         return;
     }
     launch_rope_kv<3>(q, k, v, kv_k, kv_v, scale_k, scale_v, positions, position, head_dim, n_head, n_head_kv,
-                      n_head * head_dim, n_head_kv * head_dim, theta, batch_size, stream);
+                      n_head * head_dim, n_head_kv * head_dim, theta, batch_size, stream, QkvPartials{nullptr, 0, 0, 0},
+                      (size_t)kv_stride);
     launch_attn(q, kv_k, kv_v, scale_k, scale_v, output, positions, position + 1, n_head, n_head_kv, head_dim, scale,
                 batch_size, (size_t)kv_stride, stream);
 }
 
-// launch_rope_store_attention for a batch on one shared cache region whose q | k | v projection was split
-// along K (t12_gemm_deferred, one launch for the three tensors in this order): the RoPE / KV-store kernel adds
-// the partial sums up itself.  q and k receive the rotated values; the v buffer is not written.
+// launch_rope_store_attention for a batch whose q | k | v projection was split along K (t12_gemm_deferred,
+// one launch for the three tensors in this order): the RoPE / KV-store kernel adds the partial sums up
+// itself.  q and k receive the rotated values; the v buffer is not written.  kv_stride = 0: one shared cache
+// region (lock-step copies, or the rows of one sequence's prompt at consecutive positions -- every row's
+// K / V is stored before any row attends, so row t sees rows <= t: a causal prefill); otherwise the element
+// distance between the regions of consecutive sequences.
 void launch_rope_store_attention_partials(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v,
                                           float* scale_k, float* scale_v, int16_t* output, const int* positions,
                                           int position, int n_head, int n_head_kv, int head_dim, float theta,
                                           float scale, int batch_size, const float* partials, int nsplit,
-                                          size_t split_stride, int ld, hipStream_t stream)
+                                          size_t split_stride, int ld, int kv_stride, hipStream_t stream)
 {
     if (!partials || nsplit < 1 || nsplit > T12_MAX_KSPLIT || ld < (n_head + 2 * n_head_kv) * head_dim) {
         t12_set_error("rope_store_attention_partials: nsplit %d outside 1..%d, null partials or ld %d too small", nsplit,
@@ -1022,9 +1029,9 @@ void launch_rope_store_attention_partials(float* q, float* k, const float* v, in
     }
     launch_rope_kv<3>(q, k, v, kv_k, kv_v, scale_k, scale_v, positions, position, head_dim, n_head, n_head_kv,
                       n_head * head_dim, n_head_kv * head_dim, theta, batch_size, stream,
-                      QkvPartials{partials, nsplit, ld, split_stride});
+                      QkvPartials{partials, nsplit, ld, split_stride}, (size_t)kv_stride);
     launch_attn(q, kv_k, kv_v, scale_k, scale_v, output, positions, position + 1, n_head, n_head_kv, head_dim, scale,
-                batch_size, 0, stream);
+                batch_size, (size_t)kv_stride, stream);
 }
 
 void launch_attention_all_heads(const float* q, const int8_t* k_cache, const int8_t* v_cache, const float* scale_k,
