@@ -122,9 +122,13 @@ void launch_rope_store_attention_partials(float* q, float* k, const float* v, in
                                           float scale, int batch_size, const float* partials, int nsplit,
                                           size_t split_stride, int ld, int kv_stride, hipStream_t stream);
 
-/* Benchmark switch: 1 (default) lets shapes with a specialised attention kernel (head_dim 128 with GQA ratio
- * 1/2/4/8, head_dim 64 with ratio 1/4) use it; 0 forces the general kernel. */
-int t12_tune_attention(int fast);
+/* Benchmark switch.  0: always the general attention kernel.  1 (default): shapes with a specialised kernel
+ * (head_dim 128 with GQA ratio 1/2/4/8, head_dim 64 with ratio 1/4) use it, and a launch without a position array
+ * whose batch * n_head_kv workgroups would leave the chip idle is split along the context into chunks of at
+ * least 256 positions (partial softmax per chunk, folded by the workgroup that finishes last; the partial results
+ * live in a library-owned buffer, so two such launches on different streams must not overlap).  2: specialised
+ * kernels, never split.  n >= 16: specialised kernels, chunks of at least n positions. */
+int t12_tune_attention(int mode);
 
 #ifdef __cplusplus
 }

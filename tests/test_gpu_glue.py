@@ -292,3 +292,49 @@ def test_per_sequence_caches_fused_and_from_partial_sums(t12, oracle, nh, nkv, h
         assert torch.equal(x[5], a[5]) and torch.equal(x[6], a[6])      # scales
     assert torch.equal(of, oa) and torch.equal(og, oa)
     assert not torch.equal(oa[0], oa[1])
+
+
+@pytest.mark.parametrize("nh,nkv,hd,B,pos", [(32, 8, 128, 1, 1290), (32, 8, 128, 2, 700), (16, 4, 64, 3, 333)])
+def test_context_split_equals_single_pass(t12, oracle, nh, nkv, hd, B, pos):
+    """A launch without a position array at a long context is split along the context (partial softmax per
+    chunk, folded by the workgroup that finishes last).  Same result as the single pass up to the order of the
+    fp32 sums, on repeated launches (the arrival counters reset themselves), for the fused and the plain launch."""
+    rng = np.random.default_rng(pos)
+    theta, max_seq = 500000.0, pos + 9
+    q, k, v = make_qkv(rng, B, nh, nkv, hd)
+    q[1:], k[1:], v[1:] = q[0], k[0], v[0]                     # lock-step copies on one cache region
+    kc = rng.integers(-127, 128, size=(max_seq, nkv, hd)).astype(np.int8)
+    vc = rng.integers(-127, 128, size=(max_seq, nkv, hd)).astype(np.int8)
+    ks = (rng.random((max_seq, nkv)).astype(np.float32) + 0.5) / 127
+    vs = (rng.random((max_seq, nkv)).astype(np.float32) + 0.5) / 127
+    sc = 1.0 / np.sqrt(hd)
+
+    def run(mode):
+        t12.lib.t12_tune_attention(mode)
+        f = [torch.from_numpy(a.copy()).to(dev()) for a in (q, k, v, kc, vc, ks, vs)]
+        of = torch.zeros((B, nh * hd), dtype=torch.int16, device=dev())
+        t12.lib.launch_rope_store_attention(f[0].data_ptr(), f[1].data_ptr(), f[2].data_ptr(), f[3].data_ptr(),
+                                            f[4].data_ptr(), f[5].data_ptr(), f[6].data_ptr(), of.data_ptr(), None, pos,
+                                            nh, nkv, hd, theta, sc, B, 0, st(t12))
+        torch.cuda.synchronize()
+        return f, of
+
+    try:
+        base, ob = run(2)                                       # never split
+        want = oracle.bf16_bits_to_f32(ob.cpu().numpy().view(np.uint16))
+        for mode in (1, 64, 1):                                 # default, many small chunks, default again
+            f, of = run(mode)
+            assert torch.equal(f[3], base[3]) and torch.equal(f[4], base[4])
+            assert torch.equal(f[5], base[5]) and torch.equal(f[6], base[6])
+            got = oracle.bf16_bits_to_f32(of.cpu().numpy().view(np.uint16))
+            assert np.abs(got - want).max() <= 2.0 ** -7 * np.abs(want).max(), mode     # a bf16 step at most
+            assert torch.equal(of[0], of[B - 1])
+        # against the CPU restatement, through the plain launcher (sequence 0)
+        # q in `base` was left unrotated by the fused launch: rotate on the CPU for the reference
+        qr = oracle.rope(q[0], pos, nh, hd, theta)
+        ref = oracle.attention_int8(qr, base[3].cpu().numpy(), base[4].cpu().numpy(), base[5].cpu().numpy(),
+                                    base[6].cpu().numpy(), pos + 1, nh, nkv, hd)
+        wantr = oracle.bf16_bits_to_f32(ref)
+        assert np.abs(want[0] - wantr).max() <= 2e-2 * np.abs(wantr).max()
+    finally:
+        t12.lib.t12_tune_attention(1)

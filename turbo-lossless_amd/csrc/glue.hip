@@ -13,6 +13,7 @@
 // All math is fp32; bf16 is produced with round-to-nearest-even exactly as
 // float_to_bf16 (kernels.hip:21-27).
 
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <mutex>
@@ -404,12 +405,24 @@ struct AttnFuse {
     const float* freqs;      // [HD / 2]
 };
 
-template <int HD, int RATIO, bool FUSE = false>
+// Context split (gridDim.z > 1): workgroup z attends over positions [z * chunk_len, (z + 1) * chunk_len) only and
+// leaves, per query head, its running maximum m, its sum l and its unnormalised 128 outputs in
+// ws[((b * n_head_kv + kvh) * nchunk + z) * RATIO + h][HD + 4] (m at [HD], l at [HD + 1]); the workgroup that finishes last for (b, kvh)
+// (counter[b * n_head_kv + kvh], which it resets to 0) folds the chunks: out = sum_z e^(m_z - M) acc_z /
+// sum_z e^(m_z - M) l_z.  One sequence at a long context otherwise occupies n_head_kv workgroups of the chip.
+struct AttnSplit {
+    float* ws;
+    int* counter;
+    int chunk_len;
+};
+
+template <int HD, int RATIO, bool FUSE = false, bool SPLIT = false>
 __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict__ q, const int8_t* __restrict__ ck,
                                                         const int8_t* __restrict__ cv, const float* __restrict__ sk,
                                                         const float* __restrict__ sv, uint16_t* __restrict__ out,
                                                         const int* __restrict__ positions, int seq_len_arg,
-                                                        int n_head_kv, float scale, size_t kv_stride, AttnFuse fz)
+                                                        int n_head_kv, float scale, size_t kv_stride, AttnFuse fz,
+                                                        AttnSplit sp)
 {
     constexpr int CH = HD / 16;                 // lanes per position in phase 3
     constexpr int PG = 64 / CH;                 // positions per load instruction
@@ -427,6 +440,10 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
     const float* skb = sk + (size_t)b * sstride + kvh;
     const float* svb = sv + (size_t)b * sstride + kvh;
     const float* qb = q + (size_t)b * n_head * HD + (size_t)kvh * RATIO * HD;
+    // this workgroup's share of the context
+    const int nchunk = SPLIT ? gridDim.z : 1;
+    const int c0 = SPLIT ? (int)blockIdx.z * sp.chunk_len : 0;
+    const int c1 = SPLIT ? min(seq_len, c0 + sp.chunk_len) : seq_len;
 
     // FUSE: the cache rows of the first tile are requested before anything else, so that their HBM
     // latency runs under the Q / new-K / new-V work instead of behind it: this lane's K row (phase 1)
@@ -436,16 +453,17 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
     __shared__ float vts[FUSE ? ATT_TILE : 1];
     __shared__ __attribute__((aligned(16))) int8_t knew8[FUSE ? HD : 16];
     __shared__ float knew_scale;
-    const int tl0 = min(ATT_TILE, seq_len);
+    const int tl0 = min(ATT_TILE, c1 - c0);
     const int newpos = FUSE ? seq_len - 1 : -1;
-    const bool kpre = FUSE && tid < tl0 && tid != newpos;    // (many small workgroups per CU without FUSE: the registers cost more than the latency)
+    const bool store_new = FUSE && c1 == seq_len;         // the chunk that holds the position being written
+    const bool kpre = FUSE && tid < tl0 && c0 + tid != newpos;    // (many small workgroups per CU without FUSE: the registers cost more than the latency)
     uint4 kk_pre[CH];
     float kscale_pre = 0.0f;
     if (kpre) {
-        const uint4* kr = (const uint4*)(kbase + (size_t)tid * kv_dim);
+        const uint4* kr = (const uint4*)(kbase + (size_t)(c0 + tid) * kv_dim);
 #pragma unroll
         for (int u = 0; u < CH; u++) kk_pre[u] = kr[u];
-        kscale_pre = skb[(size_t)tid * n_head_kv] * scale;
+        kscale_pre = skb[(size_t)(c0 + tid) * n_head_kv] * scale;
     }
     uint4 v_pre[VPRE > 0 ? VPRE : 1];
     float vs_pre = 0.0f;
@@ -454,9 +472,9 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
         for (int x = 0; x < VPRE; x++) {
             const int idx = tid + 256 * x, t = idx / CH, u = idx % CH;
             v_pre[x] = make_uint4(0, 0, 0, 0);
-            if (t < tl0 && t != newpos) v_pre[x] = *(const uint4*)(vbase + (size_t)t * kv_dim + u * 16);
+            if (t < tl0 && c0 + t != newpos) v_pre[x] = *(const uint4*)(vbase + (size_t)(c0 + t) * kv_dim + u * 16);
         }
-        if (tid < tl0 && tid != newpos) vs_pre = svb[(size_t)tid * n_head_kv];
+        if (tid < tl0 && c0 + tid != newpos) vs_pre = svb[(size_t)(c0 + tid) * n_head_kv];
     }
 
     if (!FUSE) {
@@ -471,7 +489,7 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
             const float x0 = qb[h * HD + d], x1 = qb[h * HD + d + HALF];
             rope_rotate(x0, x1, sn, cs, qs[h * HD + d], qs[h * HD + d + HALF]);
         }
-        if (wave < 2) {                                              // wave 0: K (rotated), wave 1: V
+        if (wave < 2 && store_new) {                                 // wave 0: K (rotated), wave 1: V
             const bool own = lane < HALF;
             const float* src = (wave == 0 ? fz.k_new : fz.v_new) + (size_t)b * kv_dim + (size_t)kvh * HD;
             float r0 = 0.0f, r1 = 0.0f;
@@ -491,8 +509,9 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
             const int8_t q0 = (int8_t)(int)fminf(fmaxf(rintf(r0 * inv), -127.0f), 127.0f);
             const int8_t q1 = (int8_t)(int)fminf(fmaxf(rintf(r1 * inv), -127.0f), 127.0f);
             // the new row: to the cache, and (first tile) to LDS where this launch reads it
-            int8_t* lrow = wave == 0 ? knew8 : vt + (size_t)(pos < ATT_TILE ? pos : 0) * HD;
-            const bool to_lds = wave == 0 || pos < ATT_TILE;
+            const int rel = pos - c0;                                // position inside this chunk
+            int8_t* lrow = wave == 0 ? knew8 : vt + (size_t)(rel < ATT_TILE ? rel : 0) * HD;
+            const bool to_lds = wave == 0 || rel < ATT_TILE;
             if (own) {
                 row[lane] = q0;
                 row[lane + HALF] = q1;
@@ -504,7 +523,7 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
             if (lane == 0) {
                 (wave == 0 ? fz.sk_w : fz.sv_w)[(size_t)b * sstride + (size_t)pos * n_head_kv + kvh] = amax / 127.0f;
                 if (wave == 0) knew_scale = amax / 127.0f;
-                else if (pos < ATT_TILE) vts[pos] = amax / 127.0f;
+                else if (rel < ATT_TILE) vts[rel] = amax / 127.0f;
             }
         }
         __threadfence();      // later tiles read the new row back through the cache pointers
@@ -512,9 +531,9 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
 #pragma unroll
         for (int x = 0; x < VPRE; x++) {
             const int idx = tid + 256 * x, t = idx / CH;
-            if (t < tl0 && t != newpos) ((uint4*)vt)[idx] = v_pre[x];
+            if (t < tl0 && c0 + t != newpos) ((uint4*)vt)[idx] = v_pre[x];
         }
-        if (tid < tl0 && tid != newpos) vts[tid] = vs_pre;
+        if (tid < tl0 && c0 + tid != newpos) vts[tid] = vs_pre;
     }
     __syncthreads();
 
@@ -528,18 +547,18 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
     }
     const int g = lane / CH, c = lane % CH;     // phase 3: position class, 16-dim chunk
 
-    for (int t0 = 0; t0 < seq_len; t0 += ATT_TILE) {
-        const int tl = min(ATT_TILE, seq_len - t0);
+    for (int t0 = c0; t0 < c1; t0 += ATT_TILE) {
+        const int tl = min(ATT_TILE, c1 - t0);
         // ---- phase 1
         if (tid < tl) {
             const int t = t0 + tid;
             uint4 kk[CH];
             float kscale;
-            if (t0 == 0 && kpre) {
+            if (t0 == c0 && kpre) {
 #pragma unroll
                 for (int u = 0; u < CH; u++) kk[u] = kk_pre[u];
                 kscale = kscale_pre;
-            } else if (FUSE && t == newpos && t0 == 0) {
+            } else if (FUSE && t == newpos && t0 == c0) {
 #pragma unroll
                 for (int u = 0; u < CH; u++) kk[u] = ((const uint4*)knew8)[u];
                 kscale = knew_scale * scale;
@@ -605,7 +624,7 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
                         const int t = (it + x) * PG + g;
                         const bool ok = t < tl;
                         const int tc = ok ? t : 0;
-                        if (FUSE && t0 == 0) {
+                        if (FUSE && t0 == c0) {
                             vv[x] = ((const uint4*)vt)[tc * CH + c];
                             w[x] = ok ? ph[tc] * vts[tc] : 0.0f;
                         } else {
@@ -637,15 +656,75 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
                 acc[j][e] = v;
             }
             if (g == 0) {
-                const float inv = 1.0f / l_run[j];
-                uint32_t o[8];
+                if (SPLIT) {
+                    float* pw = sp.ws + ((((size_t)b * n_head_kv + kvh) * nchunk + blockIdx.z) * RATIO + h) * (HD + 4);
 #pragma unroll
-                for (int e = 0; e < 8; e++)
-                    o[e] = t12_f32_to_bf16(acc[j][2 * e] * inv) | ((uint32_t)t12_f32_to_bf16(acc[j][2 * e + 1] * inv) << 16);
-                uint4* dst = (uint4*)(out + (size_t)b * n_head * HD + (size_t)(kvh * RATIO + h) * HD + c * 16);
-                dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
-                dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
+                    for (int e = 0; e < 16; e += 4)
+                        *(float4*)(pw + c * 16 + e) = make_float4(acc[j][e], acc[j][e + 1], acc[j][e + 2], acc[j][e + 3]);
+                    if (c == 0) {
+                        pw[HD] = m_run[j];
+                        pw[HD + 1] = l_run[j];
+                    }
+                } else {
+                    const float inv = 1.0f / l_run[j];
+                    uint32_t o[8];
+#pragma unroll
+                    for (int e = 0; e < 8; e++)
+                        o[e] = t12_f32_to_bf16(acc[j][2 * e] * inv) | ((uint32_t)t12_f32_to_bf16(acc[j][2 * e + 1] * inv) << 16);
+                    uint4* dst = (uint4*)(out + (size_t)b * n_head * HD + (size_t)(kvh * RATIO + h) * HD + c * 16);
+                    dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
+                    dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
+                }
             }
+        }
+    }
+    if (SPLIT) {
+        // the workgroup that arrives last for this (sequence, KV head) folds the chunks
+        __shared__ int s_last;
+        __threadfence();
+        __syncthreads();
+        if (tid == 0) s_last = atomicAdd(sp.counter + (size_t)b * n_head_kv + kvh, 1) == nchunk - 1;
+        __syncthreads();
+        if (s_last) {
+            __threadfence();
+            const float* pb = sp.ws + (((size_t)b * n_head_kv + kvh) * nchunk) * RATIO * (HD + 4);
+            // weight of chunk z for head h: e^(m_z - M) / sum_z e^(m_z - M) l_z, built in ps (free by now)
+            float* wz = ps;                                          // [RATIO][nchunk] maxima, then weights
+            float* lz = ps + RATIO * nchunk;                         // [RATIO][nchunk] sums (2 * nchunk <= ATT_TILE)
+            for (int i = tid; i < RATIO * nchunk; i += 256) {
+                const int h = i / nchunk, z = i % nchunk;
+                const float2 ml = *(const float2*)(pb + ((size_t)z * RATIO + h) * (HD + 4) + HD);
+                wz[i] = ml.x;
+                lz[i] = ml.y;
+            }
+            __syncthreads();
+            if (tid < RATIO) {
+                float mx = -1e30f;
+                for (int z = 0; z < nchunk; z++) mx = fmaxf(mx, wz[tid * nchunk + z]);
+                float den = 0.0f;
+                for (int z = 0; z < nchunk; z++) {
+                    const float w = expf(wz[tid * nchunk + z] - mx);
+                    den += w * lz[tid * nchunk + z];
+                    wz[tid * nchunk + z] = w;
+                }
+                const float inv = 1.0f / den;
+                for (int z = 0; z < nchunk; z++) wz[tid * nchunk + z] *= inv;
+            }
+            __syncthreads();
+            for (int i = tid; i < RATIO * HD / 4; i += 256) {         // four neighbouring outputs per thread
+                const int h = i / (HD / 4), d = (i % (HD / 4)) * 4;
+                float4 n = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll 8
+                for (int z = 0; z < nchunk; z++) {
+                    const float4 a = *(const float4*)(pb + ((size_t)z * RATIO + h) * (HD + 4) + d);
+                    const float w = wz[h * nchunk + z];
+                    n.x += w * a.x; n.y += w * a.y; n.z += w * a.z; n.w += w * a.w;
+                }
+                *(uint2*)(out + (size_t)b * n_head * HD + (size_t)(kvh * RATIO + h) * HD + d) =
+                    make_uint2(t12_f32_to_bf16(n.x) | ((uint32_t)t12_f32_to_bf16(n.y) << 16),
+                               t12_f32_to_bf16(n.z) | ((uint32_t)t12_f32_to_bf16(n.w) << 16));
+            }
+            if (tid == 0) sp.counter[(size_t)b * n_head_kv + kvh] = 0;
         }
     }
 }
@@ -782,6 +861,29 @@ void launch_rope_kv(float* q, float* k, const float* v, int8_t* ck, int8_t* cv, 
 }
 
 int g_attn_fast = 1;   // 0: always the general kernel (tests compare the two)
+int g_attn_chunk = 256; // context split: fewest positions per chunk; 0 = never split
+
+// Scratch of the context split: partial results of at most ATT_SPLIT_WGS workgroups and one
+// counter per (sequence, KV head); the counters start at zero and every launch leaves them there.
+constexpr int ATT_SPLIT_WGS = 512;     // also: at most ATT_TILE / 2 chunks per (sequence, KV head)
+constexpr int ATT_SPLIT_HEADS = 4096;
+float* g_split_ws = nullptr;
+int* g_split_cnt = nullptr;
+
+bool attn_split_scratch()
+{
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (g_split_ws) return true;
+    const size_t ws_bytes = (size_t)ATT_SPLIT_WGS * 8 * (128 + 4) * sizeof(float);     // RATIO <= 8, HD <= 128
+    if (hipMalloc((void**)&g_split_ws, ws_bytes) != hipSuccess) { g_split_ws = nullptr; return false; }
+    if (hipMalloc((void**)&g_split_cnt, ATT_SPLIT_HEADS * sizeof(int)) != hipSuccess ||
+        hipMemset(g_split_cnt, 0, ATT_SPLIT_HEADS * sizeof(int)) != hipSuccess) {
+        (void)hipFree(g_split_ws);
+        g_split_ws = nullptr;
+        return false;
+    }
+    return true;
+}
 
 bool attn_has_fast(int n_head, int n_head_kv, int head_dim)
 {
@@ -802,14 +904,36 @@ void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float
         fprintf(stderr, "turbo12: %s\n", t12_last_error());
         return;
     }
+    // Context split: only when the host knows the length (no per-sequence position array) and the launch
+    // would otherwise leave most of the chip idle.
+    int nchunk = 1;
+    AttnSplit sp = {nullptr, nullptr, 0};
+    if (g_attn_fast && g_attn_chunk > 0 && !positions && batch * n_head_kv <= ATT_SPLIT_HEADS) {
+        const int room = ATT_SPLIT_WGS / (batch * n_head_kv);
+        int want = std::min(std::min(room, ATT_TILE / 2), (seq_len + g_attn_chunk - 1) / g_attn_chunk);
+        if (want > 1 && attn_split_scratch()) {
+            sp.chunk_len = (((seq_len + want - 1) / want) + 63) & ~63;
+            nchunk = (seq_len + sp.chunk_len - 1) / sp.chunk_len;
+            sp.ws = g_split_ws;
+            sp.counter = g_split_cnt;
+        }
+    }
 #define T12_ATT_FAST(HD_, R_)                                                                                   \
     if (head_dim == HD_ && ratio == R_) {                                                                       \
-        if (fuse)                                                                                               \
-            hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, true>), dim3(n_head_kv, batch), dim3(256), 0, st, q, ck, cv, \
-                               sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride, *fuse);  \
+        if (fuse && nchunk > 1)                                                                                 \
+            hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, true, true>), dim3(n_head_kv, batch, nchunk), dim3(256), 0, st, q, \
+                               ck, cv, sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride, *fuse, sp); \
+        else if (fuse)                                                                                          \
+            hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, true, false>), dim3(n_head_kv, batch), dim3(256), 0, st, q, \
+                               ck, cv, sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride, *fuse, sp); \
+        else if (nchunk > 1)                                                                                    \
+            hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, false, true>), dim3(n_head_kv, batch, nchunk), dim3(256), 0, st, q, \
+                               ck, cv, sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride,  \
+                               AttnFuse(), sp);                                                                 \
         else                                                                                                    \
-            hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, false>), dim3(n_head_kv, batch), dim3(256), 0, st, q, ck, cv, \
-                               sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride, AttnFuse()); \
+            hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, false, false>), dim3(n_head_kv, batch), dim3(256), 0, st, q, \
+                               ck, cv, sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride,  \
+                               AttnFuse(), sp);                                                                 \
         report("attention");                                                                                    \
         return;                                                                                                 \
     }
@@ -869,10 +993,13 @@ void launch_rope_scaling(float factor, float low_freq_factor, float high_freq_fa
     g_rope_scale[3] = original_ctx;
 }
 
-// 1 (default): shapes with a specialised attention kernel use it; 0: always the general kernel.
-int t12_tune_attention(int fast)
+// 0: always the general kernel; 1 (default): shapes with a specialised kernel use it, one sequence at a long
+// context split into chunks of at least 256 positions; 2: specialised kernels, never split; n >= 16: specialised
+// kernels, chunks of at least n positions.
+int t12_tune_attention(int mode)
 {
-    g_attn_fast = fast;
+    g_attn_fast = mode != 0;
+    g_attn_chunk = mode >= 16 ? mode : (mode == 2 ? 0 : 256);
     return 0;
 }
 
