@@ -126,8 +126,10 @@ void launch_rope_store_attention_partials(float* q, float* k, const float* v, in
  * (head_dim 128 with GQA ratio 1/2/4/8, head_dim 64 with ratio 1/4) use it, and a launch without a position array
  * whose batch * n_head_kv workgroups would leave the chip idle is split along the context into chunks of at
  * least 256 positions (partial softmax per chunk, folded by the workgroup that finishes last; the partial results
- * live in a library-owned buffer, so two such launches on different streams must not overlap).  2: specialised
- * kernels, never split.  n >= 16: specialised kernels, chunks of at least n positions. */
+ * live in a library-owned buffer, so two such launches on different streams must not overlap); from 320
+ * positions on (the length argument, a hint when a position array is given) the kernel takes its long-context
+ * form: scores by INT8 MFMAs, P.V with one wave per 64 positions.  2: specialised kernels, never split.  3: never the long-context form.  4: always.  n >= 16:
+ * specialised kernels, chunks of at least n positions. */
 int t12_tune_attention(int mode);
 
 #ifdef __cplusplus

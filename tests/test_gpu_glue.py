@@ -130,7 +130,7 @@ def test_rope_and_store_batch_launchers(t12, oracle):
     assert torch.equal(ck, ck2) and torch.equal(cv, cv2) and torch.equal(sk, sk2) and torch.equal(q2, qd)
 
 
-@pytest.fixture(params=[1, 0], ids=["fast", "general"])
+@pytest.fixture(params=[1, 3, 4, 0], ids=["fast", "fast-wave-per-head", "fast-wave-per-64-positions", "general"])
 def attn_mode(request, t12):
     t12.lib.t12_tune_attention(request.param)
     yield request.param
@@ -204,7 +204,7 @@ def test_argmax(t12, oracle):
 
 
 @pytest.mark.parametrize("nh,nkv,hd,B", [(32, 8, 128, 1), (32, 8, 128, 5), (4, 4, 64, 2), (8, 2, 32, 3)])
-def test_fused_rope_store_attention_equals_separate_launches(t12, oracle, nh, nkv, hd, B):
+def test_fused_rope_store_attention_equals_separate_launches(t12, oracle, attn_mode, nh, nkv, hd, B):
     """launch_rope_store_attention == launch_rope_store_kv_batch + launch_attention_all_heads_batch:
     same caches, same scales, same bf16 output (the fused kernel leaves q unrotated)."""
     rng = np.random.default_rng(B)
@@ -240,7 +240,7 @@ def test_fused_rope_store_attention_equals_separate_launches(t12, oracle, nh, nk
 
 
 @pytest.mark.parametrize("nh,nkv,hd", [(32, 8, 128), (8, 2, 32), (4, 4, 64)])
-def test_per_sequence_caches_fused_and_from_partial_sums(t12, oracle, nh, nkv, hd):
+def test_per_sequence_caches_fused_and_from_partial_sums(t12, oracle, attn_mode, nh, nkv, hd):
     """Independent sequences, each with its own cache region (kv_stride != 0) and its own position: the fused
     launch and the launch that first adds up K-split partial sums of q | k | v both equal one separate
     RoPE/store + attention launch per sequence on that sequence's region."""

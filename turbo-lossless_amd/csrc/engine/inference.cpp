@@ -357,7 +357,8 @@ KvView kv_view(const InferenceState* state)
 }
 
 // One pass of the layer stack over R rows (R <= batch_size) whose token ids are in state->d_tokens and, for
-// R > 1, whose positions are in state->d_positions; pos0 = position of row 0.  Logits: for every row into
+// R > 1, whose positions are in state->d_positions; pos0 = position of the row when R == 1, else the largest
+// position of the rows (a length hint for the attention launch).  Logits: for every row into
 // state->logits (LOGITS_ALL), for the last row only into logits_last (LOGITS_LAST_ROW), or not at all.
 void forward_rows(InferenceState* state, int R, const KvView& kv, int pos0, LogitsMode lm, float* logits_last)
 {
@@ -491,7 +492,8 @@ void forward(InferenceState* state, const int* token_ids)
     }
     if (token_ids) (void)hipMemcpyAsync(state->d_tokens, token_ids, B * sizeof(int), hipMemcpyHostToDevice, st);
     if (B > 1) (void)hipMemcpyAsync(state->d_positions, state->positions, B * sizeof(int), hipMemcpyHostToDevice, st);
-    forward_rows(state, B, kv, state->positions[0], LOGITS_ALL, nullptr);
+    // with a position array the scalar position is only the attention launch's length hint: the longest row
+    forward_rows(state, B, kv, B > 1 ? max_pos : state->positions[0], LOGITS_ALL, nullptr);
     for (int b = 0; b < B; b++) state->positions[b]++;
 }
 
@@ -539,7 +541,7 @@ void prefill(InferenceState* state, int seq, const int* token_ids, int n_tokens)
         for (int r = 0; r < R; r++) pos[r] = p0 + done + r;
         (void)hipMemcpyAsync(state->d_tokens, token_ids + done, R * sizeof(int), hipMemcpyHostToDevice, st);
         (void)hipMemcpyAsync(state->d_positions, pos.data(), R * sizeof(int), hipMemcpyHostToDevice, st);
-        forward_rows(state, R, kv, p0 + done, last ? LOGITS_LAST_ROW : LOGITS_NONE, row_logits);
+        forward_rows(state, R, kv, p0 + done + (R > 1 ? R - 1 : 0), last ? LOGITS_LAST_ROW : LOGITS_NONE, row_logits);
         // pos[] is reused by the next chunk: the copies above read it when they are issued (pageable memory)
         done += R;
     }

@@ -416,8 +416,8 @@ struct AttnSplit {
     int chunk_len;
 };
 
-template <int HD, int RATIO, bool FUSE = false, bool SPLIT = false>
-__global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict__ q, const int8_t* __restrict__ ck,
+template <int HD, int RATIO, bool FUSE = false, bool SPLIT = false, bool WIDE = false>
+__global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kernel(const float* __restrict__ q, const int8_t* __restrict__ ck,
                                                         const int8_t* __restrict__ cv, const float* __restrict__ sk,
                                                         const float* __restrict__ sv, uint16_t* __restrict__ out,
                                                         const int* __restrict__ positions, int seq_len_arg,
@@ -456,14 +456,39 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
     const int tl0 = min(ATT_TILE, c1 - c0);
     const int newpos = FUSE ? seq_len - 1 : -1;
     const bool store_new = FUSE && c1 == seq_len;         // the chunk that holds the position being written
-    const bool kpre = FUSE && tid < tl0 && c0 + tid != newpos;    // (many small workgroups per CU without FUSE: the registers cost more than the latency)
-    uint4 kk_pre[CH];
-    float kscale_pre = 0.0f;
-    if (kpre) {
+    // one-wave-per-head form: thread = position, the whole K row in registers
+    const bool kpre_n = !WIDE && FUSE && tid < tl0 && c0 + tid != newpos;    // (many small workgroups per CU without FUSE: the registers cost more than the latency)
+    uint4 kk_pre_n[CH];
+    float kscale_pre_n = 0.0f;
+    if (kpre_n) {
         const uint4* kr = (const uint4*)(kbase + (size_t)(c0 + tid) * kv_dim);
 #pragma unroll
-        for (int u = 0; u < CH; u++) kk_pre[u] = kr[u];
-        kscale_pre = skb[(size_t)(c0 + tid) * n_head_kv] * scale;
+        for (int u = 0; u < CH; u++) kk_pre_n[u] = kr[u];
+        kscale_pre_n = skb[(size_t)(c0 + tid) * n_head_kv] * scale;
+    }
+    // Phase 1 layout: wave w scores positions 64 w .. 64 w + 63 of a tile in two blocks of 32; lane (ln, lh) of
+    // block nb holds half lh of the K row of position 64 w + 32 nb + ln: HD / 2 contiguous bytes = KS pieces
+    // of 16, the B operand of KS v_mfma_i32_32x32x32_i8 steps (the dims are consumed in this permuted order on
+    // both operands).
+    constexpr int KS = HD / 32;
+    const int ln = lane & 31, lh = lane >> 5;
+    typedef int t12_i32x4 __attribute__((ext_vector_type(4)));
+    typedef int t12_i32x16 __attribute__((ext_vector_type(16)));
+    uint4 kk_pre[2][KS];
+    float kscale_pre[2] = {0.0f, 0.0f};
+    bool kpre[2] = {false, false};
+    if (FUSE && WIDE) {
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) {
+            const int tp = wave * 64 + nb * 32 + ln;             // position inside the first tile
+            kpre[nb] = tp < tl0 && c0 + tp != newpos;
+            if (kpre[nb]) {
+                const uint4* kr = (const uint4*)(kbase + (size_t)(c0 + tp) * kv_dim + lh * (HD / 2));
+#pragma unroll
+                for (int u = 0; u < KS; u++) kk_pre[nb][u] = kr[u];
+                kscale_pre[nb] = skb[(size_t)(c0 + tp) * n_head_kv] * scale;
+            }
+        }
     }
     uint4 v_pre[VPRE > 0 ? VPRE : 1];
     float vs_pre = 0.0f;
@@ -537,27 +562,103 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
     }
     __syncthreads();
 
-    float m_run[OWN], l_run[OWN], acc[OWN][16];
+    // Q as two INT8 limbs per element, q ~ s_h (a1 + a2 / 254) with s_h = max|q_h| / 127 (error <= 1.6e-5 max|q_h|,
+    // below what the bf16 output resolves), laid out as the A operand of the score MFMAs: row 8 * limb + h.
+    // INT8 x INT8 products accumulate exactly in int32, so K needs no conversion at all.
+    __shared__ __attribute__((aligned(16))) int8_t qlimb[WIDE ? 32 * HD : 16];
+    __shared__ float qscale[RATIO];
+    if constexpr (WIDE) {
+    for (int i = tid; i < 32 * HD / 16; i += 256) ((uint4*)qlimb)[i] = make_uint4(0, 0, 0, 0);
+    __syncthreads();
+    for (int h = wave; h < RATIO; h += 4) {
+        float amax = 0.0f;
+        for (int d = lane; d < HD; d += 64) amax = fmaxf(amax, fabsf(qs[h * HD + d]));
+        amax = wave_max(amax);
+        const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+        for (int d = lane; d < HD; d += 64) {
+            const float r0 = qs[h * HD + d] * inv;
+            const float a1 = fminf(fmaxf(rintf(r0), -127.0f), 127.0f);
+            const float a2 = fminf(fmaxf(rintf((r0 - a1) * 254.0f), -127.0f), 127.0f);
+            qlimb[h * HD + d] = (int8_t)(int)a1;
+            qlimb[(8 + h) * HD + d] = (int8_t)(int)a2;
+        }
+        if (lane == 0) qscale[h] = amax / 127.0f;
+    }
+    __syncthreads();
+    }
+    const int8_t* qa_src = qlimb + ln * HD + lh * (HD / 2);      // this lane's A operand pieces (re-read per tile: 4 LDS loads)
+
+    // running maximum / sum of head h live in the wave that owns it (h % 4); the output sums of ALL heads live
+    // in every wave, over the 64 positions of each tile that the wave takes in phase 3
+    constexpr int NACC = WIDE ? RATIO : OWN;
+    float m_run[OWN], l_run[OWN], acc[NACC][16];
 #pragma unroll
     for (int j = 0; j < OWN; j++) {
         m_run[j] = -1e30f;
         l_run[j] = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 16; e++) acc[j][e] = 0.0f;
     }
+#pragma unroll
+    for (int h = 0; h < NACC; h++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[h][e] = 0.0f;
+    __shared__ float corr_s[RATIO];
+    constexpr int NIT = 64 / PG;                // phase 3 iterations per wave and tile
     const int g = lane / CH, c = lane % CH;     // phase 3: position class, 16-dim chunk
 
     for (int t0 = c0; t0 < c1; t0 += ATT_TILE) {
         const int tl = min(ATT_TILE, c1 - t0);
+        if constexpr (WIDE) {
+        // ---- phase 1: scores of 64 positions per wave, two blocks of 32, KS INT8 MFMAs each
+        t12_i32x4 qa[KS];
+#pragma unroll
+        for (int u = 0; u < KS; u++) qa[u] = *(const t12_i32x4*)(qa_src + 16 * u);
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) {
+            const int tp = wave * 64 + nb * 32 + ln;                 // position inside the tile
+            if (wave * 64 + nb * 32 < tl) {                          // wave-uniform: the block holds positions
+                const int t = t0 + min(tp, tl - 1);                  // rows past the end repeat the last one (masked in phase 2)
+                uint4 kk[KS];
+                float kscale;
+                if (t0 == c0 && kpre[nb]) {
+#pragma unroll
+                    for (int u = 0; u < KS; u++) kk[u] = kk_pre[nb][u];
+                    kscale = kscale_pre[nb];
+                } else if (FUSE && t == newpos && t0 == c0) {
+#pragma unroll
+                    for (int u = 0; u < KS; u++) kk[u] = ((const uint4*)(knew8 + lh * (HD / 2)))[u];
+                    kscale = knew_scale * scale;
+                } else {
+                    const uint4* kr = (const uint4*)(kbase + (size_t)t * kv_dim + lh * (HD / 2));
+#pragma unroll
+                    for (int u = 0; u < KS; u++) kk[u] = kr[u];
+                    kscale = skb[(size_t)t * n_head_kv] * scale;
+                }
+                t12_i32x16 sacc;
+#pragma unroll
+                for (int r = 0; r < 16; r++) sacc[r] = 0;
+#pragma unroll
+                for (int u = 0; u < KS; u++)
+                    sacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[u], __builtin_bit_cast(t12_i32x4, kk[u]), sacc, 0, 0, 0);
+                // lane (ln, lh) holds column ln = its position; rows 4 lh + r (limb 0) and 8 + 4 lh + r (limb 1),
+                // r = 0..3: heads 4 lh .. 4 lh + 3
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int h = 4 * lh + r;
+                    if (h < RATIO)
+                        ps[h * ATT_TILE + tp] = ((float)sacc[r] + (float)sacc[4 + r] * (1.0f / 254.0f)) * (qscale[h] * kscale);
+                }
+            }
+        }
+        } else {
         // ---- phase 1
         if (tid < tl) {
             const int t = t0 + tid;
             uint4 kk[CH];
             float kscale;
-            if (t0 == c0 && kpre) {
+            if (t0 == c0 && kpre_n) {
 #pragma unroll
-                for (int u = 0; u < CH; u++) kk[u] = kk_pre[u];
-                kscale = kscale_pre;
+                for (int u = 0; u < CH; u++) kk[u] = kk_pre_n[u];
+                kscale = kscale_pre_n;
             } else if (FUSE && t == newpos && t0 == c0) {
 #pragma unroll
                 for (int u = 0; u < CH; u++) kk[u] = ((const uint4*)knew8)[u];
@@ -584,96 +685,238 @@ __global__ __launch_bounds__(256) void attn_fast_kernel(const float* __restrict_
 #pragma unroll
             for (int h = 0; h < RATIO; h++) ps[h * ATT_TILE + tid] = dot[h] * kscale;
         }
-        __syncthreads();
-        // ---- phases 2 + 3, one wave per head
-#pragma unroll
-        for (int j = 0; j < OWN; j++) {
-            const int h = wave + 4 * j;
-            if (h < RATIO) {                                     // wave-uniform
-                float* ph = ps + h * ATT_TILE;
-                float sc[ATT_TILE / 64];
-                float tmax = -1e30f;
-#pragma unroll
-                for (int i = 0; i < ATT_TILE / 64; i++) {
-                    const int t = lane + 64 * i;
-                    sc[i] = t < tl ? ph[t] : -1e30f;
-                    tmax = fmaxf(tmax, sc[i]);
+        }
+        if constexpr (WIDE) {
+            // ---- V rows of this wave's 64 positions: requested now, consumed after the softmax bookkeeping
+            const bool v_lds = FUSE && t0 == c0;                         // first tile of the fused launch: V tile is in LDS
+            const bool v_any = wave * 64 < tl;                           // wave-uniform
+            uint4 vv[NIT];
+            float vsc[NIT];
+            if (v_any && !v_lds) {
+    #pragma unroll
+                for (int x = 0; x < NIT; x++) {
+                    const int tp = wave * 64 + x * PG + g;
+                    const int tc = min(tp, tl - 1);
+                    vv[x] = *(const uint4*)(vbase + (size_t)(t0 + tc) * kv_dim + c * 16);
+                    vsc[x] = svb[(size_t)(t0 + tc) * n_head_kv];
                 }
-                tmax = wave_max(tmax);
-                const float m_new = fmaxf(m_run[j], tmax);
-                const float corr = expf(m_run[j] - m_new);
-                float psum = 0.0f;
-#pragma unroll
-                for (int i = 0; i < ATT_TILE / 64; i++) {
-                    const int t = lane + 64 * i;
-                    const float pv = t < tl ? expf(sc[i] - m_new) : 0.0f;
-                    if (t < tl) ph[t] = pv;
-                    psum += pv;
+            }
+            __syncthreads();
+            // ---- phase 2, one wave per head: tile maximum, rescale factor, probabilities, sum
+    #pragma unroll
+            for (int j = 0; j < OWN; j++) {
+                const int h = wave + 4 * j;
+                if (h < RATIO) {                                     // wave-uniform
+                    float* ph = ps + h * ATT_TILE;
+                    float sc[ATT_TILE / 64];
+                    float tmax = -1e30f;
+    #pragma unroll
+                    for (int i = 0; i < ATT_TILE / 64; i++) {
+                        const int t = lane + 64 * i;
+                        sc[i] = t < tl ? ph[t] : -1e30f;
+                        tmax = fmaxf(tmax, sc[i]);
+                    }
+                    tmax = wave_max(tmax);
+                    const float m_new = fmaxf(m_run[j], tmax);
+                    const float corr = expf(m_run[j] - m_new);
+                    float psum = 0.0f;
+    #pragma unroll
+                    for (int i = 0; i < ATT_TILE / 64; i++) {
+                        const int t = lane + 64 * i;
+                        const float pv = t < tl ? expf(sc[i] - m_new) : 0.0f;
+                        if (t < tl) ph[t] = pv;
+                        psum += pv;
+                    }
+                    psum = t12_wave_sum(psum);
+                    l_run[j] = l_run[j] * corr + psum;
+                    m_run[j] = m_new;
+                    if (lane == 0) corr_s[h] = corr;
                 }
-                psum = t12_wave_sum(psum);
-                l_run[j] = l_run[j] * corr + psum;
-                m_run[j] = m_new;
-#pragma unroll
-                for (int e = 0; e < 16; e++) acc[j][e] *= corr;
-                // P.V: iteration it covers positions it*PG + g; loads of 4 iterations are issued together
-                for (int it = 0; it * PG < tl; it += 4) {
-                    uint4 vv[4];
-                    float w[4];
-#pragma unroll
-                    for (int x = 0; x < 4; x++) {
-                        const int t = (it + x) * PG + g;
-                        const bool ok = t < tl;
-                        const int tc = ok ? t : 0;
-                        if (FUSE && t0 == c0) {
-                            vv[x] = ((const uint4*)vt)[tc * CH + c];
-                            w[x] = ok ? ph[tc] * vts[tc] : 0.0f;
-                        } else {
-                            vv[x] = *(const uint4*)(vbase + (size_t)(t0 + tc) * kv_dim + c * 16);
-                            w[x] = ok ? ph[tc] * svb[(size_t)(t0 + tc) * n_head_kv] : 0.0f;
+            }
+            __syncthreads();
+            // ---- phase 3, one wave per 64 positions: every V value is converted once and used for all heads
+            int tl_opaque = tl;
+            asm volatile("" : "+s"(tl_opaque));
+    #pragma unroll
+            for (int h = 0; h < RATIO; h++) {
+                const float corr = corr_s[h];
+    #pragma unroll
+                for (int e = 0; e < 16; e++) acc[h][e] *= corr;
+            }
+            if (v_any) {
+    #pragma unroll
+                for (int x = 0; x < NIT; x++) {
+                    // every row is a basic block of its own (the condition always holds, but only at run time):
+                    // the compiler schedules inside basic blocks, and left to itself it converts all prefetched
+                    // rows first and keeps 16 floats per row alive (> 300 VGPRs)
+                    if (tl_opaque < 0) continue;
+                    const int tp = wave * 64 + x * PG + g;
+                    const bool ok = tp < tl;
+                    const int tc = min(tp, tl - 1);
+                    uint4 v4 = vv[x];
+                    float vscale = vsc[x];
+                    if (v_lds) {
+                        v4 = ((const uint4*)vt)[tc * CH + c];
+                        vscale = vts[tc];
+                    }
+                    const uint32_t w4[4] = {v4.x, v4.y, v4.z, v4.w};
+                    float fv[16];
+    #pragma unroll
+                    for (int e = 0; e < 16; e++) fv[e] = (float)(int8_t)((w4[e >> 2] >> (8 * (e & 3))) & 0xFF);
+    #pragma unroll
+                    for (int h = 0; h < RATIO; h++) {
+                        const float w = ok ? ps[h * ATT_TILE + tc] * vscale : 0.0f;
+    #pragma unroll
+                        for (int e = 0; e < 16; e++) acc[h][e] += w * fv[e];
+                    }
+                }
+            }
+            __syncthreads();
+        } else {
+            __syncthreads();
+            // ---- phases 2 + 3, one wave per head
+    #pragma unroll
+            for (int j = 0; j < OWN; j++) {
+                const int h = wave + 4 * j;
+                if (h < RATIO) {                                     // wave-uniform
+                    float* ph = ps + h * ATT_TILE;
+                    float sc[ATT_TILE / 64];
+                    float tmax = -1e30f;
+    #pragma unroll
+                    for (int i = 0; i < ATT_TILE / 64; i++) {
+                        const int t = lane + 64 * i;
+                        sc[i] = t < tl ? ph[t] : -1e30f;
+                        tmax = fmaxf(tmax, sc[i]);
+                    }
+                    tmax = wave_max(tmax);
+                    const float m_new = fmaxf(m_run[j], tmax);
+                    const float corr = expf(m_run[j] - m_new);
+                    float psum = 0.0f;
+    #pragma unroll
+                    for (int i = 0; i < ATT_TILE / 64; i++) {
+                        const int t = lane + 64 * i;
+                        const float pv = t < tl ? expf(sc[i] - m_new) : 0.0f;
+                        if (t < tl) ph[t] = pv;
+                        psum += pv;
+                    }
+                    psum = t12_wave_sum(psum);
+                    l_run[j] = l_run[j] * corr + psum;
+                    m_run[j] = m_new;
+    #pragma unroll
+                    for (int e = 0; e < 16; e++) acc[j][e] *= corr;
+                    // P.V: iteration it covers positions it*PG + g; loads of 4 iterations are issued together
+                    for (int it = 0; it * PG < tl; it += 4) {
+                        uint4 vv[4];
+                        float w[4];
+    #pragma unroll
+                        for (int x = 0; x < 4; x++) {
+                            const int t = (it + x) * PG + g;
+                            const bool ok = t < tl;
+                            const int tc = ok ? t : 0;
+                            if (FUSE && t0 == c0) {
+                                vv[x] = ((const uint4*)vt)[tc * CH + c];
+                                w[x] = ok ? ph[tc] * vts[tc] : 0.0f;
+                            } else {
+                                vv[x] = *(const uint4*)(vbase + (size_t)(t0 + tc) * kv_dim + c * 16);
+                                w[x] = ok ? ph[tc] * svb[(size_t)(t0 + tc) * n_head_kv] : 0.0f;
+                            }
+                        }
+    #pragma unroll
+                        for (int x = 0; x < 4; x++) {
+                            const uint32_t w4[4] = {vv[x].x, vv[x].y, vv[x].z, vv[x].w};
+    #pragma unroll
+                            for (int e = 0; e < 16; e++)
+                                acc[j][e] += w[x] * (float)(int8_t)((w4[e >> 2] >> (8 * (e & 3))) & 0xFF);
                         }
                     }
-#pragma unroll
-                    for (int x = 0; x < 4; x++) {
-                        const uint32_t w4[4] = {vv[x].x, vv[x].y, vv[x].z, vv[x].w};
-#pragma unroll
-                        for (int e = 0; e < 16; e++)
-                            acc[j][e] += w[x] * (float)(int8_t)((w4[e >> 2] >> (8 * (e & 3))) & 0xFF);
-                    }
                 }
+            }
+            __syncthreads();
+        }
+    }
+    if constexpr (WIDE) {
+        // ---- fold: position classes inside a wave, then the four waves through LDS
+        __shared__ __attribute__((aligned(16))) float red[4 * RATIO * HD];
+        __shared__ float mstat[RATIO], lstat[RATIO];
+    #pragma unroll
+        for (int h = 0; h < RATIO; h++) {
+    #pragma unroll
+            for (int e = 0; e < 16; e++) {
+                float v = acc[h][e];
+    #pragma unroll
+                for (int off = CH; off < 64; off <<= 1) v += __shfl_xor(v, off, T12_WAVE);
+                acc[h][e] = v;
+            }
+            if (g == 0) {
+    #pragma unroll
+                for (int e = 0; e < 16; e += 4)
+                    *(float4*)(red + ((size_t)wave * RATIO + h) * HD + c * 16 + e) =
+                        make_float4(acc[h][e], acc[h][e + 1], acc[h][e + 2], acc[h][e + 3]);
+            }
+        }
+    #pragma unroll
+        for (int j = 0; j < OWN; j++) {
+            const int h = wave + 4 * j;
+            if (h < RATIO && lane == 0) {
+                mstat[h] = m_run[j];
+                lstat[h] = l_run[j];
             }
         }
         __syncthreads();
-    }
-#pragma unroll
-    for (int j = 0; j < OWN; j++) {
-        const int h = wave + 4 * j;
-        if (h < RATIO) {
-#pragma unroll
-            for (int e = 0; e < 16; e++) {
-                float v = acc[j][e];
-#pragma unroll
-                for (int off = CH; off < 64; off <<= 1) v += __shfl_xor(v, off, T12_WAVE);   // fold position classes
-                acc[j][e] = v;
+        for (int i = tid; i < RATIO * HD / 4; i += 256) {
+            const int h = i / (HD / 4), d = (i % (HD / 4)) * 4;
+            float4 a = *(const float4*)(red + (size_t)h * HD + d);
+    #pragma unroll
+            for (int w = 1; w < 4; w++) {
+                const float4 o = *(const float4*)(red + ((size_t)w * RATIO + h) * HD + d);
+                a.x += o.x; a.y += o.y; a.z += o.z; a.w += o.w;
             }
-            if (g == 0) {
-                if (SPLIT) {
-                    float* pw = sp.ws + ((((size_t)b * n_head_kv + kvh) * nchunk + blockIdx.z) * RATIO + h) * (HD + 4);
-#pragma unroll
-                    for (int e = 0; e < 16; e += 4)
-                        *(float4*)(pw + c * 16 + e) = make_float4(acc[j][e], acc[j][e + 1], acc[j][e + 2], acc[j][e + 3]);
-                    if (c == 0) {
-                        pw[HD] = m_run[j];
-                        pw[HD + 1] = l_run[j];
+            if (SPLIT) {
+                float* pw = sp.ws + ((((size_t)b * n_head_kv + kvh) * nchunk + blockIdx.z) * RATIO + h) * (HD + 4);
+                *(float4*)(pw + d) = a;
+                if (d == 0) {
+                    pw[HD] = mstat[h];
+                    pw[HD + 1] = lstat[h];
+                }
+            } else {
+                const float inv = 1.0f / lstat[h];
+                *(uint2*)(out + (size_t)b * n_head * HD + (size_t)(kvh * RATIO + h) * HD + d) =
+                    make_uint2(t12_f32_to_bf16(a.x * inv) | ((uint32_t)t12_f32_to_bf16(a.y * inv) << 16),
+                               t12_f32_to_bf16(a.z * inv) | ((uint32_t)t12_f32_to_bf16(a.w * inv) << 16));
+            }
+        }
+    } else {
+    #pragma unroll
+        for (int j = 0; j < OWN; j++) {
+            const int h = wave + 4 * j;
+            if (h < RATIO) {
+    #pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    float v = acc[j][e];
+    #pragma unroll
+                    for (int off = CH; off < 64; off <<= 1) v += __shfl_xor(v, off, T12_WAVE);   // fold position classes
+                    acc[j][e] = v;
+                }
+                if (g == 0) {
+                    if (SPLIT) {
+                        float* pw = sp.ws + ((((size_t)b * n_head_kv + kvh) * nchunk + blockIdx.z) * RATIO + h) * (HD + 4);
+    #pragma unroll
+                        for (int e = 0; e < 16; e += 4)
+                            *(float4*)(pw + c * 16 + e) = make_float4(acc[j][e], acc[j][e + 1], acc[j][e + 2], acc[j][e + 3]);
+                        if (c == 0) {
+                            pw[HD] = m_run[j];
+                            pw[HD + 1] = l_run[j];
+                        }
+                    } else {
+                        const float inv = 1.0f / l_run[j];
+                        uint32_t o[8];
+    #pragma unroll
+                        for (int e = 0; e < 8; e++)
+                            o[e] = t12_f32_to_bf16(acc[j][2 * e] * inv) | ((uint32_t)t12_f32_to_bf16(acc[j][2 * e + 1] * inv) << 16);
+                        uint4* dst = (uint4*)(out + (size_t)b * n_head * HD + (size_t)(kvh * RATIO + h) * HD + c * 16);
+                        dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
+                        dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
                     }
-                } else {
-                    const float inv = 1.0f / l_run[j];
-                    uint32_t o[8];
-#pragma unroll
-                    for (int e = 0; e < 8; e++)
-                        o[e] = t12_f32_to_bf16(acc[j][2 * e] * inv) | ((uint32_t)t12_f32_to_bf16(acc[j][2 * e + 1] * inv) << 16);
-                    uint4* dst = (uint4*)(out + (size_t)b * n_head * HD + (size_t)(kvh * RATIO + h) * HD + c * 16);
-                    dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
-                    dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
                 }
             }
         }
@@ -862,6 +1105,7 @@ void launch_rope_kv(float* q, float* k, const float* v, int8_t* ck, int8_t* cv, 
 
 int g_attn_fast = 1;   // 0: always the general kernel (tests compare the two)
 int g_attn_chunk = 256; // context split: fewest positions per chunk; 0 = never split
+int g_attn_wide = 320;  // contexts from this length on take the form with INT8 MFMA scores and one wave per 64 positions
 
 // Scratch of the context split: partial results of at most ATT_SPLIT_WGS workgroups and one
 // counter per (sequence, KV head); the counters start at zero and every launch leaves them there.
@@ -918,22 +1162,31 @@ void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float
             sp.counter = g_split_cnt;
         }
     }
+    // Two forms of the kernel.  Short contexts: scores by fp32 FMAs with one thread per position, P.V with one
+    // wave per head -- few registers, four workgroups per CU, no set-up: a workgroup is a chain of latencies that
+    // only occupancy hides.  Long contexts: scores by INT8 MFMAs (Q split into two INT8 limbs, K used as stored),
+    // P.V with one wave per 64 positions, every V value converted once for all heads and requested before the
+    // softmax phase -- the kernel is bound by conversions and FMAs there.  seq_len is the caller's hint when
+    // positions are given.  Measured on per-sequence caches, B = 256: equal at 300 positions, 1.5x at 2000
+    // (503 -> 305 us for 1.08 GB), 2.5x for B = 64 at 8000.
+    const bool wide = seq_len >= g_attn_wide;
+#define T12_ATT_GO(HD_, R_, F_, S_, W_)                                                                         \
+    hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, F_, S_, W_>), dim3(n_head_kv, batch, S_ ? nchunk : 1), dim3(256), 0, \
+                       st, q, ck, cv, sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride,   \
+                       fuse ? *fuse : AttnFuse(), sp)
 #define T12_ATT_FAST(HD_, R_)                                                                                   \
     if (head_dim == HD_ && ratio == R_) {                                                                       \
-        if (fuse && nchunk > 1)                                                                                 \
-            hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, true, true>), dim3(n_head_kv, batch, nchunk), dim3(256), 0, st, q, \
-                               ck, cv, sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride, *fuse, sp); \
-        else if (fuse)                                                                                          \
-            hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, true, false>), dim3(n_head_kv, batch), dim3(256), 0, st, q, \
-                               ck, cv, sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride, *fuse, sp); \
-        else if (nchunk > 1)                                                                                    \
-            hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, false, true>), dim3(n_head_kv, batch, nchunk), dim3(256), 0, st, q, \
-                               ck, cv, sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride,  \
-                               AttnFuse(), sp);                                                                 \
-        else                                                                                                    \
-            hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, false, false>), dim3(n_head_kv, batch), dim3(256), 0, st, q, \
-                               ck, cv, sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride,  \
-                               AttnFuse(), sp);                                                                 \
+        const int sel = (fuse ? 4 : 0) | (nchunk > 1 ? 2 : 0) | (wide ? 1 : 0);                                 \
+        switch (sel) {                                                                                          \
+        case 0: T12_ATT_GO(HD_, R_, false, false, false); break;                                                \
+        case 1: T12_ATT_GO(HD_, R_, false, false, true); break;                                                 \
+        case 2: T12_ATT_GO(HD_, R_, false, true, false); break;                                                 \
+        case 3: T12_ATT_GO(HD_, R_, false, true, true); break;                                                  \
+        case 4: T12_ATT_GO(HD_, R_, true, false, false); break;                                                 \
+        case 5: T12_ATT_GO(HD_, R_, true, false, true); break;                                                  \
+        case 6: T12_ATT_GO(HD_, R_, true, true, false); break;                                                  \
+        default: T12_ATT_GO(HD_, R_, true, true, true); break;                                                  \
+        }                                                                                                       \
         report("attention");                                                                                    \
         return;                                                                                                 \
     }
@@ -946,6 +1199,7 @@ void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float
         T12_ATT_FAST(64, 4)
     }
 #undef T12_ATT_FAST
+#undef T12_ATT_GO
     const size_t smem = ((size_t)ratio * head_dim + (size_t)ratio * ATT_TILE + 17 + 2 * ratio) * sizeof(float);
     hipLaunchKernelGGL(attn_decode_kernel, dim3(n_head_kv, batch), dim3(256), smem, st, q, ck, cv, sk, sv,
                        (uint16_t*)out, positions, seq_len, n_head, n_head_kv, head_dim, scale, kv_stride);
@@ -994,12 +1248,13 @@ void launch_rope_scaling(float factor, float low_freq_factor, float high_freq_fa
 }
 
 // 0: always the general kernel; 1 (default): shapes with a specialised kernel use it, one sequence at a long
-// context split into chunks of at least 256 positions; 2: specialised kernels, never split; n >= 16: specialised
-// kernels, chunks of at least n positions.
+// context split into chunks of at least 256 positions, the form with INT8 MFMA scores and one wave per 64 positions in the P.V phase from 320 positions;
+// 2: specialised kernels, never split; 3: never that P.V phase; 4: always; n >= 16: chunks of at least n positions.
 int t12_tune_attention(int mode)
 {
     g_attn_fast = mode != 0;
     g_attn_chunk = mode >= 16 ? mode : (mode == 2 ? 0 : 256);
+    g_attn_wide = mode == 3 ? 0x7FFFFFFF : (mode == 4 ? 0 : 320);
     return 0;
 }
 
