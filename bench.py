@@ -21,6 +21,10 @@ Workloads (synthetic, seeded, random-init weights of the Llama-3.1-8B shape:
   moe             one step = one Mixtral-8x7B-shaped MoE FFN layer (8 split-12 experts, top-2) over 256 tokens
                   grouped per expert through the decode+GEMM.
 
+  attention       the attention step of one decoder layer (RoPE, INT8 KV store, GQA decode attention over the
+                  INT8 cache) with every sequence on its own cache region, at several (batch, context) points;
+                  `roofline` prices the cache bytes of B = 256 at 2000 positions against the HBM peak.
+
   gemv_stack_b1   one step = every linear layer of one decode step at B = 1 through
                   the fused split-12 decode-GEMV: per layer QKV (3 segments, one
                   launch), O, gate+up (2 segments, one launch), down; then lm_head.
@@ -342,6 +346,56 @@ def run_moe(args, t12, torch, dev):
     }
 
 
+def run_attention(args, t12, torch, dev):
+    """The attention step of one Llama-3.1-8B decoder layer (RoPE of q and k, INT8 store of the new K / V
+    row, GQA attention over the INT8 cache: launch_rope_store_attention), every sequence on its own cache
+    region, at several (batch, context) points; `value` is the B = 256, 2000-position case in GB/s of cache read."""
+    import numpy as np
+    nh, nkv, hd, theta = LLAMA8B["n_head"], LLAMA8B["n_head_kv"], LLAMA8B["n_embd"] // LLAMA8B["n_head"], 500000.0
+    kv_dim = nkv * hd
+    cur = torch.cuda.current_stream()
+    g = torch.Generator(device=dev)
+    g.manual_seed(77)
+    cases = [(256, 2048, 2000), (256, 2048, 150), (64, 8192, 8000), (16, 2048, 1000), (1, 8192, 8000), (1, 2048, 2000),
+             (1, 2048, 150)]
+    out_cases = {}
+    for B, S, ctx in cases:
+        kc = torch.randint(-127, 128, (B, S, kv_dim), dtype=torch.int8, device=dev, generator=g)
+        vc = torch.randint(-127, 128, (B, S, kv_dim), dtype=torch.int8, device=dev, generator=g)
+        ks = torch.rand((B, S, nkv), device=dev, generator=g) / 127 + 0.004
+        vs = torch.rand((B, S, nkv), device=dev, generator=g) / 127 + 0.004
+        q = torch.randn((B, nh * hd), device=dev, generator=g)
+        k = torch.randn((B, kv_dim), device=dev, generator=g)
+        v = torch.randn((B, kv_dim), device=dev, generator=g)
+        out = torch.zeros((B, nh * hd), dtype=torch.int16, device=dev)
+        pos = torch.full((B,), ctx - 1, dtype=torch.int32, device=dev)
+
+        def step():
+            t12.lib.launch_rope_store_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                                                ks.data_ptr(), vs.data_ptr(), out.data_ptr(),
+                                                pos.data_ptr() if B > 1 else None, ctx - 1, nh, nkv, hd, theta,
+                                                1.0 / np.sqrt(hd), B, S * kv_dim if B > 1 else 0, cur.cuda_stream)
+        for _ in range(max(args.warmup, 1)):
+            step()
+        _, ms = timed(torch, cur, step, args.steps)
+        nbytes = B * ctx * (2 * kv_dim + 8 * nkv)            # INT8 K and V rows + their fp32 scales
+        out_cases["b%d_ctx%d" % (B, ctx)] = {"us": ms * 1e3, "cache_MB": nbytes / 1e6, "GBps": nbytes / ms / 1e6}
+        del kc, vc, ks, vs
+    head = out_cases["b256_ctx2000"]
+    return {
+        "metric": "GB/s of INT8 KV cache read by the decode-attention step of one Llama-3.1-8B layer, B=256 at 2000 positions",
+        "value": head["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head["us"] / 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "attention: RoPE + INT8 KV store + GQA decode attention (32 / 8 heads, head_dim 128), "
+                               "per-sequence cache regions, random INT8 caches"},
+        "cases": out_cases,
+        "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": head["GBps"] / HBM_PEAK_GBS, "traffic": None, "kernel": "attn_fast_kernel<128,4> (long-context form)",
+                     "bytes_per_launch": head["cache_MB"] * 1e6, "us_per_launch": head["us"]},
+    }
+
+
 def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(16, 64, 256), iters=10):
     """decode+GEMM per layer shape: for each B, each of QKV (3 segments), O, gate|up
     (2 segments), down is timed over `n_rot` distinct weight copies in rotation, so that neither L2 nor
@@ -428,7 +482,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="decode", choices=["decode", "gemv_stack_b1", "moe", "gemm_layers"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "gemv_stack_b1", "moe", "gemm_layers", "attention"])
     ap.add_argument("--prompt", type=int, default=128)
     ap.add_argument("--no-batch256", dest="batch256", action="store_false")
     ap.add_argument("--layers", type=int, default=LLAMA8B["n_layer"], help="debug: fewer layers (invalid as a result)")
@@ -455,6 +509,9 @@ def main():
         return
     if args.workload == "moe":
         print(json.dumps(run_moe(args, t12, torch, dev)))
+        return
+    if args.workload == "attention":
+        print(json.dumps(run_attention(args, t12, torch, dev)))
         return
     cfg = dict(LLAMA8B, n_layer=args.layers)
 

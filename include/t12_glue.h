@@ -100,9 +100,11 @@ void launch_flash_attention_batch(const float* q, const int8_t* kv_k, const int8
                                   int n_head_kv, int head_dim, int max_seq, float scale, int batch_size, int kv_stride,
                                   hipStream_t stream);
 /* RoPE + KV store + attention in ONE launch (replaces inference.cpp:275-282: launch_rope_store_kv followed by
- * launch_attention_all_heads).  positions == NULL: every sequence is at `position`.  The in-kernel fusion is
- * used for batch_size 1 or per-sequence caches (kv_stride != 0); with a shared cache region the RoPE/KV kernel
- * runs first.  No counterpart of its own in the reference. */
+ * launch_attention_all_heads).  positions == NULL: every sequence is at `position`; with a position array
+ * `position` is only a length hint (the largest position) for the choice of the attention kernel's form.  The
+ * in-kernel fusion is used for batch_size 1 and for small batches on per-sequence caches (kv_stride != 0,
+ * batch_size * n_head_kv <= 256); otherwise the RoPE/KV kernel runs first and q is left rotated.  No
+ * counterpart of its own in the reference. */
 void launch_rope_store_attention(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v, float* scale_k,
                                  float* scale_v, int16_t* output, const int* positions, int position, int n_head,
                                  int n_head_kv, int head_dim, float theta, float scale, int batch_size, int kv_stride,

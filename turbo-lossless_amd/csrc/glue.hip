@@ -1361,16 +1361,19 @@ void launch_rope_store_kv_batch(float* q, float* k, const float* v, int8_t* kv_k
 
 // Extension of the reference's launch layer: RoPE (Q and K) + INT8 KV store + attention in ONE
 // launch, for B >= 1.  positions: device array [batch] (NULL: every sequence is at `position`).
-// Shapes without a specialised kernel run the separate launches.  q is left unrotated.
+// Shapes without a specialised kernel, and large batches, run the separate launches.  q is scratch: left as
+// it was by the fused kernel, rotated in place by the separate RoPE launch.
 void launch_rope_store_attention(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v, float* scale_k,
                                  float* scale_v, int16_t* output, const int* positions, int position, int n_head,
                                  int n_head_kv, int head_dim, float theta, float scale, int batch_size, int kv_stride,
                                  hipStream_t stream)
 {
-    // Fusing pays when every workgroup stores its own cache slot: one sequence, or per-sequence
-    // caches.  Lock-step copies on a shared cache (kv_stride = 0, batch > 1) would store the same
-    // slot from every workgroup, so they keep the separate store launch.
-    if (attn_has_fast(n_head, n_head_kv, head_dim) && (batch_size == 1 || kv_stride != 0)) {
+    // Fusing pays when every workgroup stores its own cache slot (one sequence, or per-sequence caches) and
+    // the launch is small enough to be a chain of latencies: the fused kernel stages a V tile in LDS and holds
+    // prefetched rows in registers, so only two or three of its workgroups fit a CU (measured at B = 256 on
+    // per-sequence caches: 221 us fused against 37 us + 9 us for the two launches at 150 positions).  Lock-step
+    // copies on a shared cache (kv_stride = 0, batch > 1) would store the same slot from every workgroup.
+    if (attn_has_fast(n_head, n_head_kv, head_dim) && (batch_size == 1 || (kv_stride != 0 && batch_size * n_head_kv <= 256))) {
         AttnFuse fz;
         fz.k_new = k;
         fz.v_new = v;
