@@ -236,7 +236,14 @@ def test_fused_rope_store_attention_equals_separate_launches(t12, oracle, attn_m
         torch.cuda.synchronize()
         assert torch.equal(f[3], a[3]) and torch.equal(f[4], a[4])      # caches
         assert torch.equal(f[5], a[5]) and torch.equal(f[6], a[6])      # scales
-        assert torch.equal(of, oa)
+        if positions is not None:
+            assert torch.equal(of, oa)
+        else:
+            # without a position array the launch may be split along the context: other tile boundaries, other
+            # rounding of the partial sums (and of the INT8 weight limbs of the long-context form)
+            got = oracle.bf16_bits_to_f32(of.cpu().numpy().view(np.uint16))
+            want = oracle.bf16_bits_to_f32(oa.cpu().numpy().view(np.uint16))
+            assert np.abs(got - want).max() <= 2.0 ** -7 * np.abs(want).max()
 
 
 @pytest.mark.parametrize("nh,nkv,hd", [(32, 8, 128), (8, 2, 32), (4, 4, 64)])

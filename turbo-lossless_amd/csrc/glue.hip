@@ -448,9 +448,10 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
     // FUSE: the cache rows of the first tile are requested before anything else, so that their HBM
     // latency runs under the Q / new-K / new-V work instead of behind it: this lane's K row (phase 1)
     // into registers and the V tile through registers into LDS (phase 3 reads it from there).  The row of the position being written (FUSE) is not in memory yet: it comes from LDS.
-    constexpr int VPRE = FUSE ? (ATT_TILE * CH) / 256 : 0;          // 16-byte V pieces per thread
-    __shared__ __attribute__((aligned(16))) int8_t vt[FUSE ? ATT_TILE * HD : 16];
-    __shared__ float vts[FUSE ? ATT_TILE : 1];
+    constexpr bool VLDS = FUSE && !WIDE;                            // (the long-context form stages V itself, tile by tile)
+    constexpr int VPRE = VLDS ? (ATT_TILE * CH) / 256 : 0;          // 16-byte V pieces per thread
+    __shared__ __attribute__((aligned(16))) int8_t vt[VLDS ? ATT_TILE * HD : 16];
+    __shared__ float vts[VLDS ? ATT_TILE : 1];
     __shared__ __attribute__((aligned(16))) int8_t knew8[FUSE ? HD : 16];
     __shared__ float knew_scale;
     const int tl0 = min(ATT_TILE, c1 - c0);
@@ -492,7 +493,7 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
     }
     uint4 v_pre[VPRE > 0 ? VPRE : 1];
     float vs_pre = 0.0f;
-    if (FUSE) {
+    if (VLDS) {
 #pragma unroll
         for (int x = 0; x < VPRE; x++) {
             const int idx = tid + 256 * x, t = idx / CH, u = idx % CH;
@@ -535,8 +536,8 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
             const int8_t q1 = (int8_t)(int)fminf(fmaxf(rintf(r1 * inv), -127.0f), 127.0f);
             // the new row: to the cache, and (first tile) to LDS where this launch reads it
             const int rel = pos - c0;                                // position inside this chunk
-            int8_t* lrow = wave == 0 ? knew8 : vt + (size_t)(rel < ATT_TILE ? rel : 0) * HD;
-            const bool to_lds = wave == 0 || rel < ATT_TILE;
+            int8_t* lrow = wave == 0 ? knew8 : vt + (size_t)(VLDS && rel < ATT_TILE ? rel : 0) * HD;
+            const bool to_lds = wave == 0 || (VLDS && rel < ATT_TILE);
             if (own) {
                 row[lane] = q0;
                 row[lane + HALF] = q1;
@@ -548,7 +549,7 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
             if (lane == 0) {
                 (wave == 0 ? fz.sk_w : fz.sv_w)[(size_t)b * sstride + (size_t)pos * n_head_kv + kvh] = amax / 127.0f;
                 if (wave == 0) knew_scale = amax / 127.0f;
-                else if (rel < ATT_TILE) vts[rel] = amax / 127.0f;
+                else if (VLDS && rel < ATT_TILE) vts[rel] = amax / 127.0f;
             }
         }
         __threadfence();      // later tiles read the new row back through the cache pointers
@@ -558,17 +559,18 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
             const int idx = tid + 256 * x, t = idx / CH;
             if (t < tl0 && c0 + t != newpos) ((uint4*)vt)[idx] = v_pre[x];
         }
-        if (tid < tl0 && c0 + tid != newpos) vts[tid] = vs_pre;
+        if (VLDS && tid < tl0 && c0 + tid != newpos) vts[tid] = vs_pre;
     }
     __syncthreads();
 
     // Q as two INT8 limbs per element, q ~ s_h (a1 + a2 / 254) with s_h = max|q_h| / 127 (error <= 1.6e-5 max|q_h|,
     // below what the bf16 output resolves), laid out as the A operand of the score MFMAs: row 8 * limb + h.
     // INT8 x INT8 products accumulate exactly in int32, so K needs no conversion at all.
-    __shared__ __attribute__((aligned(16))) int8_t qlimb[WIDE ? 32 * HD : 16];
+    constexpr int QSTR = HD + 16;               // row pitch of qlimb, for the same reason as WSTR
+    __shared__ __attribute__((aligned(16))) int8_t qlimb[WIDE ? 32 * QSTR : 16];
     __shared__ float qscale[RATIO];
     if constexpr (WIDE) {
-    for (int i = tid; i < 32 * HD / 16; i += 256) ((uint4*)qlimb)[i] = make_uint4(0, 0, 0, 0);
+    for (int i = tid; i < 32 * QSTR / 16; i += 256) ((uint4*)qlimb)[i] = make_uint4(0, 0, 0, 0);
     __syncthreads();
     for (int h = wave; h < RATIO; h += 4) {
         float amax = 0.0f;
@@ -579,18 +581,18 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
             const float r0 = qs[h * HD + d] * inv;
             const float a1 = fminf(fmaxf(rintf(r0), -127.0f), 127.0f);
             const float a2 = fminf(fmaxf(rintf((r0 - a1) * 254.0f), -127.0f), 127.0f);
-            qlimb[h * HD + d] = (int8_t)(int)a1;
-            qlimb[(8 + h) * HD + d] = (int8_t)(int)a2;
+            qlimb[h * QSTR + d] = (int8_t)(int)a1;
+            qlimb[(8 + h) * QSTR + d] = (int8_t)(int)a2;
         }
         if (lane == 0) qscale[h] = amax / 127.0f;
     }
     __syncthreads();
     }
-    const int8_t* qa_src = qlimb + ln * HD + lh * (HD / 2);      // this lane's A operand pieces (re-read per tile: 4 LDS loads)
+    const int8_t* qa_src = qlimb + ln * QSTR + lh * (HD / 2);      // this lane's A operand pieces (re-read per tile: 4 LDS loads)
 
     // running maximum / sum of head h live in the wave that owns it (h % 4); the output sums of ALL heads live
     // in every wave, over the 64 positions of each tile that the wave takes in phase 3
-    constexpr int NACC = WIDE ? RATIO : OWN;
+    constexpr int NACC = WIDE ? 1 : OWN;
     float m_run[OWN], l_run[OWN], acc[NACC][16];
 #pragma unroll
     for (int j = 0; j < OWN; j++) {
@@ -602,52 +604,110 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
 #pragma unroll
         for (int e = 0; e < 16; e++) acc[h][e] = 0.0f;
     __shared__ float corr_s[RATIO];
-    constexpr int NIT = 64 / PG;                // phase 3 iterations per wave and tile
-    const int g = lane / CH, c = lane % CH;     // phase 3: position class, 16-dim chunk
-
-    for (int t0 = c0; t0 < c1; t0 += ATT_TILE) {
-        const int tl = min(ATT_TILE, c1 - t0);
-        if constexpr (WIDE) {
-        // ---- phase 1: scores of 64 positions per wave, two blocks of 32, KS INT8 MFMAs each
-        t12_i32x4 qa[KS];
-#pragma unroll
-        for (int u = 0; u < KS; u++) qa[u] = *(const t12_i32x4*)(qa_src + 16 * u);
+    // Long-context form, P.V phase: out[h, d] = sum_t w[h, t] V8[t, d] with w = p * v_scale, again as INT8 MFMAs: w in two
+    // INT8 limbs per (head, position) (rows 8 * limb + h of wq), V staged 128 positions at a time in LDS (rows padded to
+    // VSTR bytes: conflict-free) and read back TRANSPOSED (ds_read_b64_tr_b8: inside 16 lanes, lane 8 par + c receives
+    // byte c of the rows that lanes par, 2 + par, ... 14 + par point at), which is the B operand: 16 consecutive
+    // positions of one dim per lane.  Wave w owns dims 32 w .. 32 w + 31; lane (ln, lh) ends with heads 4 lh .. 4 lh + 3 of
+    // dim 32 w + ln in o_w[].
+    constexpr int VSTR = HD + 16;
+    constexpr int NBLK = HD / 32;               // dim blocks = waves busy in this phase
+    __shared__ __attribute__((aligned(16))) int8_t vth[WIDE ? 128 * VSTR : 16];
+    constexpr int WSTR = ATT_TILE + 16;         // row pitch of wq: 32 lanes reading 16 bytes of 32 different rows, no bank shared
+    __shared__ __attribute__((aligned(16))) int8_t wq[WIDE ? 32 * WSTR : 16];
+    __shared__ float wscale_s[RATIO];
+    float o_w[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    constexpr int VP = WIDE ? 128 * CH / 256 : 1;   // 16-byte V pieces per thread and half tile
+    t12_u32x4 vreg[VP];     // (a native vector type: the compiler keeps this loop-carried array in registers)
+    float vsc[OWN][ATT_TILE / 64], vsc_n[OWN][ATT_TILE / 64];
+    uint4 kk[2][WIDE ? KS : 1];
+    float kscale[2] = {0.0f, 0.0f};
+    // Requests of the long-context form.  Every tile's K rows, V scales and first 128 V rows are asked for one tile
+    // ahead (the registers they land in are free by then), its other 128 V rows during its softmax phase: no
+    // memory latency stays exposed inside a workgroup.
+    auto issue_k = [&](int t0x, int tlx, bool first) __attribute__((always_inline)) {
 #pragma unroll
         for (int nb = 0; nb < 2; nb++) {
             const int tp = wave * 64 + nb * 32 + ln;                 // position inside the tile
-            if (wave * 64 + nb * 32 < tl) {                          // wave-uniform: the block holds positions
-                const int t = t0 + min(tp, tl - 1);                  // rows past the end repeat the last one (masked in phase 2)
-                uint4 kk[KS];
-                float kscale;
-                if (t0 == c0 && kpre[nb]) {
+            if (wave * 64 + nb * 32 < tlx) {                         // wave-uniform: the block holds positions
+                const int t = t0x + min(tp, tlx - 1);                // rows past the end repeat the last one (masked in phase 2)
+                if (first && kpre[nb]) {
 #pragma unroll
-                    for (int u = 0; u < KS; u++) kk[u] = kk_pre[nb][u];
-                    kscale = kscale_pre[nb];
-                } else if (FUSE && t == newpos && t0 == c0) {
+                    for (int u = 0; u < KS; u++) kk[nb][u] = kk_pre[nb][u];
+                    kscale[nb] = kscale_pre[nb];
+                } else if (FUSE && first && t == newpos) {
 #pragma unroll
-                    for (int u = 0; u < KS; u++) kk[u] = ((const uint4*)(knew8 + lh * (HD / 2)))[u];
-                    kscale = knew_scale * scale;
+                    for (int u = 0; u < KS; u++) kk[nb][u] = ((const uint4*)(knew8 + lh * (HD / 2)))[u];
+                    kscale[nb] = knew_scale * scale;
                 } else {
                     const uint4* kr = (const uint4*)(kbase + (size_t)t * kv_dim + lh * (HD / 2));
 #pragma unroll
-                    for (int u = 0; u < KS; u++) kk[u] = kr[u];
-                    kscale = skb[(size_t)t * n_head_kv] * scale;
+                    for (int u = 0; u < KS; u++) kk[nb][u] = kr[u];
+                    kscale[nb] = skb[(size_t)t * n_head_kv] * scale;
                 }
+            }
+        }
+    };
+    auto issue_v = [&](int t0x, int tlx, int half) __attribute__((always_inline)) {
+#pragma unroll
+        for (int x = 0; x < VP; x++) {
+            const int idx = tid + 256 * x, t = min(half * 128 + idx / CH, tlx - 1), u = idx % CH;
+            vreg[x] = *(const t12_u32x4*)(vbase + (size_t)(t0x + t) * kv_dim + u * 16);
+        }
+    };
+    auto issue_vsc = [&](int t0x, int tlx, float (&dst)[OWN][ATT_TILE / 64]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < OWN; j++)
+#pragma unroll
+            for (int i = 0; i < ATT_TILE / 64; i++) {
+                const int t = lane + 64 * i;
+                dst[j][i] = (wave + 4 * j < RATIO && t < tlx) ? svb[(size_t)(t0x + t) * n_head_kv] : 0.0f;
+            }
+    };
+    if constexpr (WIDE) {
+        for (int i = tid; i < 32 * WSTR / 16; i += 256) ((uint4*)wq)[i] = make_uint4(0, 0, 0, 0);
+        __syncthreads();
+    }
+    const int g = lane / CH, c = lane % CH;     // phase 3: position class, 16-dim chunk
+    if constexpr (WIDE) {
+        issue_k(c0, tl0, true);
+        issue_vsc(c0, tl0, vsc);
+        issue_v(c0, tl0, 0);
+    }
+
+    for (int t0 = c0; t0 < c1; t0 += ATT_TILE) {
+        const int tl = min(ATT_TILE, c1 - t0);
+        const int t0n = t0 + ATT_TILE;
+        const bool has_next = t0n < c1;
+        const int tln = min(ATT_TILE, c1 - t0n);
+        if constexpr (WIDE) {
+        // ---- phase 1: scores of 64 positions per wave, two blocks of 32, KS INT8 MFMAs each
+        // (the K rows, V rows and V scales of this tile were requested during the previous tile, or before the loop)
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) {
+            const int tp = wave * 64 + nb * 32 + ln;
+            if (wave * 64 + nb * 32 < tl) {
                 t12_i32x16 sacc;
 #pragma unroll
                 for (int r = 0; r < 16; r++) sacc[r] = 0;
 #pragma unroll
                 for (int u = 0; u < KS; u++)
-                    sacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[u], __builtin_bit_cast(t12_i32x4, kk[u]), sacc, 0, 0, 0);
+                    sacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(*(const t12_i32x4*)(qa_src + 16 * u),
+                                                                 __builtin_bit_cast(t12_i32x4, kk[nb][u]), sacc, 0, 0, 0);
                 // lane (ln, lh) holds column ln = its position; rows 4 lh + r (limb 0) and 8 + 4 lh + r (limb 1),
                 // r = 0..3: heads 4 lh .. 4 lh + 3
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const int h = 4 * lh + r;
                     if (h < RATIO)
-                        ps[h * ATT_TILE + tp] = ((float)sacc[r] + (float)sacc[4 + r] * (1.0f / 254.0f)) * (qscale[h] * kscale);
+                        ps[h * ATT_TILE + tp] = ((float)sacc[r] + (float)sacc[4 + r] * (1.0f / 254.0f)) * (qscale[h] * kscale[nb]);
                 }
             }
+        }
+        // the next tile's K rows and V scales travel under the rest of this tile
+        if (has_next) {
+            issue_k(t0n, tln, false);
+            issue_vsc(t0n, tln, vsc_n);
         }
         } else {
         // ---- phase 1
@@ -687,30 +747,26 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
         }
         }
         if constexpr (WIDE) {
-            // ---- V rows of this wave's 64 positions: requested now, consumed after the softmax bookkeeping
-            const bool v_lds = FUSE && t0 == c0;                         // first tile of the fused launch: V tile is in LDS
-            const bool v_any = wave * 64 < tl;                           // wave-uniform
-            uint4 vv[NIT];
-            float vsc[NIT];
-            if (v_any && !v_lds) {
-    #pragma unroll
-                for (int x = 0; x < NIT; x++) {
-                    const int tp = wave * 64 + x * PG + g;
-                    const int tc = min(tp, tl - 1);
-                    vv[x] = *(const uint4*)(vbase + (size_t)(t0 + tc) * kv_dim + c * 16);
-                    vsc[x] = svb[(size_t)(t0 + tc) * n_head_kv];
-                }
+            // ---- V, first 128 positions of the tile: registers -> LDS (rows past the end repeat the last one; their
+            //      weights are zero)
+#pragma unroll
+            for (int x = 0; x < VP; x++) {
+                const int idx = tid + 256 * x;
+                *(t12_u32x4*)(vth + (idx / CH) * VSTR + (idx % CH) * 16) = vreg[x];
             }
+            if (128 < tl) issue_v(t0, tl, 1);                       // the other 128 rows: in flight under the softmax phase
+            else if (has_next) issue_v(t0n, tln, 0);                 // (only the last tile of a chunk can be this short)
             __syncthreads();
-            // ---- phase 2, one wave per head: tile maximum, rescale factor, probabilities, sum
-    #pragma unroll
+            // ---- phase 2, one wave per head: tile maximum, rescale factor, probabilities and their sum; the weights
+            //      w = p * v_scale of the tile as two INT8 limbs, w ~ wscale (a1 + a2 / 254)
+#pragma unroll
             for (int j = 0; j < OWN; j++) {
                 const int h = wave + 4 * j;
                 if (h < RATIO) {                                     // wave-uniform
                     float* ph = ps + h * ATT_TILE;
                     float sc[ATT_TILE / 64];
                     float tmax = -1e30f;
-    #pragma unroll
+#pragma unroll
                     for (int i = 0; i < ATT_TILE / 64; i++) {
                         const int t = lane + 64 * i;
                         sc[i] = t < tl ? ph[t] : -1e30f;
@@ -719,58 +775,84 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
                     tmax = wave_max(tmax);
                     const float m_new = fmaxf(m_run[j], tmax);
                     const float corr = expf(m_run[j] - m_new);
-                    float psum = 0.0f;
-    #pragma unroll
+                    float psum = 0.0f, wv[ATT_TILE / 64], wmax = 0.0f;
+#pragma unroll
                     for (int i = 0; i < ATT_TILE / 64; i++) {
                         const int t = lane + 64 * i;
                         const float pv = t < tl ? expf(sc[i] - m_new) : 0.0f;
-                        if (t < tl) ph[t] = pv;
                         psum += pv;
+                        wv[i] = pv * vsc[j][i];
+                        wmax = fmaxf(wmax, wv[i]);
                     }
                     psum = t12_wave_sum(psum);
+                    wmax = wave_max(wmax);
+                    const float inv = wmax > 0.0f ? 127.0f / wmax : 0.0f;
+#pragma unroll
+                    for (int i = 0; i < ATT_TILE / 64; i++) {
+                        const int t = lane + 64 * i;
+                        const float r0 = wv[i] * inv;
+                        const float a1 = fminf(rintf(r0), 127.0f);
+                        const float a2 = fminf(fmaxf(rintf((r0 - a1) * 254.0f), -127.0f), 127.0f);
+                        wq[h * WSTR + t] = (int8_t)(int)a1;
+                        wq[(8 + h) * WSTR + t] = (int8_t)(int)a2;
+                    }
                     l_run[j] = l_run[j] * corr + psum;
                     m_run[j] = m_new;
-                    if (lane == 0) corr_s[h] = corr;
+                    if (lane == 0) {
+                        corr_s[h] = corr;
+                        wscale_s[h] = wmax / 127.0f;
+                    }
                 }
             }
             __syncthreads();
-            // ---- phase 3, one wave per 64 positions: every V value is converted once and used for all heads
-            int tl_opaque = tl;
-            asm volatile("" : "+s"(tl_opaque));
-    #pragma unroll
-            for (int h = 0; h < RATIO; h++) {
-                const float corr = corr_s[h];
-    #pragma unroll
-                for (int e = 0; e < 16; e++) acc[h][e] *= corr;
-            }
-            if (v_any) {
-    #pragma unroll
-                for (int x = 0; x < NIT; x++) {
-                    // every row is a basic block of its own (the condition always holds, but only at run time):
-                    // the compiler schedules inside basic blocks, and left to itself it converts all prefetched
-                    // rows first and keeps 16 floats per row alive (> 300 VGPRs)
-                    if (tl_opaque < 0) continue;
-                    const int tp = wave * 64 + x * PG + g;
-                    const bool ok = tp < tl;
-                    const int tc = min(tp, tl - 1);
-                    uint4 v4 = vv[x];
-                    float vscale = vsc[x];
-                    if (v_lds) {
-                        v4 = ((const uint4*)vt)[tc * CH + c];
-                        vscale = vts[tc];
+            // ---- phase 3: two halves of 128 positions = 4 MFMA steps of 32 positions each
+            t12_i32x16 oacc;
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[r] = 0;
+            const int s16 = lane & 15;
+            // transposed read: lane s16 = 2 j + par points at row j (a position), 8 dims from 8 par on, of its 16-dim group
+            const int8_t* vsrc = vth + (s16 >> 1) * VSTR + wave * 32 + ((lane >> 4) & 1) * 16 + (s16 & 1) * 8;
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+                if (half * 128 < tl) {                               // workgroup-uniform
+                    if (half == 1) {
+                        // second half of the tile through the same LDS rows
+                        __syncthreads();                             // every wave is done with the first half
+#pragma unroll
+                        for (int x = 0; x < VP; x++) {
+                            const int idx = tid + 256 * x;
+                            *(t12_u32x4*)(vth + (idx / CH) * VSTR + (idx % CH) * 16) = vreg[x];
+                        }
+                        if (has_next) issue_v(t0n, tln, 0);           // the next tile's first 128 V rows
+                        __syncthreads();
                     }
-                    const uint32_t w4[4] = {v4.x, v4.y, v4.z, v4.w};
-                    float fv[16];
-    #pragma unroll
-                    for (int e = 0; e < 16; e++) fv[e] = (float)(int8_t)((w4[e >> 2] >> (8 * (e & 3))) & 0xFF);
-    #pragma unroll
-                    for (int h = 0; h < RATIO; h++) {
-                        const float w = ok ? ps[h * ATT_TILE + tc] * vscale : 0.0f;
-    #pragma unroll
-                        for (int e = 0; e < 16; e++) acc[h][e] += w * fv[e];
+                    if (wave < NBLK) {
+#pragma unroll
+                        for (int ks = 0; ks < 4; ks++) {
+                            const t12_i32x4 wa = *(const t12_i32x4*)(wq + ln * WSTR + half * 128 + ks * 32 + 16 * lh);
+                            typedef int t12_i32x2 __attribute__((ext_vector_type(2)));
+                            typedef __attribute__((address_space(3))) t12_i32x2 lds_i32x2;
+                            const t12_i32x2 b0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                                (lds_i32x2*)(vsrc + (ks * 32 + 16 * lh) * VSTR));
+                            const t12_i32x2 b1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                                (lds_i32x2*)(vsrc + (ks * 32 + 16 * lh + 8) * VSTR));
+                            t12_i32x4 vb;
+                            vb[0] = b0[0]; vb[1] = b0[1]; vb[2] = b1[0]; vb[3] = b1[1];
+                            oacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa, vb, oacc, 0, 0, 0);
+                        }
                     }
                 }
             }
+            // lane (ln, lh): column = dim 32 wave + ln; rows 4 lh + r (limb 0) and 8 + 4 lh + r (limb 1) = heads 4 lh + r
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int h = min(4 * lh + r, RATIO - 1);
+                o_w[r] = o_w[r] * corr_s[h] + ((float)oacc[r] + (float)oacc[4 + r] * (1.0f / 254.0f)) * wscale_s[h];
+            }
+#pragma unroll
+            for (int j = 0; j < OWN; j++)
+#pragma unroll
+                for (int i = 0; i < ATT_TILE / 64; i++) vsc[j][i] = vsc_n[j][i];
             __syncthreads();
         } else {
             __syncthreads();
@@ -835,26 +917,9 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
         }
     }
     if constexpr (WIDE) {
-        // ---- fold: position classes inside a wave, then the four waves through LDS
-        __shared__ __attribute__((aligned(16))) float red[4 * RATIO * HD];
+        // ---- every lane holds finished sums of its dim for up to four heads; the owners publish maximum and sum
         __shared__ float mstat[RATIO], lstat[RATIO];
-    #pragma unroll
-        for (int h = 0; h < RATIO; h++) {
-    #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                float v = acc[h][e];
-    #pragma unroll
-                for (int off = CH; off < 64; off <<= 1) v += __shfl_xor(v, off, T12_WAVE);
-                acc[h][e] = v;
-            }
-            if (g == 0) {
-    #pragma unroll
-                for (int e = 0; e < 16; e += 4)
-                    *(float4*)(red + ((size_t)wave * RATIO + h) * HD + c * 16 + e) =
-                        make_float4(acc[h][e], acc[h][e + 1], acc[h][e + 2], acc[h][e + 3]);
-            }
-        }
-    #pragma unroll
+#pragma unroll
         for (int j = 0; j < OWN; j++) {
             const int h = wave + 4 * j;
             if (h < RATIO && lane == 0) {
@@ -863,26 +928,23 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
             }
         }
         __syncthreads();
-        for (int i = tid; i < RATIO * HD / 4; i += 256) {
-            const int h = i / (HD / 4), d = (i % (HD / 4)) * 4;
-            float4 a = *(const float4*)(red + (size_t)h * HD + d);
-    #pragma unroll
-            for (int w = 1; w < 4; w++) {
-                const float4 o = *(const float4*)(red + ((size_t)w * RATIO + h) * HD + d);
-                a.x += o.x; a.y += o.y; a.z += o.z; a.w += o.w;
-            }
-            if (SPLIT) {
-                float* pw = sp.ws + ((((size_t)b * n_head_kv + kvh) * nchunk + blockIdx.z) * RATIO + h) * (HD + 4);
-                *(float4*)(pw + d) = a;
-                if (d == 0) {
-                    pw[HD] = mstat[h];
-                    pw[HD + 1] = lstat[h];
+        if (wave < NBLK) {
+            const int d = wave * 32 + ln;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int h = 4 * lh + r;
+                if (h < RATIO) {
+                    if (SPLIT) {
+                        float* pw = sp.ws + ((((size_t)b * n_head_kv + kvh) * nchunk + blockIdx.z) * RATIO + h) * (HD + 4);
+                        pw[d] = o_w[r];
+                        if (d == 0) {
+                            pw[HD] = mstat[h];
+                            pw[HD + 1] = lstat[h];
+                        }
+                    } else {
+                        out[(size_t)b * n_head * HD + (size_t)(kvh * RATIO + h) * HD + d] = t12_f32_to_bf16(o_w[r] / lstat[h]);
+                    }
                 }
-            } else {
-                const float inv = 1.0f / lstat[h];
-                *(uint2*)(out + (size_t)b * n_head * HD + (size_t)(kvh * RATIO + h) * HD + d) =
-                    make_uint2(t12_f32_to_bf16(a.x * inv) | ((uint32_t)t12_f32_to_bf16(a.y * inv) << 16),
-                               t12_f32_to_bf16(a.z * inv) | ((uint32_t)t12_f32_to_bf16(a.w * inv) << 16));
             }
         }
     } else {
