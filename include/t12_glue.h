@@ -125,13 +125,13 @@ void launch_rope_store_attention_partials(float* q, float* k, const float* v, in
                                           size_t split_stride, int ld, int kv_stride, hipStream_t stream);
 
 /* Benchmark switch.  0: always the general attention kernel.  1 (default): shapes with a specialised kernel
- * (head_dim 128 with GQA ratio 1/2/4/8, head_dim 64 with ratio 1/4) use it, and a launch without a position array
- * whose batch * n_head_kv workgroups would leave the chip idle is split along the context into chunks of at
- * least 256 positions (partial softmax per chunk, folded by the workgroup that finishes last; the partial results
- * live in a library-owned buffer, so two such launches on different streams must not overlap); from 320
- * positions on (the length argument, a hint when a position array is given) the kernel takes its long-context
- * form: scores by INT8 MFMAs, P.V with one wave per 64 positions.  2: specialised kernels, never split.  3: never the long-context form.  4: always.  n >= 16:
- * specialised kernels, chunks of at least n positions. */
+ * (head_dim 128 with GQA ratio 1/2/4/8, head_dim 64 with ratio 1/4) use it in its INT8 MFMA form (scores and P.V by
+ * v_mfma_i32_32x32x32_i8: Q and the softmax weights in two INT8 limbs, K and V as stored), and a launch without a
+ * position array whose batch * n_head_kv workgroups would leave the chip idle is split along the context into
+ * chunks of at least 256 positions (partial softmax per chunk, folded by the workgroup that finishes last; the
+ * partial results live in a library-owned buffer, so two such launches on different streams must not overlap).
+ * 2: never split.  3: the specialised kernels in their fp32 FMA form.  4: same as 1.  n >= 16: chunks of at least n
+ * positions. */
 int t12_tune_attention(int mode);
 
 #ifdef __cplusplus

@@ -1167,7 +1167,7 @@ void launch_rope_kv(float* q, float* k, const float* v, int8_t* ck, int8_t* cv, 
 
 int g_attn_fast = 1;   // 0: always the general kernel (tests compare the two)
 int g_attn_chunk = 256; // context split: fewest positions per chunk; 0 = never split
-int g_attn_wide = 320;  // contexts from this length on take the form with INT8 MFMA scores and one wave per 64 positions
+int g_attn_wide = 0;    // contexts from this length on take the INT8 MFMA form (measured faster at every length)
 
 // Scratch of the context split: partial results of at most ATT_SPLIT_WGS workgroups and one
 // counter per (sequence, KV head); the counters start at zero and every launch leaves them there.
@@ -1224,13 +1224,12 @@ void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float
             sp.counter = g_split_cnt;
         }
     }
-    // Two forms of the kernel.  Short contexts: scores by fp32 FMAs with one thread per position, P.V with one
-    // wave per head -- few registers, four workgroups per CU, no set-up: a workgroup is a chain of latencies that
-    // only occupancy hides.  Long contexts: scores by INT8 MFMAs (Q split into two INT8 limbs, K used as stored),
-    // P.V with one wave per 64 positions, every V value converted once for all heads and requested before the
-    // softmax phase -- the kernel is bound by conversions and FMAs there.  seq_len is the caller's hint when
-    // positions are given.  Measured on per-sequence caches, B = 256: equal at 300 positions, 1.5x at 2000
-    // (503 -> 305 us for 1.08 GB), 2.5x for B = 64 at 8000.
+    // Two forms of the kernel.  First form: scores by fp32 FMAs with one thread per position, P.V with one wave per
+    // head (few registers, no set-up).  Second form: both products by INT8 MFMAs (Q and the softmax weights split
+    // into two INT8 limbs, K used as stored, V read transposed out of LDS), requests one tile ahead.  Measured on
+    // per-sequence caches the second is faster at every length (B = 256: 28 against 38 us at 150 positions, 259
+    // against 501 us at 2000; B = 1 at 150 positions: 7.0 against 10.3 us), so it is the default; the first stays
+    // selectable (t12_tune_attention(3)) and is what the tests compare it with.
     const bool wide = seq_len >= g_attn_wide;
 #define T12_ATT_GO(HD_, R_, F_, S_, W_)                                                                         \
     hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, F_, S_, W_>), dim3(n_head_kv, batch, S_ ? nchunk : 1), dim3(256), 0, \
@@ -1309,14 +1308,14 @@ void launch_rope_scaling(float factor, float low_freq_factor, float high_freq_fa
     g_rope_scale[3] = original_ctx;
 }
 
-// 0: always the general kernel; 1 (default): shapes with a specialised kernel use it, one sequence at a long
-// context split into chunks of at least 256 positions, the form with INT8 MFMA scores and one wave per 64 positions in the P.V phase from 320 positions;
-// 2: specialised kernels, never split; 3: never that P.V phase; 4: always; n >= 16: chunks of at least n positions.
+// 0: always the general kernel; 1 (default): shapes with a specialised kernel use it in its INT8 MFMA form, one
+// sequence at a long context split into chunks of at least 256 positions; 2: never split; 3: the specialised
+// kernels in their fp32 FMA form (one wave per head); 4: same as 1; n >= 16: chunks of at least n positions.
 int t12_tune_attention(int mode)
 {
     g_attn_fast = mode != 0;
     g_attn_chunk = mode >= 16 ? mode : (mode == 2 ? 0 : 256);
-    g_attn_wide = mode == 3 ? 0x7FFFFFFF : (mode == 4 ? 0 : 320);
+    g_attn_wide = mode == 3 ? 0x7FFFFFFF : 0;
     return 0;
 }
 
