@@ -126,7 +126,7 @@ void launch_rope_store_attention_partials(float* q, float* k, const float* v, in
 
 /* Benchmark switch.  0: always the general attention kernel.  1 (default): shapes with a specialised kernel
  * (head_dim 128 with GQA ratio 1/2/4/8, head_dim 64 with ratio 1/4) use it in its INT8 MFMA form (scores and P.V by
- * v_mfma_i32_32x32x32_i8: Q and the softmax weights in two INT8 limbs, K and V as stored), and a launch without a
+ * v_mfma_i32_32x32x32_i8: Q in three INT8 limbs, the softmax weights in two, K and V as stored), and a launch without a
  * position array whose batch * n_head_kv workgroups would leave the chip idle is split along the context into
  * chunks of at least 256 positions (partial softmax per chunk, folded by the workgroup that finishes last; the
  * partial results live in a library-owned buffer, so two such launches on different streams must not overlap).

@@ -563,8 +563,9 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
     }
     __syncthreads();
 
-    // Q as two INT8 limbs per element, q ~ s_h (a1 + a2 / 254) with s_h = max|q_h| / 127 (error <= 1.6e-5 max|q_h|,
-    // below what the bf16 output resolves), laid out as the A operand of the score MFMAs: row 8 * limb + h.
+    // Q as three INT8 limbs per element, q ~ s_h (a1 + a2 / 254 + a3 / 254^2) with s_h = max|q_h| / 127 (error <=
+    // 6e-8 max|q_h|: fp32 level, also for heads with outlier dims), laid out as the A operand of the score MFMAs: row
+    // 8 * limb + h (the 32 rows of the MFMA are there anyway).
     // INT8 x INT8 products accumulate exactly in int32, so K needs no conversion at all.
     constexpr int QSTR = HD + 16;               // row pitch of qlimb, for the same reason as WSTR
     __shared__ __attribute__((aligned(16))) int8_t qlimb[WIDE ? 32 * QSTR : 16];
@@ -580,9 +581,12 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
         for (int d = lane; d < HD; d += 64) {
             const float r0 = qs[h * HD + d] * inv;
             const float a1 = fminf(fmaxf(rintf(r0), -127.0f), 127.0f);
-            const float a2 = fminf(fmaxf(rintf((r0 - a1) * 254.0f), -127.0f), 127.0f);
+            const float r1 = (r0 - a1) * 254.0f;
+            const float a2 = fminf(fmaxf(rintf(r1), -127.0f), 127.0f);
+            const float a3 = fminf(fmaxf(rintf((r1 - a2) * 254.0f), -127.0f), 127.0f);
             qlimb[h * QSTR + d] = (int8_t)(int)a1;
             qlimb[(8 + h) * QSTR + d] = (int8_t)(int)a2;
+            qlimb[(16 + h) * QSTR + d] = (int8_t)(int)a3;
         }
         if (lane == 0) qscale[h] = amax / 127.0f;
     }
@@ -694,13 +698,14 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
                 for (int u = 0; u < KS; u++)
                     sacc = __builtin_amdgcn_mfma_i32_32x32x32_i8(*(const t12_i32x4*)(qa_src + 16 * u),
                                                                  __builtin_bit_cast(t12_i32x4, kk[nb][u]), sacc, 0, 0, 0);
-                // lane (ln, lh) holds column ln = its position; rows 4 lh + r (limb 0) and 8 + 4 lh + r (limb 1),
-                // r = 0..3: heads 4 lh .. 4 lh + 3
+                // lane (ln, lh) holds column ln = its position; rows 4 lh + r (limb 0), 8 + 4 lh + r (limb 1) and
+                // 16 + 4 lh + r (limb 2), r = 0..3: heads 4 lh .. 4 lh + 3
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const int h = 4 * lh + r;
                     if (h < RATIO)
-                        ps[h * ATT_TILE + tp] = ((float)sacc[r] + (float)sacc[4 + r] * (1.0f / 254.0f)) * (qscale[h] * kscale[nb]);
+                        ps[h * ATT_TILE + tp] = ((float)sacc[r] + ((float)sacc[4 + r] + (float)sacc[8 + r] * (1.0f / 254.0f)) *
+                                                                      (1.0f / 254.0f)) * (qscale[h] * kscale[nb]);
                 }
             }
         }
@@ -1225,8 +1230,8 @@ void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float
         }
     }
     // Two forms of the kernel.  First form: scores by fp32 FMAs with one thread per position, P.V with one wave per
-    // head (few registers, no set-up).  Second form: both products by INT8 MFMAs (Q and the softmax weights split
-    // into two INT8 limbs, K used as stored, V read transposed out of LDS), requests one tile ahead.  Measured on
+    // head (few registers, no set-up).  Second form: both products by INT8 MFMAs (Q split into three INT8 limbs, the softmax
+    // weights into two, K used as stored, V read transposed out of LDS), requests one tile ahead.  Measured on
     // per-sequence caches the second is faster at every length (B = 256: 28 against 38 us at 150 positions, 259
     // against 501 us at 2000; B = 1 at 150 positions: 7.0 against 10.3 us), so it is the default; the first stays
     // selectable (t12_tune_attention(3)) and is what the tests compare it with.
