@@ -383,14 +383,23 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
 }
 
 // ---- fast decode attention for the common shapes (head_dim 64 / 128, GQA ratio 1/2/4/8) ----
-// Same function as attn_decode_kernel; compile-time shapes let every loop unroll:
+// Same function as attn_decode_kernel, per tile of 256 positions, in one of two forms.
+// WIDE = true (the default), both products on the matrix cores with INT8 operands:
+//   phase 1  Q split into three INT8 limbs per element (rows 8 * limb + head of the A operand), K rows
+//            as stored = B operand; v_mfma_i32_32x32x32_i8, exact int32 sums, 64 positions per wave;
+//   phase 2  one wave per query head: tile max, exp, sum with wave reductions only; the weights
+//            p * v_scale of the tile go to LDS as two INT8 limbs;
+//   phase 3  out[head, dim] += w . V: V staged 128 positions at a time in LDS and read back
+//            transposed (ds_read_b64_tr_b8), one wave per 32 dims, again v_mfma_i32_32x32x32_i8;
+//   every tile's K rows, V rows and scales are requested one tile ahead.
+// WIDE = false, the first form, kept for comparison (t12_tune_attention(3)):
 //   phase 1  lane = position: the K row is fetched with HD/16 128-bit loads issued together,
-//            then dotted with the RATIO query vectors broadcast from LDS;
-//   phase 2  one wave per query head: tile max, exp, sum with wave reductions only
-//            (running max / sum are wave-uniform registers);
+//            then dotted with the RATIO query vectors broadcast from LDS (fp32 FMAs);
+//   phase 2  as above, without the limbs;
 //   phase 3  the same wave: P.V with 128-bit V loads -- 8 (HD=128) or 4 (HD=64) lanes span one
 //            position, so one load instruction covers 8 / 16 positions; each lane keeps 16
 //            output dims for its position class, classes are folded by xor shuffles at the end.
+// SPLIT: see AttnSplit.
 // FUSE: the kernel first does what rope_kv_kernel<3> does for its own heads -- rotates the
 // RATIO query heads while loading them, rotates this KV head's new K, quantises K and V to
 // INT8 and stores them at position pos -- and only then attends over positions 0..pos.
