@@ -54,6 +54,29 @@ int   t12_engine_decode(void* state, int max_tokens, int stop_on_eos, int* out);
  * for max_tokens * batch ints, may be NULL); returns the number of steps. */
 int   t12_engine_decode_all(void* state, int max_tokens, int* out);
 
+/* shift_context: cache rows [discard, current_pos) of sequence seq -> rows [0, current_pos - discard), all layers,
+ * K, V and scales (the reference does this inline, engine/main.cpp:147-173). */
+int   t12_engine_shift_context(void* state, int seq, int current_pos, int discard);
+/* chat_turn: one turn of the reference's interactive loop (engine/main.cpp:139-213) on a batch-1 state: drops a
+ * leading BOS after the first turn, shifts the context when it is too long, enters the n_tokens ids at *current_pos,
+ * generates up to max_tokens ids until eos_id / bos_id (into out, room for max_tokens), feeds eos_id, advances
+ * *current_pos; *discarded (may be NULL) = cache rows dropped by the shift.  Returns the number generated. */
+int   t12_engine_chat_turn(void* state, int* current_pos, const int* tokens, int n_tokens, int max_tokens, int bos_id,
+                           int eos_id, int* discarded, int* out);
+
+/* ---- tokenizer: C face of include/turbo/tokenizer.h (the reference's engine/tokenizer.h:19-23), host only ---- */
+void* t12_tokenizer_load(const char* model_dir);                      /* load_tokenizer; NULL without vocab.bin + merges.bin */
+void  t12_tokenizer_free(void* tok);                                  /* free_tokenizer */
+int   t12_tokenizer_info(void* tok, int* bos_id, int* eos_id, int* vocab_size);
+/* Adds to Tokenizer::special_tokens (kept longest first, engine/tokenizer.cpp:136-140): the text is cut out of
+ * inputs before encoding and becomes `id` (engine/tokenizer.cpp:366-425). */
+int   t12_tokenizer_add_special(void* tok, const char* text, int id);
+/* tokenize (BOS first, engine/tokenizer.cpp:427-431): writes at most cap ids, returns how many the text has. */
+int   t12_tokenizer_encode(void* tok, const char* text, size_t len, int* ids_out, int cap);
+/* detokenize / detokenize_one (engine/tokenizer.cpp:433-506): write at most cap bytes (no terminator), return the length. */
+int   t12_tokenizer_decode(void* tok, const int* ids, int n, char* out, size_t cap);
+int   t12_tokenizer_decode_one(void* tok, int id, char* out, size_t cap);
+
 /* Synthetic tensors on the device (what create_synthetic_model is built from). */
 int   t12_synth_normal_bf16(void* out_bf16, size_t n, uint64_t seed, float sigma, float p_outlier, float sigma_outlier,
                             void* stream);

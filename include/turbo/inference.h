@@ -1,6 +1,7 @@
 // Decode loop of the split-12 engine: the reference's engine/inference.h API
 // (InferenceState, create/free, forward, generate -- engine/inference.h:5-55).
 #pragma once
+#include <functional>
 #include "model.h"
 
 struct InferenceState {
@@ -72,3 +73,21 @@ std::vector<int> decode_greedy(InferenceState* state, int max_tokens, bool stop_
 
 // decode_greedy without the stop rule, returning every sequence's ids: element [t * batch_size + b].
 std::vector<int> decode_greedy_all(InferenceState* state, int max_tokens);
+
+// Extension: the context shift of the reference's interactive loop (engine/main.cpp:147-173) as a function.  The
+// cache rows [discard, current_pos) of sequence `seq`, all layers, move to rows [0, current_pos - discard): int8 K
+// and V as stored -- keys keep the rotation of the positions they were written at, as in the reference -- and
+// their scales.  Enqueued on state->stream; the caller continues at position current_pos - discard.  On a state
+// that shares the model's one region `seq` only has to be a valid row.
+void shift_context(InferenceState* state, int seq, int current_pos, int discard);
+
+// Extension: one turn of the reference's interactive loop (engine/main.cpp:139-213) for a state of batch size 1.
+// turn_tokens = tokenize(line) (BOS first; dropped unless *current_pos == 0); when *current_pos + |tokens| +
+// max_tokens + 64 exceeds the cache, or *current_pos > 1024, the older half of the context is discarded first
+// (shift_context; *discarded receives the count).  Then the new tokens enter at *current_pos, up to max_tokens
+// greedy tokens follow until eos_id or bos_id is sampled (neither is returned), and eos_id (2 when eos_id <= 0)
+// is fed so that the context records the end of the turn.  *current_pos is advanced past all of it.  on_token
+// (optional) receives every generated id as soon as the host has it.
+std::vector<int> chat_turn(InferenceState* state, int* current_pos, const std::vector<int>& turn_tokens, int max_tokens,
+                           int bos_id, int eos_id, int* discarded = nullptr,
+                           const std::function<void(int)>& on_token = nullptr);

@@ -65,7 +65,8 @@ def test_cpp_api_symbols_present():
     out = subprocess.run(["nm", "-D", "--defined-only", LIB], capture_output=True, text=True).stdout
     for ident in ["load_model", "free_model", "create_inference_state", "free_inference_state", "forward",
                   "generate", "init_sampler", "sample_greedy", "sample_greedy_batch", "create_synthetic_model",
-                  "save_model"]:
+                  "save_model", "prefill", "shift_context", "chat_turn",
+                  "load_tokenizer", "free_tokenizer", "tokenize", "detokenize", "detokenize_one"]:   # engine/tokenizer.h:19-23
         assert re.search(r"_Z\d+%s" % ident, out), ident
 
 

@@ -98,6 +98,16 @@ _SIGS = {
     "t12_engine_generate": (_i, [_vp, C.POINTER(C.c_int), _i, _i, C.POINTER(C.c_int)]),
     "t12_engine_decode": (_i, [_vp, _i, _i, C.POINTER(C.c_int)]),
     "t12_engine_sync": (_i, [_vp]),
+    "t12_engine_shift_context": (_i, [_vp, _i, _i, _i]),
+    "t12_engine_chat_turn": (_i, [_vp, C.POINTER(C.c_int), C.POINTER(C.c_int), _i, _i, _i, _i, C.POINTER(C.c_int),
+                                  C.POINTER(C.c_int)]),
+    "t12_tokenizer_load": (_vp, [C.c_char_p]),
+    "t12_tokenizer_free": (None, [_vp]),
+    "t12_tokenizer_info": (_i, [_vp, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "t12_tokenizer_add_special": (_i, [_vp, C.c_char_p, _i]),
+    "t12_tokenizer_encode": (_i, [_vp, C.c_char_p, C.c_size_t, C.POINTER(C.c_int), _i]),
+    "t12_tokenizer_decode": (_i, [_vp, C.POINTER(C.c_int), _i, C.c_char_p, C.c_size_t]),
+    "t12_tokenizer_decode_one": (_i, [_vp, _i, C.c_char_p, C.c_size_t]),
     "t12_engine_weight": (_i, [_vp, _i, _i, C.POINTER(Segment), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "t12_gemv_add": (_i, [C.POINTER(Segment), _vp, _i, _vp, _vp]),
     "t12_gemv_swiglu": (_i, [C.POINTER(Segment), C.POINTER(Segment), _vp, _i, _vp, _vp]),
@@ -364,6 +374,19 @@ class Engine:
         n = lib.t12_engine_decode(self.state, max_tokens, int(stop_on_eos), out)
         return list(out[:n])
 
+    def shift_context(self, current_pos, discard, seq=0):
+        """Cache rows [discard, current_pos) of sequence seq move to the front (engine/main.cpp:147-173)."""
+        check(lib.t12_engine_shift_context(self.state, int(seq), int(current_pos), int(discard)), "shift_context")
+
+    def chat_turn(self, current_pos, tokens, max_tokens, bos_id, eos_id):
+        """One interactive turn (engine/main.cpp:139-213) -> (generated ids, new current_pos, rows discarded)."""
+        pos, dropped = C.c_int(int(current_pos)), C.c_int(0)
+        arr = (C.c_int * max(len(tokens), 1))(*[int(t) for t in tokens])
+        out = (C.c_int * max(max_tokens, 1))()
+        n = lib.t12_engine_chat_turn(self.state, C.byref(pos), arr, len(tokens), int(max_tokens), int(bos_id), int(eos_id),
+                                     C.byref(dropped), out)
+        return list(out[:n]), pos.value, dropped.value
+
     def weight(self, layer, which):
         seg, K, P = Segment(), C.c_int(), C.c_int()
         check(lib.t12_engine_weight(self.model, layer, which, C.byref(seg), C.byref(K), C.byref(P)), "engine_weight")
@@ -388,3 +411,50 @@ def _hip_memcpy_d2d(dst, src, nbytes):
         _hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
         _hip.hipMemcpy.restype = C.c_int
     return _hip.hipMemcpy(dst, src, nbytes, 3)   # hipMemcpyDeviceToDevice
+
+
+class Tokenizer:
+    """The engine's byte-level BPE tokenizer (include/turbo/tokenizer.h) through its C face; text is bytes."""
+
+    def __init__(self, model_dir):
+        self.handle = lib.t12_tokenizer_load(os.fsencode(model_dir))
+        if not self.handle:
+            raise T12Error("no tokenizer in %s (vocab.bin + merges.bin)" % model_dir)
+        b, e, v = C.c_int(), C.c_int(), C.c_int()
+        lib.t12_tokenizer_info(self.handle, C.byref(b), C.byref(e), C.byref(v))
+        self.bos_id, self.eos_id, self.vocab_size = b.value, e.value, v.value
+
+    def add_special(self, text: bytes, tid: int):
+        check(lib.t12_tokenizer_add_special(self.handle, bytes(text), int(tid)), "add_special")
+
+    def tokenize(self, text) -> list:
+        data = text.encode("utf-8") if isinstance(text, str) else bytes(text)
+        cap = len(data) + 8
+        out = (C.c_int * cap)()
+        n = lib.t12_tokenizer_encode(self.handle, data, len(data), out, cap)
+        if n < 0:
+            raise T12Error("tokenize failed")
+        if n > cap:
+            out = (C.c_int * n)()
+            n = lib.t12_tokenizer_encode(self.handle, data, len(data), out, n)
+        return list(out[:n])
+
+    def _text(self, fn, *args) -> bytes:
+        n = fn(self.handle, *args, None, 0)
+        if n < 0:
+            raise T12Error("detokenize failed")
+        buf = C.create_string_buffer(max(n, 1))
+        fn(self.handle, *args, buf, n)
+        return buf.raw[:n]
+
+    def detokenize(self, ids) -> bytes:
+        arr = (C.c_int * max(len(ids), 1))(*[int(t) for t in ids])
+        return self._text(lib.t12_tokenizer_decode, arr, len(ids))
+
+    def detokenize_one(self, tid) -> bytes:
+        return self._text(lib.t12_tokenizer_decode_one, int(tid))
+
+    def close(self):
+        if self.handle:
+            lib.t12_tokenizer_free(self.handle)
+            self.handle = None

@@ -564,9 +564,13 @@ void prefill(InferenceState* state, int seq, const int* token_ids, int n_tokens)
 // 0 ends the stream when stop_on_eos): the one forward issued past an end-of-stream token is undone
 // by stepping the positions back.  TURBO_NO_PIPELINE=1 restores the reference's order.
 namespace {
-std::vector<int> decode_loop(InferenceState* state, int max_tokens, bool stop_on_eos, bool all_rows)
+// Sequence 0 sampling stop_a or stop_b (ids, -1 = none) ends the stream; on_token (may be empty) sees every id of
+// sequence 0 that is kept, as soon as the host has it.
+std::vector<int> decode_loop(InferenceState* state, int max_tokens, int stop_a, int stop_b, bool all_rows,
+                             const std::function<void(int)>& on_token)
 {
     std::vector<int> output;
+    auto is_stop = [&](int t) { return (stop_a >= 0 && t == stop_a) || (stop_b >= 0 && t == stop_b); };
     const int n_vocab = state->model->config.n_vocab;
     const int bs = state->batch_size;
     hipStream_t st = state->stream;
@@ -576,9 +580,10 @@ std::vector<int> decode_loop(InferenceState* state, int max_tokens, bool stop_on
         for (int t = 0; t < max_tokens; t++) {
             if (bs == 1) tokens[0] = sample_greedy(state->logits, n_vocab, st);
             else sample_greedy_batch(state->logits, tokens.data(), n_vocab, bs, st);
-            if (stop_on_eos && tokens[0] == 2) break;
+            if (is_stop(tokens[0])) break;
             if (all_rows) output.insert(output.end(), tokens.begin(), tokens.end());
             else output.push_back(tokens[0]);
+            if (on_token) on_token(tokens[0]);
             forward(state, tokens.data());
         }
         return output;
@@ -601,12 +606,13 @@ std::vector<int> decode_loop(InferenceState* state, int max_tokens, bool stop_on
         if (t + 1 < max_tokens) enqueue_sample((t + 1) & 1);
         check_gpu(hipEventSynchronize(impl->sampled[t & 1]), "hipEventSynchronize");
         const int tok = impl->h_tokens[t & 1][0];
-        if (stop_on_eos && tok == 2) {
+        if (is_stop(tok)) {
             for (int b = 0; b < bs; b++) state->positions[b]--;   // the forward on the end-of-stream id does not count
             break;
         }
         if (all_rows) output.insert(output.end(), impl->h_tokens[t & 1], impl->h_tokens[t & 1] + bs);
         else output.push_back(tok);
+        if (on_token) on_token(tok);
     }
     check_gpu(hipStreamSynchronize(st), "hipStreamSynchronize");
     return output;
@@ -615,12 +621,12 @@ std::vector<int> decode_loop(InferenceState* state, int max_tokens, bool stop_on
 
 std::vector<int> decode_greedy(InferenceState* state, int max_tokens, bool stop_on_eos)
 {
-    return decode_loop(state, max_tokens, stop_on_eos, false);
+    return decode_loop(state, max_tokens, stop_on_eos ? 2 : -1, -1, false, nullptr);
 }
 
 std::vector<int> decode_greedy_all(InferenceState* state, int max_tokens)
 {
-    return decode_loop(state, max_tokens, false, true);
+    return decode_loop(state, max_tokens, -1, -1, true, nullptr);
 }
 
 std::vector<int> generate(InferenceState* state, const std::vector<int>& prompt_tokens, int max_tokens)
@@ -635,4 +641,70 @@ std::vector<int> generate(InferenceState* state, const std::vector<int>& prompt_
         forward(state, tokens.data());
     }
     return decode_greedy(state, max_tokens, true);
+}
+
+// engine/main.cpp:147-173: the cache rows [discard, current_pos) of every layer move to [0, current_pos - discard),
+// keys as stored (rotated for their old positions), scales along.  The reference issues one copy per array
+// whose source and destination overlap whenever more than `discard` rows are kept; here the rows move in
+// pieces of at most `discard` rows, front to back on the state's stream, so no copy overlaps itself.
+void shift_context(InferenceState* state, int seq, int current_pos, int discard)
+{
+    const KvView kv = kv_view(state);
+    const ModelConfig& c = state->model->config;
+    const int hd = c.n_embd / c.n_head, nkv = c.n_head_kv, kv_dim = nkv * hd;
+    if (seq < 0 || seq >= state->batch_size || discard < 0 || discard > current_pos || current_pos > kv.max_seq) {
+        fprintf(stderr, "ERROR: shift_context(seq %d, current_pos %d, discard %d) outside the cache (%d sequences, %d positions)\n",
+                seq, current_pos, discard, state->batch_size, kv.max_seq);
+        exit(1);
+    }
+    const int keep = current_pos - discard;
+    if (discard == 0 || keep == 0) return;
+    const size_t seq_kv = (size_t)seq * kv.kv_stride, seq_sc = seq_kv / hd;
+    hipStream_t st = state->stream;
+    for (int layer = 0; layer < c.n_layer; layer++) {
+        int8_t* k = kv.k + layer * kv.layer_kv + seq_kv;
+        int8_t* v = kv.v + layer * kv.layer_kv + seq_kv;
+        float* sk = kv.sk + layer * kv.layer_sc + seq_sc;
+        float* sv = kv.sv + layer * kv.layer_sc + seq_sc;
+        for (int done = 0; done < keep; done += discard) {
+            const size_t rows = (size_t)std::min(discard, keep - done);
+            const size_t to = (size_t)done, from = (size_t)done + discard;
+            check_gpu(hipMemcpyAsync(k + to * kv_dim, k + from * kv_dim, rows * kv_dim, hipMemcpyDeviceToDevice, st), "shift K");
+            check_gpu(hipMemcpyAsync(v + to * kv_dim, v + from * kv_dim, rows * kv_dim, hipMemcpyDeviceToDevice, st), "shift V");
+            check_gpu(hipMemcpyAsync(sk + to * nkv, sk + from * nkv, rows * nkv * sizeof(float), hipMemcpyDeviceToDevice, st),
+                      "shift K scales");
+            check_gpu(hipMemcpyAsync(sv + to * nkv, sv + from * nkv, rows * nkv * sizeof(float), hipMemcpyDeviceToDevice, st),
+                      "shift V scales");
+        }
+    }
+}
+
+// One turn of the reference's interactive loop, engine/main.cpp:139-203, without its printing.
+std::vector<int> chat_turn(InferenceState* state, int* current_pos, const std::vector<int>& turn_tokens, int max_tokens,
+                           int bos_id, int eos_id, int* discarded, const std::function<void(int)>& on_token)
+{
+    if (discarded) *discarded = 0;
+    if (state->batch_size != 1) {
+        fprintf(stderr, "ERROR: chat_turn needs a state of batch size 1 (got %d)\n", state->batch_size);
+        exit(1);
+    }
+    std::vector<int> tokens = turn_tokens;
+    int pos = *current_pos;
+    if (pos > 0 && !tokens.empty() && tokens[0] == bos_id) tokens.erase(tokens.begin());   // BOS only opens the first turn (:141-143)
+    const int max_seq = kv_view(state).max_seq;
+    const int shift_limit = 1024;                                                            // :148
+    const int headroom = (int)tokens.size() + max_tokens + 64;
+    if (pos + headroom > max_seq || pos > shift_limit) {
+        const int discard = pos / 2;
+        shift_context(state, 0, pos, discard);
+        pos -= discard;
+        if (discarded) *discarded = discard;
+    }
+    state->positions[0] = pos;
+    prefill(state, 0, tokens.data(), (int)tokens.size());        // batch size 1: one forward per new token (:181-184)
+    std::vector<int> out = decode_loop(state, max_tokens, eos_id, bos_id, false, on_token);   // :192-202
+    const int eos_tok = eos_id > 0 ? eos_id : 2;                 // the turn's end enters the context (:207-213)
+    forward(state, &eos_tok);
+    *current_pos = state->positions[0];
+    return out;
 }
