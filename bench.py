@@ -25,6 +25,10 @@ Workloads (synthetic, seeded, random-init weights of the Llama-3.1-8B shape:
                   INT8 cache) with every sequence on its own cache region, at several (batch, context) points;
                   `roofline` prices the cache bytes of B = 256 at 2000 positions against the HBM peak.
 
+  tokenizer       host only: one step = encoding ~1 MB of text (150 000 words of a 4000-word list) with the engine's
+                  byte-level BPE tokenizer over the ~20 000 merges that build those words; `cpu_baseline` is the reference's rule restated literally (one pass over the
+                  text per merge) on a 4 KB sample of the same text.
+
   gemv_stack_b1   one step = every linear layer of one decode step at B = 1 through
                   the fused split-12 decode-GEMV: per layer QKV (3 segments, one
                   launch), O, gate+up (2 segments, one launch), down; then lm_head.
@@ -432,6 +436,67 @@ def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(16, 
     return out
 
 
+def run_tokenizer(args, t12):
+    """Encoding throughput of the tokenizer (host code, no GPU): seeded word list, the merge table that builds its
+    words, text of those words."""
+    import importlib
+    import random
+    import tempfile
+
+    tf = importlib.import_module(t12.__name__ + ".tokenizer_files")
+    rng = random.Random(1234)
+    letters = b"etaoinshrldcumwfgypbvk"
+    words = sorted({bytes(rng.choice(letters) for _ in range(rng.randint(2, 11))) for _ in range(4000)})
+    merges, seen = [], set()
+    for w in words:                          # a word is built left to right: (w0, w1), (w0w1, w2), ...
+        for i in range(1, len(w)):
+            pair = (w[:i], w[i:i + 1])
+            if pair not in seen:
+                seen.add(pair)
+                merges.append(pair)
+    rng.shuffle(merges)
+    merges.sort(key=lambda m: len(m[0]))     # every merge after the one that builds its left part
+    toks = [b"<unk>", b"<s>", b"</s>"] + sorted({bytes([c]) for c in letters + b" "} | {a + b for a, b in merges})
+    text = b" ".join(rng.choice(words) for _ in range(150000))
+    with tempfile.TemporaryDirectory() as d:
+        tf.write_files(d, toks, merges, 1, 2, None)
+        sys.stdout.flush()
+        keep = os.dup(1)                     # the loader reports on stdout, which carries the JSON line
+        os.dup2(2, 1)
+        try:
+            tok = t12.Tokenizer(d)
+        finally:
+            import ctypes
+            ctypes.CDLL(None).fflush(None)   # the C library's buffer, while descriptor 1 still points away
+            os.dup2(keep, 1)
+            os.close(keep)
+        steps = max(args.steps, 3)
+        for _ in range(max(args.warmup, 1)):
+            ids = tok.tokenize(text)
+        t0 = time.time()
+        for _ in range(steps):
+            ids = tok.tokenize(text)
+        dt = (time.time() - t0) / steps
+        cpu = None
+        if not args.no_cpu_baseline:
+            from oracle.tokenizer_oracle import RefTokenizer
+            ref = RefTokenizer(d)
+            sample = text[:4096]
+            t1 = time.time()
+            want = ref.tokenize(sample)
+            t_ref = time.time() - t1
+            assert tok.tokenize(sample) == want, "tokenizer differs from the reference rule"
+            cpu = {"value": len(sample) / t_ref / 1e6, "unit": "MB/s of text", "cores": 1, "kind": "port",
+                   "sample": "first 4 KB of the same text, same merge table, reference rule restated in Python "
+                             "(one pass over the text per merge; its cost grows with text length x merges)"}
+        tok.close()
+    return {"metric": "byte-level BPE encoding throughput (host)", "value": len(text) / dt / 1e6, "unit": "MB/s of text",
+            "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 1), "ms_per_step": dt * 1e3, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": "tokenizer: %d bytes of text, %d merges, %d ids out" % (len(text), len(merges), len(ids))},
+            "roofline": None, "cpu_baseline": cpu}
+
+
 def run_gemm_layers(args, t12, torch, dev):
     """The four Llama-3.1-8B linear-layer shapes through the fused decode+GEMM at B = 16, 64, 256 on three
     rotating weight copies; one step = the four layer GEMMs of one decoder layer at B = 256."""
@@ -482,7 +547,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="decode", choices=["decode", "gemv_stack_b1", "moe", "gemm_layers", "attention"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "gemv_stack_b1", "moe", "gemm_layers", "attention", "tokenizer"])
     ap.add_argument("--prompt", type=int, default=128)
     ap.add_argument("--no-batch256", dest="batch256", action="store_false")
     ap.add_argument("--layers", type=int, default=LLAMA8B["n_layer"], help="debug: fewer layers (invalid as a result)")
@@ -499,6 +564,9 @@ def main():
     import torch
     import __graft_entry__ as ge
     t12 = ge.load_package()
+    if args.workload == "tokenizer":
+        print(json.dumps(run_tokenizer(args, t12)))
+        return
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.workload == "decode":

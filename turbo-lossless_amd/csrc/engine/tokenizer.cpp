@@ -7,7 +7,6 @@
 #include <cstdio>
 #include <cstring>
 #include <fstream>
-#include <queue>
 #include <unordered_map>
 
 namespace {
@@ -139,25 +138,30 @@ std::vector<int> bpe_encode(const BpeModel* m, const std::string& text)
         int rank, pos, l, r;
     };
     auto later = [](const Cand& x, const Cand& y) { return x.rank != y.rank ? x.rank > y.rank : x.pos > y.pos; };
-    std::priority_queue<Cand, std::vector<Cand>, decltype(later)> queue(later);
-    auto offer = [&](int i, int after) {
+    std::vector<Cand> heap;                    // binary heap, earliest (rank, position) on top
+    heap.reserve((size_t)n);
+    auto offer = [&](int i, int after, bool sift) {
         const int j = next[i];
         if (j < 0) return;
         const int rank = m->rank_after(sym[i], sym[j], after);
-        if (rank >= 0) queue.push({rank, i, sym[i], sym[j]});
+        if (rank < 0) return;
+        heap.push_back({rank, i, sym[i], sym[j]});
+        if (sift) std::push_heap(heap.begin(), heap.end(), later);
     };
-    for (int i = 0; i + 1 < n; i++) offer(i, -1);
-    while (!queue.empty()) {
-        const Cand c = queue.top();
-        queue.pop();
+    for (int i = 0; i + 1 < n; i++) offer(i, -1, false);
+    std::make_heap(heap.begin(), heap.end(), later);
+    while (!heap.empty()) {
+        std::pop_heap(heap.begin(), heap.end(), later);
+        const Cand c = heap.back();
+        heap.pop_back();
         const int i = c.pos, j = next[i];
         if (sym[i] != c.l || j < 0 || sym[j] != c.r) continue;
         sym[i] = m->merges[c.rank].result;
         sym[j] = -1;
         next[i] = next[j];
         if (next[j] >= 0) prev[next[j]] = i;
-        if (prev[i] >= 0) offer(prev[i], c.rank);
-        offer(i, c.rank);
+        if (prev[i] >= 0) offer(prev[i], c.rank, true);
+        offer(i, c.rank, true);
     }
     std::vector<int> ids;
     for (int i = n > 0 ? 0 : -1; i >= 0; i = next[i]) ids.push_back(m->symbol_id[sym[i]]);
