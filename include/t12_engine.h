@@ -65,9 +65,12 @@ int   t12_engine_chat_turn(void* state, int* current_pos, const int* tokens, int
                            int eos_id, int* discarded, int* out);
 
 /* ---- tokenizer: C face of include/turbo/tokenizer.h (the reference's engine/tokenizer.h:19-23), host only ---- */
-void* t12_tokenizer_load(const char* model_dir);                      /* load_tokenizer; NULL without vocab.bin + merges.bin */
+void* t12_tokenizer_load(const char* model_dir);                      /* load_tokenizer; NULL without tokenizer.model or vocab.bin + merges.bin */
 void  t12_tokenizer_free(void* tok);                                  /* free_tokenizer */
 int   t12_tokenizer_info(void* tok, int* bos_id, int* eos_id, int* vocab_size);
+int   t12_tokenizer_type(void* tok);                                  /* Tokenizer::type: 0 sentencepiece model, 1 byte-level BPE tables */
+/* Tokenizer::special_tokens: returns their number; for 0 <= index < number also the text (NUL-terminated, cut to cap) and id. */
+int   t12_tokenizer_special(void* tok, int index, char* text_out, size_t cap, int* id_out);
 /* Adds to Tokenizer::special_tokens (kept longest first, engine/tokenizer.cpp:136-140): the text is cut out of
  * inputs before encoding and becomes `id` (engine/tokenizer.cpp:366-425). */
 int   t12_tokenizer_add_special(void* tok, const char* text, int id);

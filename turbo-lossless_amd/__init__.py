@@ -104,6 +104,8 @@ _SIGS = {
     "t12_tokenizer_load": (_vp, [C.c_char_p]),
     "t12_tokenizer_free": (None, [_vp]),
     "t12_tokenizer_info": (_i, [_vp, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "t12_tokenizer_type": (_i, [_vp]),
+    "t12_tokenizer_special": (_i, [_vp, _i, C.c_char_p, C.c_size_t, C.POINTER(C.c_int)]),
     "t12_tokenizer_add_special": (_i, [_vp, C.c_char_p, _i]),
     "t12_tokenizer_encode": (_i, [_vp, C.c_char_p, C.c_size_t, C.POINTER(C.c_int), _i]),
     "t12_tokenizer_decode": (_i, [_vp, C.POINTER(C.c_int), _i, C.c_char_p, C.c_size_t]),
@@ -414,15 +416,25 @@ def _hip_memcpy_d2d(dst, src, nbytes):
 
 
 class Tokenizer:
-    """The engine's byte-level BPE tokenizer (include/turbo/tokenizer.h) through its C face; text is bytes."""
+    """The engine's tokenizer (include/turbo/tokenizer.h: sentencepiece BPE model or byte-level BPE tables) through
+    its C face; text is bytes."""
 
     def __init__(self, model_dir):
         self.handle = lib.t12_tokenizer_load(os.fsencode(model_dir))
         if not self.handle:
-            raise T12Error("no tokenizer in %s (vocab.bin + merges.bin)" % model_dir)
+            raise T12Error("no tokenizer in %s (tokenizer.model, or vocab.bin + merges.bin)" % model_dir)
         b, e, v = C.c_int(), C.c_int(), C.c_int()
         lib.t12_tokenizer_info(self.handle, C.byref(b), C.byref(e), C.byref(v))
         self.bos_id, self.eos_id, self.vocab_size = b.value, e.value, v.value
+        self.type = lib.t12_tokenizer_type(self.handle)
+
+    def special_tokens(self) -> list:
+        """[(text bytes, id)] in matching order (longest first)."""
+        out, buf, tid = [], C.create_string_buffer(1024), C.c_int()
+        for i in range(lib.t12_tokenizer_special(self.handle, -1, None, 0, None)):
+            lib.t12_tokenizer_special(self.handle, i, buf, 1024, C.byref(tid))
+            out.append((buf.value, tid.value))
+        return out
 
     def add_special(self, text: bytes, tid: int):
         check(lib.t12_tokenizer_add_special(self.handle, bytes(text), int(tid)), "add_special")

@@ -1,12 +1,16 @@
-// Byte-level BPE tokenizer behind the reference's engine/tokenizer.h API (see include/turbo/tokenizer.h).
-// Host code only.
+// The two tokenizer backends behind the reference's engine/tokenizer.h API (see include/turbo/tokenizer.h):
+// sentencepiece BPE models (sp_model.cpp) and byte-level BPE tables (this file).  Host code only.
 #include "turbo/tokenizer.h"
+
+#include "sp_model.h"
 
 #include <algorithm>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <cstdlib>
 #include <fstream>
+#include <iterator>
 #include <unordered_map>
 
 namespace {
@@ -170,7 +174,66 @@ std::vector<int> bpe_encode(const BpeModel* m, const std::string& text)
 
 std::vector<int> encode_plain(Tokenizer* tok, const std::string& text)
 {
+    if (tok->type == 0) return ((const SpModel*)tok->sp_model)->encode(text);
     return bpe_encode((const BpeModel*)tok->sp_model, text);
+}
+
+// engine/tokenizer.cpp:50-59: the integer after "key": in a JSON fragment, -1 when the key is absent
+int json_int_after(const std::string& json, const std::string& key)
+{
+    size_t pos = json.find("\"" + key + "\"");
+    if (pos == std::string::npos) return -1;
+    pos = json.find(':', pos);
+    if (pos == std::string::npos) return -1;
+    pos++;
+    while (pos < json.size() && (json[pos] == ' ' || json[pos] == '\t')) pos++;
+    return atoi(json.c_str() + pos);
+}
+
+// engine/tokenizer.cpp:85-152, same reading of tokenizer.json, quirks included: every object of the "added_tokens"
+// array that contains the text "special" (quoted) and the text true anywhere counts as special; its "content" is
+// taken raw up to the next quote (no unescaping); ids <= 2 and one-character contents are left out; a content of
+// </s> moves eos_id.
+void load_special_tokens(Tokenizer* tok, const std::string& model_dir)
+{
+    std::ifstream f(model_dir + "/tokenizer.json");
+    if (!f) return;
+    const std::string json((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+    const size_t added = json.find("\"added_tokens\"");
+    if (added == std::string::npos) return;
+    const size_t open = json.find('[', added);
+    if (open == std::string::npos) return;
+    size_t pos = open + 1;
+    while (pos < json.size()) {
+        const size_t b = json.find('{', pos);
+        if (b == std::string::npos) break;
+        size_t e = b + 1;
+        bool in_str = false;
+        while (e < json.size()) {
+            if (json[e] == '"' && json[e - 1] != '\\') in_str = !in_str;
+            else if (!in_str && json[e] == '}') break;
+            e++;
+        }
+        if (e >= json.size()) break;
+        const std::string obj = json.substr(b, e - b + 1);
+        if (obj.find("\"special\"") != std::string::npos && obj.find("true") != std::string::npos) {
+            const int id = json_int_after(obj, "id");
+            size_t cs = obj.find("\"content\"");
+            if (cs != std::string::npos && (cs = obj.find('"', cs + 9)) != std::string::npos) {
+                const size_t ce = obj.find('"', cs + 1);
+                if (ce != std::string::npos) {
+                    const std::string content = obj.substr(cs + 1, ce - cs - 1);
+                    if (id > 2 && content.size() > 1) tok->special_tokens.push_back({content, id});
+                    if (content == "</s>" && id != tok->eos_id) tok->eos_id = id;
+                }
+            }
+        }
+        pos = e + 1;
+        const size_t nxt = json.find_first_not_of(" \t\n\r,", pos);
+        if (nxt != std::string::npos && json[nxt] == ']') break;
+    }
+    std::stable_sort(tok->special_tokens.begin(), tok->special_tokens.end(),
+                     [](const SpecialToken& a, const SpecialToken& b) { return a.text.size() > b.text.size(); });
 }
 
 // engine/tokenizer.cpp:366-425: special-token texts are cut out of the input (first the longest that matches at the
@@ -207,15 +270,29 @@ std::vector<int> encode_with_special(Tokenizer* tok, const std::string& text)
 
 Tokenizer* load_tokenizer(const std::string& model_path)
 {
+    // sentencepiece model first, like the reference (engine/tokenizer.cpp:332-346)
+    const std::string sp_path = model_path + "/tokenizer.model";
+    if (std::ifstream(sp_path, std::ios::binary)) {
+        auto* sp = new SpModel();
+        const std::string err = sp->load(sp_path);
+        if (err.empty()) {
+            auto* tok = new Tokenizer();
+            tok->sp_model = sp;
+            tok->bos_id = sp->bos_id;
+            tok->eos_id = sp->eos_id;
+            tok->vocab_size = (int)sp->pieces.size();
+            tok->type = 0;
+            printf("  Tokenizer: sentencepiece, vocab=%d bos=%d eos=%d\n", tok->vocab_size, tok->bos_id, tok->eos_id);
+            load_special_tokens(tok, model_path);
+            return tok;
+        }
+        fprintf(stderr, "tokenizer: %s: %s\n", sp_path.c_str(), err.c_str());
+        delete sp;
+    }
     int bos = 0, eos = 0;
     BpeModel* m = load_bpe(model_path, &bos, &eos);
     if (!m) {
-        std::ifstream sp(model_path + "/tokenizer.model", std::ios::binary);
-        if (sp)
-            fprintf(stderr, "No tokenizer loaded from %s: tokenizer.model is a sentencepiece model, which this build does "
-                            "not read (vocab.bin + merges.bin wanted)\n", model_path.c_str());
-        else
-            fprintf(stderr, "No tokenizer found in %s (vocab.bin + merges.bin wanted)\n", model_path.c_str());
+        fprintf(stderr, "No tokenizer found in %s (tried tokenizer.model, and vocab.bin + merges.bin)\n", model_path.c_str());
         return nullptr;
     }
     auto* tok = new Tokenizer();
@@ -231,7 +308,8 @@ Tokenizer* load_tokenizer(const std::string& model_path)
 void free_tokenizer(Tokenizer* tok)
 {
     if (!tok) return;
-    delete (BpeModel*)tok->sp_model;
+    if (tok->type == 0) delete (SpModel*)tok->sp_model;
+    else delete (BpeModel*)tok->sp_model;
     delete tok;
 }
 
@@ -244,6 +322,7 @@ std::vector<int> tokenize(Tokenizer* tok, const std::string& text)
 
 std::string detokenize(Tokenizer* tok, const std::vector<int>& tokens)
 {
+    if (tok->type == 0) return ((const SpModel*)tok->sp_model)->decode(tokens);
     const BpeModel* m = (const BpeModel*)tok->sp_model;
     std::string text;
     for (int id : tokens)
@@ -255,6 +334,29 @@ std::string detokenize_one(Tokenizer* tok, int token)
 {
     for (const SpecialToken& st : tok->special_tokens)
         if (st.id == token) return st.text;
+    if (tok->type == 0) {
+        // engine/tokenizer.cpp:484-506: the piece with every escaped blank as a space and a <0xXX> piece as its byte
+        const std::string& piece = ((const SpModel*)tok->sp_model)->id_to_piece(token);
+        std::string out;
+        size_t i = 0;
+        while (i < piece.size()) {
+            if (piece.compare(i, 3, "\xE2\x96\x81") == 0) {
+                out += ' ';
+                i += 3;
+            } else if (piece[i] == '<' && i + 5 < piece.size() && piece[i + 1] == '0' && piece[i + 2] == 'x') {
+                const size_t close = piece.find('>', i);
+                if (close != std::string::npos) {
+                    out += (char)strtol(piece.substr(i + 3, close - i - 3).c_str(), nullptr, 16);
+                    i = close + 1;
+                } else {
+                    out += piece[i++];
+                }
+            } else {
+                out += piece[i++];
+            }
+        }
+        return out;
+    }
     const BpeModel* m = (const BpeModel*)tok->sp_model;
     if (token < 0 || (size_t)token >= m->id_to_token.size()) return "";
     // engine/tokenizer.cpp:452-479: at every offset the longest (4..1 bytes) stretch that is a byte-encoder
@@ -293,6 +395,25 @@ int t12_tokenizer_info(void* tok, int* bos_id, int* eos_id, int* vocab_size)
     if (eos_id) *eos_id = t->eos_id;
     if (vocab_size) *vocab_size = t->vocab_size;
     return 0;
+}
+
+int t12_tokenizer_type(void* tok) { return tok ? ((Tokenizer*)tok)->type : -1; }
+
+// Number of special tokens; with index >= 0 also copies that token's text (at most cap bytes) and id.
+int t12_tokenizer_special(void* tok, int index, char* text_out, size_t cap, int* id_out)
+{
+    auto* t = (Tokenizer*)tok;
+    if (!t) return -1;
+    if (index >= 0 && index < (int)t->special_tokens.size()) {
+        const SpecialToken& st = t->special_tokens[index];
+        if (text_out && cap) {
+            const size_t n = std::min(cap - 1, st.text.size());
+            memcpy(text_out, st.text.data(), n);
+            text_out[n] = 0;
+        }
+        if (id_out) *id_out = st.id;
+    }
+    return (int)t->special_tokens.size();
 }
 
 // Appends to Tokenizer::special_tokens, keeping the list longest-first (stable), the order the reference
