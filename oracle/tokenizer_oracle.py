@@ -12,7 +12,8 @@ Only tests/ may import this file.  It follows engine/tokenizer.cpp line by line,
 Pinned by tests/test_tokenizer.py: on merge tables trained by the `tokenizers` library the encoder
 equals that library's BPE model (no pre-tokenizer); the byte table of `bytes_to_unicode`
 (engine/extract_tokenizer.py:12-22) equals the one `transformers` ships for GPT-2.  The reference's
-sentencepiece backend needs the sentencepiece C++ library and is not restated.
+sentencepiece backend (engine/tokenizer.cpp:12-29) is a call into the sentencepiece library and is not
+restated here: tests/test_tokenizer_sp.py checks the product against that library (its Python package).
 """
 import os
 import struct
