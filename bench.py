@@ -460,16 +460,7 @@ def run_tokenizer(args, t12):
     text = b" ".join(rng.choice(words) for _ in range(150000))
     with tempfile.TemporaryDirectory() as d:
         tf.write_files(d, toks, merges, 1, 2, None)
-        sys.stdout.flush()
-        keep = os.dup(1)                     # the loader reports on stdout, which carries the JSON line
-        os.dup2(2, 1)
-        try:
-            tok = t12.Tokenizer(d)
-        finally:
-            import ctypes
-            ctypes.CDLL(None).fflush(None)   # the C library's buffer, while descriptor 1 still points away
-            os.dup2(keep, 1)
-            os.close(keep)
+        tok = t12.Tokenizer(d)
         steps = max(args.steps, 3)
         for _ in range(max(args.warmup, 1)):
             ids = tok.tokenize(text)
@@ -542,6 +533,15 @@ def run_gemm_layers(args, t12, torch, dev):
     }
 
 
+def emit(result, json_fd):
+    """The ONE line of standard output.  Descriptor 1 was pointed at standard error for the whole run (the native
+    library reports model and cache sizes with printf); json_fd is the original descriptor 1."""
+    import ctypes
+    sys.stdout.flush()
+    ctypes.CDLL(None).fflush(None)           # the C library's own buffer, while descriptor 1 still points away
+    os.write(json_fd, (json.dumps(result) + "\n").encode())
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -561,25 +561,27 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
+    json_fd = os.dup(1)
+    os.dup2(2, 1)
     import torch
     import __graft_entry__ as ge
     t12 = ge.load_package()
     if args.workload == "tokenizer":
-        print(json.dumps(run_tokenizer(args, t12)))
+        emit(run_tokenizer(args, t12), json_fd)
         return
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.workload == "decode":
-        print(json.dumps(run_decode(args, t12, torch, dev)))
+        emit(run_decode(args, t12, torch, dev), json_fd)
         return
     if args.workload == "gemm_layers":
-        print(json.dumps(run_gemm_layers(args, t12, torch, dev)))
+        emit(run_gemm_layers(args, t12, torch, dev), json_fd)
         return
     if args.workload == "moe":
-        print(json.dumps(run_moe(args, t12, torch, dev)))
+        emit(run_moe(args, t12, torch, dev), json_fd)
         return
     if args.workload == "attention":
-        print(json.dumps(run_attention(args, t12, torch, dev)))
+        emit(run_attention(args, t12, torch, dev), json_fd)
         return
     cfg = dict(LLAMA8B, n_layer=args.layers)
 
@@ -650,7 +652,7 @@ def main():
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(torch, launches, cfg)
-    print(json.dumps(result))
+    emit(result, json_fd)
 
 
 if __name__ == "__main__":
