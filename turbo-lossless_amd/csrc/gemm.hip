@@ -35,6 +35,10 @@
 // Fast path requirements: K % 64 == 0, 0 <= base_exp <= 240, 16-byte aligned
 // activation rows.  Everything else goes to the general kernel below.
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "t12_device.h"
 #include "t12_host.h"
 
@@ -551,22 +555,29 @@ __global__ __launch_bounds__(256) void gemm_general_kernel(const GemmParams p)
     }
 }
 
-// ---- workspace for the K-split partial sums (grown on demand, per device) ----
-float* g_ws[16] = {};
-size_t g_ws_bytes[16] = {};
+// ---- workspace for the K-split partial sums: one per (device, stream), grown on demand.  Launches on different
+//      streams may overlap, so they must not share partial sums; launches on one stream are ordered.
+struct Workspace {
+    float* ptr;
+    size_t bytes;
+};
+std::mutex g_ws_mutex;
+std::map<std::pair<int, hipStream_t>, Workspace> g_ws;
 
-float* workspace(size_t bytes)
+float* workspace(size_t bytes, hipStream_t st)
 {
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
-    if (g_ws_bytes[dev] < bytes) {
-        if (g_ws[dev]) (void)hipFree(g_ws[dev]);
-        g_ws[dev] = nullptr;
-        g_ws_bytes[dev] = 0;
-        if (hipMalloc((void**)&g_ws[dev], bytes) != hipSuccess) return nullptr;
-        g_ws_bytes[dev] = bytes;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    Workspace& w = g_ws[{dev, st}];
+    if (w.bytes < bytes) {
+        if (w.ptr) (void)hipFree(w.ptr);          // waits for the device: nothing still reads the old buffer
+        w.ptr = nullptr;
+        w.bytes = 0;
+        if (hipMalloc((void**)&w.ptr, bytes) != hipSuccess) return nullptr;
+        w.bytes = bytes;
     }
-    return g_ws[dev];
+    return w.ptr;
 }
 
 int g_gemm_ksplit = 0;   // 0 = choose by shape
@@ -731,7 +742,7 @@ int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, in
     p.ksplit = ks;
     p.kslice = kslice;
     if (ks > 1) {
-        p.ws = workspace((size_t)ks * B * m_total * sizeof(float));
+        p.ws = workspace((size_t)ks * B * m_total * sizeof(float), st);
         if (!p.ws) {
             t12_set_error("t12_gemm: cannot allocate %zu bytes of K-split workspace",
                           (size_t)ks * B * m_total * sizeof(float));
