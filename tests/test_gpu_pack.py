@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from gpu_util import dev, to_dev_bits
+from gpu_util import to_dev_bits
 
 pytestmark = pytest.mark.gpu
 

@@ -3,7 +3,6 @@ engine/tokenizer.cpp:12-29,366-506, which calls the sentencepiece library) again
 `sentencepiece` Python package wraps the same C++ code.  Models are trained here, by the library, on seeded text."""
 import io
 import json
-import os
 import random
 
 import pytest

@@ -131,7 +131,6 @@ _SIGS = {
     "launch_patches_v2": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "launch_patches_b1_batched_async": (_i, [_vp, C.POINTER(PatchBatchDesc), _i, _i, _vp]),
 }
-_OPTIONAL = {}
 for _name, (_res, _args) in _SIGS.items():
     _fn = getattr(lib, _name)
     _fn.restype, _fn.argtypes = _res, _args
