@@ -203,7 +203,8 @@ def add_rms_norm_bf16(x: np.ndarray, residual: np.ndarray, weight: np.ndarray, e
 def silu_mul_bf16(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
     """bf16_rne(g / (1 + exp(-g)) * up) (kernels.hip:447-459)."""
     g = gate.astype(np.float32)
-    s = g / (np.float32(1.0) + np.exp(-g, dtype=np.float32))
+    with np.errstate(over="ignore"):          # exp(-g) = inf for g < -88: g / inf = -0, what expf gives on the GPU too
+        s = g / (np.float32(1.0) + np.exp(-g, dtype=np.float32))
     return f32_to_bf16_bits(s * up.astype(np.float32))
 
 
