@@ -54,15 +54,20 @@ int   t12_engine_decode(void* state, int max_tokens, int stop_on_eos, int* out);
  * for max_tokens * batch ints, may be NULL); returns the number of steps. */
 int   t12_engine_decode_all(void* state, int max_tokens, int* out);
 
+/* prefill_rows: prompt pass of a batch-1 state, `rows` tokens per pass through a helper state of that many rows that
+ * the state creates on first use (decode+GEMM kernels; the reference prompts one token per forward,
+ * inference.cpp:721-724); logits of the last token in state->logits, positions[0] advanced. */
+int   t12_engine_prefill_rows(void* state, const int* tokens_host, int n_tokens, int rows);
 /* shift_context: cache rows [discard, current_pos) of sequence seq -> rows [0, current_pos - discard), all layers,
  * K, V and scales (the reference does this inline, engine/main.cpp:147-173). */
 int   t12_engine_shift_context(void* state, int seq, int current_pos, int discard);
 /* chat_turn: one turn of the reference's interactive loop (engine/main.cpp:139-213) on a batch-1 state: drops a
  * leading BOS after the first turn, shifts the context when it is too long, enters the n_tokens ids at *current_pos,
  * generates up to max_tokens ids until eos_id / bos_id (into out, room for max_tokens), feeds eos_id, advances
- * *current_pos; *discarded (may be NULL) = cache rows dropped by the shift.  Returns the number generated. */
+ * *current_pos; *discarded (may be NULL) = cache rows dropped by the shift.  prompt_rows > 1: the new ids enter that
+ * many per pass (prefill_rows) instead of one per forward.  Returns the number generated. */
 int   t12_engine_chat_turn(void* state, int* current_pos, const int* tokens, int n_tokens, int max_tokens, int bos_id,
-                           int eos_id, int* discarded, int* out);
+                           int eos_id, int prompt_rows, int* discarded, int* out);
 
 /* ---- tokenizer: C face of include/turbo/tokenizer.h (the reference's engine/tokenizer.h:19-23), host only ---- */
 void* t12_tokenizer_load(const char* model_dir);                      /* load_tokenizer; NULL without tokenizer.model or vocab.bin + merges.bin */

@@ -61,6 +61,14 @@ void forward(InferenceState* state, const int* token_ids);
 // With batch_size 1 it is n_tokens calls of forward.
 void prefill(InferenceState* state, int seq, const int* token_ids, int n_tokens);
 
+// Extension: prefill for a state of batch size 1, `rows` prompt tokens per pass.  Such a state has no rows to
+// batch over (prefill runs it token by token); here a helper state of `rows` rows on the same model, created on
+// first use and kept by the state, lends its buffers: the prompt goes through the decode+GEMM kernels into this
+// state's cache region, the last token's logits land in state->logits, positions[0] advances by n_tokens.
+// rows <= 1 is prefill(state, 0, ...).  The logits agree with the token-by-token pass to rounding (other kernels,
+// other summation order), not bit for bit.
+void prefill_rows(InferenceState* state, const int* token_ids, int n_tokens, int rows);
+
 // Prompt one token per forward, then greedy decode; stops at token id 2 like the
 // reference (engine/inference.cpp:716-748).
 std::vector<int> generate(InferenceState* state, const std::vector<int>& prompt_tokens, int max_tokens);
@@ -87,7 +95,8 @@ void shift_context(InferenceState* state, int seq, int current_pos, int discard)
 // (shift_context; *discarded receives the count).  Then the new tokens enter at *current_pos, up to max_tokens
 // greedy tokens follow until eos_id or bos_id is sampled (neither is returned), and eos_id (2 when eos_id <= 0)
 // is fed so that the context records the end of the turn.  *current_pos is advanced past all of it.  on_token
-// (optional) receives every generated id as soon as the host has it.
+// (optional) receives every generated id as soon as the host has it.  prompt_rows > 1 enters the new tokens that
+// many per pass (prefill_rows) instead of one per forward.
 std::vector<int> chat_turn(InferenceState* state, int* current_pos, const std::vector<int>& turn_tokens, int max_tokens,
                            int bos_id, int eos_id, int* discarded = nullptr,
-                           const std::function<void(int)>& on_token = nullptr);
+                           const std::function<void(int)>& on_token = nullptr, int prompt_rows = 1);

@@ -147,6 +147,51 @@ def test_chat_turns_with_context_shifts_equal_the_reference_loop(t12, oracle, mo
         eng.close()
 
 
+def test_batched_prompt_pass_of_a_batch_one_state(t12, oracle, model):
+    """prefill_rows: 37 prompt tokens, 16 per pass (16 + 16 + 5), into the batch-1 state's own cache region through a helper
+    state; the logits equal the CPU step token by token to rounding, the cache serves the decode that follows, and
+    a second prompt continues from the new position."""
+    path, parts = model
+    rng = np.random.default_rng(34)
+    eng = load(t12, path, batch=1)
+    try:
+        ref = oracle.RefModel(*parts, max_seq=CTX)
+        pos = 0
+        for n, rows in [(37, 16), (1, 16), (9, 4), (5, 1)]:
+            toks = [int(x) for x in rng.integers(3, V, size=n)]
+            for t in toks:
+                want = ref.step(t, pos)
+                pos += 1
+            eng.prefill_rows(toks, rows)
+            assert eng.positions() == [pos]
+            assert rel(eng.logits(V).cpu().numpy()[0], want) < 2e-2, (n, rows)
+            got = eng.decode(3)
+            for g in got:
+                assert g == oracle.argmax_first(want)
+                want = ref.step(g, pos)
+                pos += 1
+            assert eng.positions() == [pos]
+    finally:
+        eng.close()
+
+
+def test_chat_turns_with_batched_prompts(t12, oracle, model):
+    path, parts = model
+    rng = np.random.default_rng(35)
+    eng = load(t12, path, batch=1)
+    try:
+        chat = RefChat(oracle.RefModel(*parts, max_seq=CTX), CTX)
+        pos = 0
+        for turn in range(7):
+            tokens = [BOS] + [int(x) for x in rng.integers(3, V, size=6 + 3 * (turn % 3))]
+            want, want_discard = chat.turn(tokens, 8, oracle)
+            got, pos, discarded = eng.chat_turn(pos, tokens, 8, BOS, EOS, prompt_rows=8)
+            assert got == want, turn
+            assert (pos, discarded) == (chat.pos, want_discard), turn
+    finally:
+        eng.close()
+
+
 def test_text_in_text_out(t12, oracle, model, tmp_path):
     """tokenize -> chat_turn -> detokenize_one over a tokenizer whose ids fit the model's vocabulary."""
     tf = importlib.import_module("turbo_lossless_amd.tokenizer_files")

@@ -99,8 +99,9 @@ _SIGS = {
     "t12_engine_decode": (_i, [_vp, _i, _i, C.POINTER(C.c_int)]),
     "t12_engine_sync": (_i, [_vp]),
     "t12_engine_shift_context": (_i, [_vp, _i, _i, _i]),
-    "t12_engine_chat_turn": (_i, [_vp, C.POINTER(C.c_int), C.POINTER(C.c_int), _i, _i, _i, _i, C.POINTER(C.c_int),
+    "t12_engine_chat_turn": (_i, [_vp, C.POINTER(C.c_int), C.POINTER(C.c_int), _i, _i, _i, _i, _i, C.POINTER(C.c_int),
                                   C.POINTER(C.c_int)]),
+    "t12_engine_prefill_rows": (_i, [_vp, C.POINTER(C.c_int), _i, _i]),
     "t12_tokenizer_load": (_vp, [C.c_char_p]),
     "t12_tokenizer_free": (None, [_vp]),
     "t12_tokenizer_info": (_i, [_vp, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
@@ -379,13 +380,18 @@ class Engine:
         """Cache rows [discard, current_pos) of sequence seq move to the front (engine/main.cpp:147-173)."""
         check(lib.t12_engine_shift_context(self.state, int(seq), int(current_pos), int(discard)), "shift_context")
 
-    def chat_turn(self, current_pos, tokens, max_tokens, bos_id, eos_id):
+    def prefill_rows(self, tokens, rows):
+        """Prompt pass of a batch-1 engine, `rows` tokens per pass (a helper state lends its buffers)."""
+        arr = (C.c_int * max(len(tokens), 1))(*[int(t) for t in tokens])
+        check(lib.t12_engine_prefill_rows(self.state, arr, len(tokens), int(rows)), "prefill_rows")
+
+    def chat_turn(self, current_pos, tokens, max_tokens, bos_id, eos_id, prompt_rows=1):
         """One interactive turn (engine/main.cpp:139-213) -> (generated ids, new current_pos, rows discarded)."""
         pos, dropped = C.c_int(int(current_pos)), C.c_int(0)
         arr = (C.c_int * max(len(tokens), 1))(*[int(t) for t in tokens])
         out = (C.c_int * max(max_tokens, 1))()
         n = lib.t12_engine_chat_turn(self.state, C.byref(pos), arr, len(tokens), int(max_tokens), int(bos_id), int(eos_id),
-                                     C.byref(dropped), out)
+                                     int(prompt_rows), C.byref(dropped), out)
         return list(out[:n]), pos.value, dropped.value
 
     def weight(self, layer, which):

@@ -93,6 +93,12 @@ int t12_engine_decode_all(void* state, int max_tokens, int* out)
     return (int)(r.size() / (size_t)s->batch_size);
 }
 
+int t12_engine_prefill_rows(void* state, const int* tokens_host, int n_tokens, int rows)
+{
+    prefill_rows((InferenceState*)state, tokens_host, n_tokens, rows);
+    return 0;
+}
+
 int t12_engine_shift_context(void* state, int seq, int current_pos, int discard)
 {
     shift_context((InferenceState*)state, seq, current_pos, discard);
@@ -101,10 +107,11 @@ int t12_engine_shift_context(void* state, int seq, int current_pos, int discard)
 
 // chat_turn(); out has room for max_tokens ids; returns how many were generated.
 int t12_engine_chat_turn(void* state, int* current_pos, const int* tokens, int n_tokens, int max_tokens, int bos_id,
-                         int eos_id, int* discarded, int* out)
+                         int eos_id, int prompt_rows, int* discarded, int* out)
 {
     std::vector<int> t(tokens, tokens + n_tokens);
-    std::vector<int> r = chat_turn((InferenceState*)state, current_pos, t, max_tokens, bos_id, eos_id, discarded);
+    std::vector<int> r = chat_turn((InferenceState*)state, current_pos, t, max_tokens, bos_id, eos_id, discarded, nullptr,
+                                   prompt_rows);
     if (out)
         for (size_t i = 0; i < r.size(); i++) out[i] = r[i];
     return (int)r.size();

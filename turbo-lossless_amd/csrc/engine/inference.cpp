@@ -64,6 +64,8 @@ struct Impl {
     int8_t* pv = nullptr;
     float* psk = nullptr;
     float* psv = nullptr;
+    // prefill_rows: a state of that many rows on the same model, whose buffers carry a batch-1 state's prompt passes
+    InferenceState* helper = nullptr;
 };
 
 // Where a forward reads and writes the KV cache: layer l of sequence b starts at
@@ -239,6 +241,7 @@ void free_inference_state(InferenceState* state)
         }
         for (void* p : {(void*)impl->pk, (void*)impl->pv, (void*)impl->psk, (void*)impl->psv})
             if (p) (void)hipFree(p);
+        free_inference_state(impl->helper);
     }
     delete impl;
     delete state;
@@ -555,6 +558,54 @@ void prefill(InferenceState* state, int seq, const int* token_ids, int n_tokens)
     }
 }
 
+// A batch-1 state has no rows to batch a prompt over; a helper state of `rows` rows on the same model lends its
+// buffers: the prompt goes through the decode+GEMM kernels `rows` tokens per pass into THIS state's cache region,
+// and the last token's logits land in this state's logits.  The helper works on its own stream, ordered after what
+// this state has enqueued and before what it enqueues next.
+void prefill_rows(InferenceState* state, const int* token_ids, int n_tokens, int rows)
+{
+    if (state->batch_size != 1) {
+        fprintf(stderr, "ERROR: prefill_rows is for states of batch size 1 (got %d): use prefill\n", state->batch_size);
+        exit(1);
+    }
+    if (rows <= 1 || n_tokens <= 1) {
+        prefill(state, 0, token_ids, n_tokens);
+        return;
+    }
+    Impl* impl = (Impl*)state->impl;
+    if (impl->helper && impl->helper->batch_size != rows) {
+        check_gpu(hipStreamSynchronize(impl->helper->stream), "hipStreamSynchronize");
+        free_inference_state(impl->helper);
+        impl->helper = nullptr;
+    }
+    if (!impl->helper) impl->helper = create_inference_state(state->model, rows, 0);
+    InferenceState* h = impl->helper;
+    const ModelConfig& c = state->model->config;
+    launch_rope_scaling(c.rope_scaling[0], c.rope_scaling[1], c.rope_scaling[2], c.rope_scaling[3]);
+    KvView kv = kv_view(state);                    // this state's region (batch 1: sequence 0)
+    kv.kv_stride = 0;
+    const int p0 = state->positions[0];
+    if (p0 + n_tokens > kv.max_seq) {
+        fprintf(stderr, "ERROR: position %d exceeds the KV cache (%d)\n", p0 + n_tokens - 1, kv.max_seq);
+        exit(1);
+    }
+    check_gpu(hipEventRecord(state->sync_event, state->stream), "hipEventRecord");
+    check_gpu(hipStreamWaitEvent(h->stream, state->sync_event, 0), "hipStreamWaitEvent");
+    std::vector<int> pos(rows);
+    for (int done = 0; done < n_tokens;) {
+        const int R = std::min(rows, n_tokens - done);
+        const bool last = done + R == n_tokens;
+        for (int r = 0; r < R; r++) pos[r] = p0 + done + r;
+        (void)hipMemcpyAsync(h->d_tokens, token_ids + done, R * sizeof(int), hipMemcpyHostToDevice, h->stream);
+        (void)hipMemcpyAsync(h->d_positions, pos.data(), R * sizeof(int), hipMemcpyHostToDevice, h->stream);
+        forward_rows(h, R, kv, p0 + done + (R > 1 ? R - 1 : 0), last ? LOGITS_LAST_ROW : LOGITS_NONE, state->logits);
+        done += R;
+    }
+    check_gpu(hipEventRecord(h->sync_event, h->stream), "hipEventRecord");
+    check_gpu(hipStreamWaitEvent(state->stream, h->sync_event, 0), "hipStreamWaitEvent");
+    state->positions[0] = p0 + n_tokens;
+}
+
 // Greedy decoding from the logits the state holds, `max_tokens` steps of (sample, forward).
 // The reference's loop (inference.cpp:726-746) waits for every sampled token on the host before it
 // enqueues the next forward, so the GPU idles for a host round trip per token.  Here the argmax
@@ -681,7 +732,7 @@ void shift_context(InferenceState* state, int seq, int current_pos, int discard)
 
 // One turn of the reference's interactive loop, engine/main.cpp:139-203, without its printing.
 std::vector<int> chat_turn(InferenceState* state, int* current_pos, const std::vector<int>& turn_tokens, int max_tokens,
-                           int bos_id, int eos_id, int* discarded, const std::function<void(int)>& on_token)
+                           int bos_id, int eos_id, int* discarded, const std::function<void(int)>& on_token, int prompt_rows)
 {
     if (discarded) *discarded = 0;
     if (state->batch_size != 1) {
@@ -701,7 +752,8 @@ std::vector<int> chat_turn(InferenceState* state, int* current_pos, const std::v
         if (discarded) *discarded = discard;
     }
     state->positions[0] = pos;
-    prefill(state, 0, tokens.data(), (int)tokens.size());        // batch size 1: one forward per new token (:181-184)
+    // one forward per new token like the reference (:181-184), or prompt_rows tokens per pass
+    prefill_rows(state, tokens.data(), (int)tokens.size(), prompt_rows);
     std::vector<int> out = decode_loop(state, max_tokens, eos_id, bos_id, false, on_token);   // :192-202
     const int eos_tok = eos_id > 0 ? eos_id : 2;                 // the turn's end enters the context (:207-213)
     forward(state, &eos_tok);
