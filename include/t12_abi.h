@@ -211,6 +211,23 @@ int launch_split12_batch8_async(const void* sm, const void* gr, int base_exp,
                                 void* o0, void* o1, void* o2, void* o3,
                                 void* o4, void* o5, void* o6, void* o7, int M, int K, void* stream);
 
+/* The reference's larger-batch entry points (nvidia_kernels.cu:444-524, 426-442, 550-584), same names and arguments.
+ * fused_gemm: out[b*out_stride + m] = sum_k dec(W[m,k]) * act[b*act_stride + k], escapes exact when all four list
+ * pointers are non-NULL, "wrong" values otherwise.  patches_batch: the separate correction launch over the listed
+ * rows, out[b*out_stride + row] += sum (correct - wrong) * act[b*act_stride + col].  cublas_batch: the unpatched
+ * product; the reference decodes into bf16_weight_buf and calls a vendor GEMM, this build runs the fused kernel and
+ * leaves the buffer alone. */
+int nv_launch_split12_fused_gemm_async(const void* sm, const void* gr, int base_exp, const void* act, int act_stride,
+                                       void* out, int out_stride, int M, int K, int B, void* stream,
+                                       const void* patch_row_off, const void* patch_cols, const void* patch_correct,
+                                       const void* patch_wrong);
+int nv_launch_patches_batch_async(const void* row_off, const void* cols, const void* correct, const void* wrong,
+                                  const void* nonempty_rows, int num_nonempty, const void* act, int act_stride,
+                                  void* out, int out_stride, int B, void* stream);
+int nv_launch_split12_cublas_batch_async(const void* sign_mantissa, const void* groups, int base_exp,
+                                         const void* activations, int act_stride, void* output, int out_stride,
+                                         void* bf16_weight_buf, int buf_half_elems, int M, int K, int B, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

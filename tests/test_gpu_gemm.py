@@ -229,3 +229,46 @@ def test_gemm_swiglu_declines_shapes_without_a_fused_kernel(t12, oracle, synth):
     assert t12.lib.t12_gemm_swiglu(s1, s1, X.data_ptr(), 256, 256, 256, out.data_ptr(), 512, st) == 1      # few rows
     assert t12.lib.t12_gemm_swiglu(s1, s1, X.data_ptr(), 256, 256, 64, out.data_ptr(), 512, st) == 1       # small batch
     assert t12.lib.t12_gemm_swiglu(s1, s1, X.data_ptr(), 256, 256, 256, out.data_ptr(), 100, st) == -1     # out_stride < M
+
+
+@pytest.mark.parametrize("M,K,B", [(300, 1024, 48), (1024, 4096, 256), (77, 320, 9)])
+def test_reference_named_batch_entry_points(t12, oracle, synth, M, K, B):
+    """nv_launch_split12_fused_gemm_async with and without the escape lists, the separate correction launch
+    nv_launch_patches_batch_async on top of the unpatched product, and nv_launch_split12_cublas_batch_async
+    (nvidia_kernels.cu:426-584), called with the reference's argument lists."""
+    p = oracle.pack(synth.weights_llm(M, K, seed=M + B, p_outlier=3e-3))
+    X = synth.activations(B, K, seed=K + B)
+    ref, ref_un = oracle.gemm(p, X), oracle.gemm(p, X, patched=False)
+    d = t12.DeviceTensor12.from_packed(p, dev())
+    Xd = to_dev_bits(X).reshape(X.shape)
+    st = t12.current_stream()
+    ptr = lambda t: t.data_ptr()
+
+    out = torch.full((B, M + 3), float("nan"), device=dev())                 # out_stride > M
+    rc = t12.lib.nv_launch_split12_fused_gemm_async(ptr(d.sm), ptr(d.gr), d.base_exp, ptr(Xd), K, ptr(out), M + 3, M, K, B, st,
+                                                    ptr(d.row_off), ptr(d.cols), ptr(d.correct), ptr(d.wrong))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert rel_err(out[:, :M].cpu().numpy(), ref) < TOL
+
+    un = torch.zeros((B, M), device=dev())
+    assert t12.lib.nv_launch_split12_fused_gemm_async(ptr(d.sm), ptr(d.gr), d.base_exp, ptr(Xd), K, ptr(un), M, M, K, B, st,
+                                                      None, None, None, None) == 0
+    via_buf = torch.zeros((B, M), device=dev())
+    scratch = torch.zeros(8, dtype=torch.int16, device=dev())                # not touched by this build
+    assert t12.lib.nv_launch_split12_cublas_batch_async(ptr(d.sm), ptr(d.gr), d.base_exp, ptr(Xd), K, ptr(via_buf), M,
+                                                        ptr(scratch), 4, M, K, B, st) == 0
+    torch.cuda.synchronize()
+    assert rel_err(un.cpu().numpy(), ref_un) < TOL
+    assert torch.equal(un, via_buf) and int(scratch.abs().sum()) == 0
+
+    # the reference's two-launch form: unpatched product, then the correction over the rows that have escapes
+    ro = p.row_off
+    rows = np.nonzero(ro[1:] > ro[:-1])[0].astype(np.int32)
+    assert 0 < len(rows)
+    rows_d = torch.from_numpy(rows).to(dev())
+    assert t12.lib.nv_launch_patches_batch_async(ptr(d.row_off), ptr(d.cols), ptr(d.correct), ptr(d.wrong), ptr(rows_d), len(rows),
+                                                 ptr(Xd), K, ptr(un), M, B, st) == 0
+    torch.cuda.synchronize()
+    assert rel_err(un.cpu().numpy(), ref) < TOL
+    assert t12.lib.nv_launch_patches_batch_async(None, None, None, None, None, 0, None, K, None, M, B, st) == 0   # nothing to do

@@ -119,6 +119,9 @@ _SIGS = {
     "t12_gemv_batch": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
     "launch_split12_batch4_async": (_i, [_vp] * 2 + [_i] + [_vp] * 4 + [_vp] * 3 + [_vp] * 4 + [_i, _i, _vp]),
     "launch_split12_batch8_async": (_i, [_vp] * 2 + [_i] + [_vp] * 8 + [_vp] * 3 + [_vp] * 8 + [_i, _i, _vp]),
+    "nv_launch_split12_fused_gemm_async": (_i, [_vp, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
+    "nv_launch_patches_batch_async": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _i, _vp]),
+    "nv_launch_split12_cublas_batch_async": (_i, [_vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_gemm": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_tune_gemm": (_i, [_i]),
     "t12_gemm_swiglu": (_i, [C.POINTER(Segment), C.POINTER(Segment), _vp, _i, _i, _i, _vp, _i, _vp]),

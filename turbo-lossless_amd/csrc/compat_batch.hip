@@ -1,5 +1,6 @@
-// Reference-named small-batch launchers: launch_split12_batch4_async /
-// launch_split12_batch8_async (decompress_v2.hip:860-901).
+// Reference-named batch launchers: launch_split12_batch4_async / launch_split12_batch8_async
+// (decompress_v2.hip:860-901) and, at the end of the file, the three entry points of the reference's larger-batch path
+// (nvidia_kernels.cu:426-584).
 //
 // Their interface carries the escapes not as a CSR list but as the derived
 // tables of engine/model.cpp:86-160: esc_row_base[row], optional
@@ -97,6 +98,26 @@ int launch(const void* sm, const void* gr, int base_exp, const void* const* a, c
     return T12_OK;
 }
 
+
+// nv_apply_patches_batch (nvidia_kernels.cu:295-319): one thread per (listed row, batch row) pair walks the row's
+// escape slice: out[b, row] += sum over entries of (correct - wrong) * x[b, col]; nothing is written when the sum is 0.
+__global__ __launch_bounds__(256) void patches_batch_kernel(const int32_t* __restrict__ row_off, const int32_t* __restrict__ cols,
+                                                            const int16_t* __restrict__ correct, const int16_t* __restrict__ wrong,
+                                                            const int32_t* __restrict__ rows, const uint16_t* __restrict__ act,
+                                                            int act_stride, float* __restrict__ out, int out_stride, int n_rows,
+                                                            int B)
+{
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const int ri = (int)(idx / B), b = (int)(idx % B);
+    if (ri >= n_rows) return;
+    const int row = rows[ri];
+    const uint16_t* x = act + (size_t)b * act_stride;
+    float c = 0.0f;
+    for (int q = row_off[row]; q < row_off[row + 1]; q++)
+        c += (t12_bf16_to_f32((uint16_t)correct[q]) - t12_bf16_to_f32((uint16_t)wrong[q])) * t12_bf16_to_f32(x[cols[q]]);
+    if (c != 0.0f) out[(size_t)b * out_stride + row] += c;
+}
+
 }  // namespace
 
 extern "C" {
@@ -120,6 +141,53 @@ int launch_split12_batch8_async(const void* sm, const void* gr, int base_exp, co
     const void* a[8] = {a0, a1, a2, a3, a4, a5, a6, a7};
     void* o[8] = {o0, o1, o2, o3, o4, o5, o6, o7};
     return launch<8>(sm, gr, base_exp, a, esc_row_base, esc_counts, esc_vals, o, M, K, stream);
+}
+
+// ---- the reference's entry points for larger batches (nvidia_kernels.cu:426-584), same names and arguments ----
+
+// out[b, m] = sum_k dec(W[m, k]) * X[b, k]; escapes exact when the four list pointers are given, "wrong" values when
+// they are null (the reference's V1 kernel adds the correction in its epilogue under the same condition,
+// split12_gemm.cuh:273-284).  The reference reads the activations with a row stride of K whatever act_stride says
+// (nvidia_kernels.cu:446,467); its callers pass K, and this entry point honours the argument.
+int nv_launch_split12_fused_gemm_async(const void* sm, const void* gr, int base_exp, const void* act, int act_stride,
+                                       void* out, int out_stride, int M, int K, int B, void* stream,
+                                       const void* patch_row_off, const void* patch_cols, const void* patch_correct,
+                                       const void* patch_wrong)
+{
+    const bool lists = patch_row_off && patch_cols && patch_correct && patch_wrong;
+    T12Segment g = {(const uint8_t*)sm, (const uint8_t*)gr, lists ? (const int32_t*)patch_row_off : nullptr,
+                    lists ? (const int32_t*)patch_cols : nullptr, lists ? (const int16_t*)patch_correct : nullptr,
+                    lists ? (const int16_t*)patch_wrong : nullptr, (float*)out, M, base_exp, out_stride, 0};
+    return t12_gemm(&g, 1, act, act_stride, out_stride, K, B, stream);
+}
+
+// The separate correction launch that follows an unpatched GEMM in the reference (nvidia_kernels.cu:426-442).
+int nv_launch_patches_batch_async(const void* row_off, const void* cols, const void* correct, const void* wrong,
+                                  const void* nonempty_rows, int num_nonempty, const void* act, int act_stride, void* out,
+                                  int out_stride, int B, void* stream)
+{
+    if (num_nonempty == 0 || B == 0) return 0;
+    T12_REQUIRE(row_off && cols && correct && wrong && nonempty_rows && act && out && num_nonempty > 0 && B > 0,
+                "nv_launch_patches_batch_async: null operand or negative count");
+    const long pairs = (long)num_nonempty * B;
+    hipLaunchKernelGGL(patches_batch_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const int32_t*)row_off, (const int32_t*)cols, (const int16_t*)correct, (const int16_t*)wrong,
+                       (const int32_t*)nonempty_rows, (const uint16_t*)act, act_stride, (float*)out, out_stride, num_nonempty, B);
+    T12_CHECK_LAUNCH("nv_launch_patches_batch_async");
+    return T12_OK;
+}
+
+// The reference decodes the tensor (unpatched) into bf16_weight_buf and calls a vendor GEMM on it
+// (nvidia_kernels.cu:550-584).  Here the same product comes from the fused decode+GEMM: the buffer is not touched.
+int nv_launch_split12_cublas_batch_async(const void* sign_mantissa, const void* groups, int base_exp, const void* activations,
+                                         int act_stride, void* output, int out_stride, void* bf16_weight_buf,
+                                         int buf_half_elems, int M, int K, int B, void* stream)
+{
+    (void)bf16_weight_buf;
+    (void)buf_half_elems;
+    T12Segment g = {(const uint8_t*)sign_mantissa, (const uint8_t*)groups, nullptr, nullptr, nullptr, nullptr, (float*)output,
+                    M, base_exp, out_stride, 0};
+    return t12_gemm(&g, 1, activations, act_stride, out_stride, K, B, stream);
 }
 
 // Small-batch entry point: 1 <= B <= 8 rows of activations; same contract as t12_gemm.
