@@ -217,6 +217,13 @@ int launch_split12_batch8_async(const void* sm, const void* gr, int base_exp,
  * rows, out[b*out_stride + row] += sum (correct - wrong) * act[b*act_stride + col].  cublas_batch: the unpatched
  * product; the reference decodes into bf16_weight_buf and calls a vendor GEMM, this build runs the fused kernel and
  * leaves the buffer alone. */
+int nv_launch_split12_v2_async(const void* sm, const void* gr, int base_exp, const void* act, void* out, int M, int K,
+                               void* stream);                                   /* nvidia_kernels.cu:385 = launch_split12_v2_async */
+int nv_launch_split12_v2_dual_async(const void* sm_a, const void* gr_a, int base_exp_a, const void* sm_b, const void* gr_b,
+                                    int base_exp_b, const void* act, void* out_a, void* out_b, int M, int K,
+                                    void* stream);                              /* :402 = launch_split12_v2_dual_async */
+int nv_launch_patches_async(const void* row_off, const void* cols, const void* correct, const void* wrong, const void* act,
+                            void* out, int M, void* stream);                    /* :414 = launch_patches_v2_async */
 int nv_launch_split12_fused_gemm_async(const void* sm, const void* gr, int base_exp, const void* act, int act_stride,
                                        void* out, int out_stride, int M, int K, int B, void* stream,
                                        const void* patch_row_off, const void* patch_cols, const void* patch_correct,

@@ -53,6 +53,10 @@ def test_library_exports_glue_and_engine_c_face():
             "launch_attention_all_heads", "launch_attention_all_heads_batch", "launch_flash_attention",
             "launch_flash_attention_batch", "launch_rope_store_kv", "launch_rope_init", "launch_argmax",
             "launch_argmax_batch"]                      # engine/inference.cpp:9-20, sampler.cpp:4-5
+    other_build = ["nv_launch_split12_v2_async", "nv_launch_split12_v2_dual_async", "nv_launch_patches_async",
+                   "nv_launch_patches_batch_async", "nv_launch_split12_fused_gemm_async",
+                   "nv_launch_split12_cublas_batch_async"]                         # engine/inference.cpp:33-41
+    glue = glue + other_build
     engine = ["t12_engine_load", "t12_engine_create_state", "t12_engine_forward", "t12_engine_generate",
               "t12_engine_sample", "t12_engine_free_state", "t12_engine_free_model"]
     missing = [n for n in glue + engine if not hasattr(lib, n)]

@@ -190,6 +190,26 @@ int nv_launch_split12_cublas_batch_async(const void* sign_mantissa, const void* 
     return t12_gemm(&g, 1, activations, act_stride, out_stride, K, B, stream);
 }
 
+// The B = 1 entry points under the names the reference's other build uses (nvidia_kernels.cu:385-424): same
+// arguments and meaning as launch_split12_v2_async / _v2_dual_async / launch_patches_v2_async.
+int nv_launch_split12_v2_async(const void* sm, const void* gr, int base_exp, const void* act, void* out, int M, int K,
+                               void* stream)
+{
+    return launch_split12_v2_async(sm, gr, base_exp, act, out, M, K, stream);
+}
+
+int nv_launch_split12_v2_dual_async(const void* sm_a, const void* gr_a, int base_exp_a, const void* sm_b, const void* gr_b,
+                                    int base_exp_b, const void* act, void* out_a, void* out_b, int M, int K, void* stream)
+{
+    return launch_split12_v2_dual_async(sm_a, gr_a, base_exp_a, sm_b, gr_b, base_exp_b, act, out_a, out_b, M, K, stream);
+}
+
+int nv_launch_patches_async(const void* row_off, const void* cols, const void* correct, const void* wrong, const void* act,
+                            void* out, int M, void* stream)
+{
+    return launch_patches_v2_async(row_off, cols, correct, wrong, act, out, M, stream);
+}
+
 // Small-batch entry point: 1 <= B <= 8 rows of activations; same contract as t12_gemm.
 int t12_gemv_batch(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride, int out_stride, int K,
                    int B, void* stream)
