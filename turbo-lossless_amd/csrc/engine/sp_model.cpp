@@ -157,7 +157,8 @@ std::string SpModel::load(const std::string& path)
     for (int b = 0; b < 256; b++) byte_id[b] = -1;
     for (int i = 0; i < (int)pieces.size(); i++) {
         const Piece& pc = pieces[i];
-        if (pc.type == NORMAL || pc.type == USER_DEFINED || pc.type == UNUSED) merge_ids.emplace(pc.text, i);
+        if (pc.type == UNUSED) return "the model marks pieces unused (their resegmentation is not built)";
+        if (pc.type == NORMAL || pc.type == USER_DEFINED) merge_ids.emplace(pc.text, i);
         else reserved_ids.emplace(pc.text, i);
         if (pc.type == USER_DEFINED && !pc.text.empty()) user_defined.push_back(pc.text);
         if (pc.type == BYTE && pc.text.size() == 6) byte_id[strtol(pc.text.c_str() + 3, nullptr, 16) & 255] = i;

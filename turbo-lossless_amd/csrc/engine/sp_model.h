@@ -4,8 +4,8 @@
 //
 // Supported: model_type BPE, identity normalisation (no precompiled character map) with the three whitespace
 // rules (add_dummy_prefix, remove_extra_whitespaces, escape_whitespaces), byte fallback, user-defined pieces.
-// That covers the Llama-2 / Mistral tokenizers the reference targets.  A unigram model or a model with a
-// character map fails to load with a message.
+// That covers the Llama-2 / Mistral tokenizers the reference targets.  A unigram model, a model with a character
+// map, or one with pieces marked unused fails to load with a message.
 #pragma once
 #include <cstdint>
 #include <string>
@@ -20,7 +20,7 @@ struct SpModel {
         int type;
     };
     std::vector<Piece> pieces;
-    std::unordered_map<std::string, int> merge_ids;      // NORMAL / USER_DEFINED / UNUSED pieces: what merging may produce
+    std::unordered_map<std::string, int> merge_ids;      // NORMAL / USER_DEFINED pieces: what merging may produce
     std::unordered_map<std::string, int> reserved_ids;   // every other piece
     std::vector<std::string> user_defined;               // longest first
     int byte_id[256];
