@@ -189,10 +189,12 @@ def test_gemm_more_escapes_than_the_lds_list_holds(t12, oracle, synth, B):
 
 
 @pytest.mark.parametrize("M,K,B,p_out", [(14336, 4096, 256, 3e-4), (12300, 512, 129, 2e-3), (12352, 256, 300, 5e-2),
-                                          (12288, 64, 512, 0.0)])
+                                          (12288, 64, 512, 0.0), (14336, 4096, 128, 3e-4), (12300, 512, 65, 2e-3),
+                                          (12352, 256, 100, 5e-2)])
 def test_gemm_swiglu_epilogue_is_bit_identical_to_unfused(t12, synth, M, K, B, p_out):
     """t12_gemm_swiglu == t12_gemm on (gate, up) + launch_silu_mul_bf16_batch, bit for bit (ragged last tile,
-    escape lists that fit the LDS staging and ones that overflow it, tensors without escapes)."""
+    escape lists that fit the LDS staging and ones that overflow it, tensors without escapes; batch tiles of 256
+    rows and, for 65 .. 128 rows, of 128)."""
     g = torch.Generator(device=dev())
 
     def mk(seed):

@@ -635,7 +635,7 @@ int t12_gemm_swiglu(const T12Segment* gate, const T12Segment* up, const void* ac
     T12_REQUIRE(gate->M >= 1 && gate->M == up->M, "t12_gemm_swiglu: gate has %d rows, up has %d", gate->M, up->M);
     T12_REQUIRE(out_stride >= gate->M, "t12_gemm_swiglu: out_stride %d < M %d", out_stride, gate->M);
     const T12Segment* two[2] = {gate, up};
-    bool fast = (K % KC == 0) && (act_stride % 8 == 0) && ((uintptr_t)act_bf16 % 16 == 0) && B > 128;
+    bool fast = (K % KC == 0) && (act_stride % 8 == 0) && ((uintptr_t)act_bf16 % 16 == 0) && B > 64;
     for (const T12Segment* g : two) {
         T12_REQUIRE(g->sm && g->gr, "t12_gemm_swiglu: a plane is null");
         T12_REQUIRE(!g->row_off || (g->cols && g->correct && g->wrong), "t12_gemm_swiglu: row_off without lists");
@@ -643,7 +643,7 @@ int t12_gemm_swiglu(const T12Segment* gate, const T12Segment* up, const void* ac
         if (g->base_exp < 0 || g->base_exp > 240) fast = false;
     }
     const int tiles = (gate->M + TM / 2 - 1) / (TM / 2);
-    const int btiles = (B + 255) / 256;
+    const int btiles = B > 128 ? (B + 255) / 256 : 1;
     if (!fast || tiles * btiles * 4 < 256 * 3) return 1;      // would need a K split: partial sums cannot be gated
     GemmParams p;
     p.seg[0] = *gate;
@@ -662,6 +662,8 @@ int t12_gemm_swiglu(const T12Segment* gate, const T12Segment* up, const void* ac
     p.seg_row0[0] = p.seg_row0[1] = 0;
     p.out_bf16 = (uint16_t*)out_bf16;
     p.out_bf16_ld = out_stride;
+    // batch tile of 256 rows, or of 128 for 65 .. 128 rows (one accumulator pair per wave)
+    if (B <= 128) return launch_mfma<4, 2, 1, 2, true>(p, tiles, (hipStream_t)stream);
     return launch_mfma<4, 2, 2, 2, true>(p, tiles, (hipStream_t)stream);
 }
 
