@@ -286,3 +286,34 @@ def test_extract_writes_the_reference_file_formats(tf, tmp_path):
     be = (tmp_path / "byte_encoder.bin").read_bytes()
     # byte 0 -> U+0100; 94 printable ASCII bytes keep 1 UTF-8 byte, the other 162 characters take 2
     assert be[:3] == b"\x02\xc4\x80" and len(be) == 256 + 94 + 2 * 162
+
+
+def test_encode_equals_reference_rule_on_generated_tables(t12, tf, tmp_path):
+    """Property test (hypothesis): any merge table over a three-letter alphabet -- pairs repeated, merges listed
+    before their parts exist, results missing from the vocabulary -- and any text: same ids as the literal rule."""
+    hyp = pytest.importorskip("hypothesis")
+    st = pytest.importorskip("hypothesis.strategies")
+    sym = st.text(alphabet="abc", min_size=1, max_size=4).map(str.encode)
+    tables = st.lists(st.tuples(sym, sym), min_size=0, max_size=12)
+    texts_ = st.lists(st.text(alphabet="abc", min_size=0, max_size=40).map(str.encode), min_size=1, max_size=6)
+    counter = [0]
+
+    @hyp.settings(max_examples=150, deadline=None, suppress_health_check=list(hyp.HealthCheck))
+    @hyp.given(merges=tables, texts=texts_, drop=st.integers(0, 3))
+    def check(merges, texts, drop):
+        counter[0] += 1
+        d = tmp_path / ("t%d" % counter[0])
+        d.mkdir()
+        toks = [b"?", b"<s>", b"</s>", b"a", b"b", b"c"]
+        for i, (x, y) in enumerate(merges):
+            if x + y not in toks and i % 4 != drop:
+                toks.append(x + y)
+        tf.write_files(str(d), toks, merges, 1, 2, None)
+        ours, ref = t12.Tokenizer(str(d)), RefTokenizer(str(d))
+        try:
+            for text in texts:
+                assert ours.tokenize(text) == ref.tokenize(text), (merges, text)
+        finally:
+            ours.close()
+
+    check()
