@@ -143,3 +143,26 @@ def test_models_this_build_does_not_read_fall_through_to_the_bpe_tables(t12, tmp
     tok = t12.Tokenizer(str(tmp_path))                      # like the reference: the second backend gets its turn
     assert tok.type == 1
     tok.close()
+
+
+@pytest.mark.parametrize("name", ["llama_like", "defaults"])
+def test_arbitrary_unicode_text_equals_the_library(t12, tmp_path, name):
+    """Property test (hypothesis): any Unicode text -- blanks of every kind, control characters, astral code points,
+    the escaped-blank character itself -- encodes to the library's ids and decodes to the library's text."""
+    hyp = pytest.importorskip("hypothesis")
+    st = pytest.importorskip("hypothesis.strategies")
+    proto, words = train(11, **CONFIGS[name])
+    ours, sp = load_both(t12, tmp_path, proto)
+    alphabet = st.one_of(st.sampled_from(list("abcdefghij éß \t\n" + SPACE + "<>0x/")), st.characters(blacklist_categories=("Cs",)))
+
+    @hyp.settings(max_examples=300, deadline=None, suppress_health_check=list(hyp.HealthCheck))
+    @hyp.given(text=st.text(alphabet=alphabet, max_size=60))
+    def check(text):
+        want = sp.encode(text)
+        assert ours.tokenize(text)[1:] == want, (text, sp.encode(text, out_type=str))
+        assert ours.detokenize(want) == sp.decode(want).encode(), text
+
+    try:
+        check()
+    finally:
+        ours.close()
