@@ -496,7 +496,7 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
                 const uint4* kr = (const uint4*)(kbase + (size_t)(c0 + tp) * kv_dim + lh * (HD / 2));
 #pragma unroll
                 for (int u = 0; u < KS; u++) kk_pre[nb][u] = kr[u];
-                kscale_pre[nb] = skb[(size_t)(c0 + tp) * n_head_kv] * scale;
+                kscale_pre[nb] = skb[(size_t)(c0 + tp) * n_head_kv];     // as stored; multiplied where it is used
             }
         }
     }
@@ -634,7 +634,7 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
     t12_u32x4 vreg[VP];     // (a native vector type: the compiler keeps this loop-carried array in registers)
     float vsc[OWN][ATT_TILE / 64], vsc_n[OWN][ATT_TILE / 64];
     uint4 kk[2][WIDE ? KS : 1];
-    float kscale[2] = {0.0f, 0.0f};
+    float kscale[2] = {0.0f, 0.0f};      // K scales as loaded: nothing touches a requested value before its tile comes up
     // Requests of the long-context form.  Every tile's K rows, V scales and first 128 V rows are asked for one tile
     // ahead (the registers they land in are free by then), its other 128 V rows during its softmax phase: no
     // memory latency stays exposed inside a workgroup.
@@ -651,12 +651,12 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
                 } else if (FUSE && first && t == newpos) {
 #pragma unroll
                     for (int u = 0; u < KS; u++) kk[nb][u] = ((const uint4*)(knew8 + lh * (HD / 2)))[u];
-                    kscale[nb] = knew_scale * scale;
+                    kscale[nb] = knew_scale;
                 } else {
                     const uint4* kr = (const uint4*)(kbase + (size_t)t * kv_dim + lh * (HD / 2));
 #pragma unroll
                     for (int u = 0; u < KS; u++) kk[nb][u] = kr[u];
-                    kscale[nb] = skb[(size_t)t * n_head_kv] * scale;
+                    kscale[nb] = skb[(size_t)t * n_head_kv];
                 }
             }
         }
@@ -714,14 +714,9 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
                     const int h = 4 * lh + r;
                     if (h < RATIO)
                         ps[h * ATT_TILE + tp] = ((float)sacc[r] + ((float)sacc[4 + r] + (float)sacc[8 + r] * (1.0f / 254.0f)) *
-                                                                      (1.0f / 254.0f)) * (qscale[h] * kscale[nb]);
+                                                                      (1.0f / 254.0f)) * (qscale[h] * (kscale[nb] * scale));
                 }
             }
-        }
-        // the next tile's K rows and V scales travel under the rest of this tile
-        if (has_next) {
-            issue_k(t0n, tln, false);
-            issue_vsc(t0n, tln, vsc_n);
         }
         } else {
         // ---- phase 1
@@ -768,7 +763,13 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
                 const int idx = tid + 256 * x;
                 *(t12_u32x4*)(vth + (idx / CH) * VSTR + (idx % CH) * 16) = vreg[x];
             }
-            if (128 < tl) issue_v(t0, tl, 1);                       // the other 128 rows: in flight under the softmax phase
+            // requests, after the wait for this tile's V rows so that it does not cover them: the next tile's K rows and
+            // V scales, and this tile's other 128 V rows, travel under the softmax phase
+            if (has_next) {
+                issue_k(t0n, tln, false);
+                issue_vsc(t0n, tln, vsc_n);
+            }
+            if (128 < tl) issue_v(t0, tl, 1);
             else if (has_next) issue_v(t0n, tln, 0);                 // (only the last tile of a chunk can be this short)
             __syncthreads();
             // ---- phase 2, one wave per head: tile maximum, rescale factor, probabilities and their sum; the weights
@@ -837,6 +838,12 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
                             const int idx = tid + 256 * x;
                             *(t12_u32x4*)(vth + (idx / CH) * VSTR + (idx % CH) * 16) = vreg[x];
                         }
+                        // the next tile's V scales were requested before the rows just written, so they are here:
+                        // taken over now, nothing is left to wait for at the end of the tile
+#pragma unroll
+                        for (int j = 0; j < OWN; j++)
+#pragma unroll
+                            for (int i = 0; i < ATT_TILE / 64; i++) vsc[j][i] = vsc_n[j][i];
                         if (has_next) issue_v(t0n, tln, 0);           // the next tile's first 128 V rows
                         __syncthreads();
                     }
@@ -863,11 +870,7 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
                 const int h = min(4 * lh + r, RATIO - 1);
                 o_w[r] = o_w[r] * corr_s[h] + ((float)oacc[r] + (float)oacc[4 + r] * (1.0f / 254.0f)) * wscale_s[h];
             }
-#pragma unroll
-            for (int j = 0; j < OWN; j++)
-#pragma unroll
-                for (int i = 0; i < ATT_TILE / 64; i++) vsc[j][i] = vsc_n[j][i];
-            __syncthreads();
+            __syncthreads();                                         // (a tile of 128 positions or fewer is a chunk's last: no scales to take over)
         } else {
             __syncthreads();
             // ---- phases 2 + 3, one wave per head
