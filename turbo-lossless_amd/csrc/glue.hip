@@ -17,6 +17,7 @@
 #include <cmath>
 #include <cstring>
 #include <mutex>
+#include <type_traits>
 #include <vector>
 
 #include "t12_device.h"
@@ -426,7 +427,7 @@ struct AttnSplit {
 };
 
 template <int HD, int RATIO, bool FUSE = false, bool SPLIT = false, bool WIDE = false>
-__global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kernel(const float* __restrict__ q, const int8_t* __restrict__ ck,
+__global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kernel(const float* __restrict__ q, const int8_t* __restrict__ ck,
                                                         const int8_t* __restrict__ cv, const float* __restrict__ sk,
                                                         const float* __restrict__ sv, uint16_t* __restrict__ out,
                                                         const int* __restrict__ positions, int seq_len_arg,
@@ -688,18 +689,22 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
         issue_v(c0, tl0, 0);
     }
 
-    for (int t0 = c0; t0 < c1; t0 += ATT_TILE) {
-        const int tl = min(ATT_TILE, c1 - t0);
+    // One tile.  full_c = std::true_type: this tile and the next one are complete, so every request of the tile is issued
+    // without a condition around it.  (The compiler counts outstanding loads per path: behind a load that sits under a
+    // condition it must assume that none of the later ones was issued, and then waits for all of them.)
+    auto tile = [&](const int t0, auto full_c) __attribute__((always_inline)) {
+        constexpr bool FULLT = decltype(full_c)::value;
+        const int tl = FULLT ? ATT_TILE : min(ATT_TILE, c1 - t0);
         const int t0n = t0 + ATT_TILE;
-        const bool has_next = t0n < c1;
-        const int tln = min(ATT_TILE, c1 - t0n);
+        const bool has_next = FULLT || t0n < c1;
+        const int tln = FULLT ? ATT_TILE : min(ATT_TILE, c1 - t0n);
         if constexpr (WIDE) {
         // ---- phase 1: scores of 64 positions per wave, two blocks of 32, KS INT8 MFMAs each
         // (the K rows, V rows and V scales of this tile were requested during the previous tile, or before the loop)
 #pragma unroll
         for (int nb = 0; nb < 2; nb++) {
             const int tp = wave * 64 + nb * 32 + ln;
-            if (wave * 64 + nb * 32 < tl) {
+            if (FULLT || wave * 64 + nb * 32 < tl) {
                 t12_i32x16 sacc;
 #pragma unroll
                 for (int r = 0; r < 16; r++) sacc[r] = 0;
@@ -765,12 +770,35 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
             }
             // requests, after the wait for this tile's V rows so that it does not cover them: the next tile's K rows and
             // V scales, and this tile's other 128 V rows, travel under the softmax phase
-            if (has_next) {
-                issue_k(t0n, tln, false);
-                issue_vsc(t0n, tln, vsc_n);
+            if constexpr (FULLT) {
+#pragma unroll
+                for (int nb = 0; nb < 2; nb++) {
+                    const int t = t0n + wave * 64 + nb * 32 + ln;
+                    const uint4* kr = (const uint4*)(kbase + (size_t)t * kv_dim + lh * (HD / 2));
+#pragma unroll
+                    for (int u = 0; u < KS; u++) kk[nb][u] = kr[u];
+                    kscale[nb] = skb[(size_t)t * n_head_kv];
+                }
+#pragma unroll
+                for (int j = 0; j < OWN; j++)
+#pragma unroll
+                    for (int i = 0; i < ATT_TILE / 64; i++) {
+                        const float s = svb[(size_t)(t0n + lane + 64 * i) * n_head_kv];
+                        vsc_n[j][i] = (RATIO % 4 == 0 || wave + 4 * j < RATIO) ? s : 0.0f;
+                    }
+#pragma unroll
+                for (int x = 0; x < VP; x++) {
+                    const int idx = tid + 256 * x;
+                    vreg[x] = *(const t12_u32x4*)(vbase + (size_t)(t0 + 128 + idx / CH) * kv_dim + (idx % CH) * 16);
+                }
+            } else {
+                if (has_next) {
+                    issue_k(t0n, tln, false);
+                    issue_vsc(t0n, tln, vsc_n);
+                }
+                if (128 < tl) issue_v(t0, tl, 1);
+                else if (has_next) issue_v(t0n, tln, 0);             // (only the last tile of a chunk can be this short)
             }
-            if (128 < tl) issue_v(t0, tl, 1);
-            else if (has_next) issue_v(t0n, tln, 0);                 // (only the last tile of a chunk can be this short)
             __syncthreads();
             // ---- phase 2, one wave per head: tile maximum, rescale factor, probabilities and their sum; the weights
             //      w = p * v_scale of the tile as two INT8 limbs, w ~ wscale (a1 + a2 / 254)
@@ -829,7 +857,7 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
             const int8_t* vsrc = vth + (s16 >> 1) * VSTR + wave * 32 + ((lane >> 4) & 1) * 16 + (s16 & 1) * 8;
 #pragma unroll
             for (int half = 0; half < 2; half++) {
-                if (half * 128 < tl) {                               // workgroup-uniform
+                if (FULLT || half * 128 < tl) {                      // workgroup-uniform
                     if (half == 1) {
                         // second half of the tile through the same LDS rows
                         __syncthreads();                             // every wave is done with the first half
@@ -844,7 +872,13 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
                         for (int j = 0; j < OWN; j++)
 #pragma unroll
                             for (int i = 0; i < ATT_TILE / 64; i++) vsc[j][i] = vsc_n[j][i];
-                        if (has_next) issue_v(t0n, tln, 0);           // the next tile's first 128 V rows
+                        if constexpr (FULLT) {
+#pragma unroll
+                            for (int x = 0; x < VP; x++) {
+                                const int idx = tid + 256 * x;
+                                vreg[x] = *(const t12_u32x4*)(vbase + (size_t)(t0n + idx / CH) * kv_dim + (idx % CH) * 16);
+                            }
+                        } else if (has_next) issue_v(t0n, tln, 0);    // the next tile's first 128 V rows
                         __syncthreads();
                     }
                     if (wave < NBLK) {
@@ -932,6 +966,12 @@ __global__ __launch_bounds__(256, (!FUSE && !WIDE) ? 4 : 1) void attn_fast_kerne
             }
             __syncthreads();
         }
+    };
+    {
+        int t0 = c0;
+        if constexpr (WIDE)
+            for (; t0 + 2 * ATT_TILE <= c1; t0 += ATT_TILE) tile(t0, std::true_type{});
+        for (; t0 < c1; t0 += ATT_TILE) tile(t0, std::false_type{});
     }
     if constexpr (WIDE) {
         // ---- every lane holds finished sums of its dim for up to four heads; the owners publish maximum and sum
