@@ -562,7 +562,10 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
                 else if (VLDS && rel < ATT_TILE) vts[rel] = amax / 127.0f;
             }
         }
-        __threadfence();      // later tiles read the new row back through the cache pointers
+        // later tiles read the new row back through the cache pointers: only this workgroup does (the chunk that
+        // stores the row is the chunk that holds it), so workgroup scope is enough -- a device-scope fence here
+        // writes back and invalidates the L2 in every launch
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
         // the prefetched V tile: registers -> LDS (row-major, 16-byte pieces)
 #pragma unroll
         for (int x = 0; x < VPRE; x++) {
