@@ -72,6 +72,7 @@ __device__ __forceinline__ float patch_partial(const T12Segment& sg, int row, in
 // in 1024-column tiles, software pipelined D tiles deep through a register
 // ring: every lane keeps D*R 128-bit + D*R 64-bit loads in flight.
 // Order inside a wave, arranged so that no dependent load chain is exposed:
+//   (0) the activations (bf16 input: up to SU 16-byte pieces per thread),
 //   (1) CSR row pointers of the R rows (one vector load, lanes 0..R),
 //   (2) the first D tiles of weight loads,
 //   (3) the workgroup stages the activations into LDS, barrier,
@@ -125,6 +126,21 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
     for (int r = 0; r < R; r++)
         be2r[r] = t12_opaque(((uint32_t)SEG(r).base_exp << 7) | ((uint32_t)SEG(r).base_exp << 23));
 
+    // The activations are requested FIRST: they come out of the L2 (every workgroup reads the same vector) and so
+    // arrive before the weight tiles requested behind them; loads complete in order, so requested after the tiles
+    // they would wait for HBM, and staged in a loop they would cost one round trip per pass.  Piece q = 8 columns.
+    constexpr int SU = 4;                      // pieces per thread requested up front (16 * NW * 64 * SU / 8 columns)
+    uint4 xpre[SU];
+    if (NORM == 0) {
+#pragma unroll
+        for (int u = 0; u < SU; u++) {
+            const int k = (tid + u * NW * 64) * 8;
+            xpre[u] = make_uint4(0, 0, 0, 0);
+            if (u == 0 || u * NW * 64 * 8 < K)                       // workgroup-uniform
+                xpre[u] = *(const uint4*)(p.act + min(k, K - 8));    // (clamped: columns >= K are zeroed below)
+        }
+    }
+
     // CSR row pointers: lane 2r holds the begin and lane 2r+1 the end of row r's escape slice
     int ro = 0;
     if (live && lane < 2 * R) {
@@ -167,7 +183,14 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
     }
 
     if (NORM == 0) {
-        for (int q = tid; q < nchunk * 128; q += NW * 64) {
+#pragma unroll
+        for (int u = 0; u < SU; u++) {
+            const int q = tid + u * NW * 64;
+            if (q < nchunk * 128)
+                lds_act[(q >> 7) * 128 + (q & 1) * 64 + ((q & 127) >> 1)] =
+                    t12_pair_acts(q * 8 < K ? xpre[u] : make_uint4(0, 0, 0, 0));
+        }
+        for (int q = tid + SU * NW * 64; q < nchunk * 128; q += NW * 64) {     // K beyond the pieces requested up front
             const int k = q * 8;
             uint4 v = make_uint4(0, 0, 0, 0);
             if (k < K) v = *(const uint4*)(p.act + k);
