@@ -141,6 +141,25 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
         }
     }
 
+    // NORM: the same for the fp32 residual stream, its addend and the norm weights (8 columns per piece, 2 pieces per thread)
+    float4 npre[NORM ? 2 : 1][2], rpre[NORM == 2 ? 2 : 1][2], wpre[NORM ? 2 : 1][2];
+    if (NORM != 0) {
+#pragma unroll
+        for (int gi = 0; gi < 2; gi++) {
+            const int k = min((tid + gi * NW * 64) * 8, K - 8);      // (clamped: pieces beyond K are not used)
+            if (gi == 0 || NW * 64 * 8 < K) {                        // workgroup-uniform
+                npre[gi][0] = *(const float4*)(p.nx + k);
+                npre[gi][1] = *(const float4*)(p.nx + k + 4);
+                if (NORM == 2) {
+                    rpre[gi][0] = *(const float4*)(p.nres + k);
+                    rpre[gi][1] = *(const float4*)(p.nres + k + 4);
+                }
+                wpre[gi][0] = *(const float4*)(p.nw + k);
+                wpre[gi][1] = *(const float4*)(p.nw + k + 4);
+            }
+        }
+    }
+
     // CSR row pointers: lane 2r holds the begin and lane 2r+1 the end of row r's escape slice
     int ro = 0;
     if (live && lane < 2 * R) {
@@ -206,11 +225,11 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
 #pragma unroll
             for (int e = 0; e < 8; e++) v[gi][e] = 0.0f;
             if (k < K) {
-                const float4 a = *(const float4*)(p.nx + k), b = *(const float4*)(p.nx + k + 4);
+                const float4 a = npre[gi][0], b = npre[gi][1];
                 v[gi][0] = a.x; v[gi][1] = a.y; v[gi][2] = a.z; v[gi][3] = a.w;
                 v[gi][4] = b.x; v[gi][5] = b.y; v[gi][6] = b.z; v[gi][7] = b.w;
                 if (NORM == 2) {
-                    const float4 c = *(const float4*)(p.nres + k), d = *(const float4*)(p.nres + k + 4);
+                    const float4 c = rpre[gi][0], d = rpre[gi][1];
                     v[gi][0] += c.x; v[gi][1] += c.y; v[gi][2] += c.z; v[gi][3] += c.w;
                     v[gi][4] += d.x; v[gi][5] += d.y; v[gi][6] += d.z; v[gi][7] += d.w;
                     if (blockIdx.x == 0 && p.hidden_out) {
@@ -236,7 +255,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
             if (q < nchunk * 128) {
                 uint4 y = make_uint4(0, 0, 0, 0);
                 if (k < K) {
-                    const float4 wa = *(const float4*)(p.nw + k), wb = *(const float4*)(p.nw + k + 4);
+                    const float4 wa = wpre[gi][0], wb = wpre[gi][1];
                     y.x = t12_f32_to_bf16(v[gi][0] * rn * wa.x) | ((uint32_t)t12_f32_to_bf16(v[gi][1] * rn * wa.y) << 16);
                     y.y = t12_f32_to_bf16(v[gi][2] * rn * wa.z) | ((uint32_t)t12_f32_to_bf16(v[gi][3] * rn * wa.w) << 16);
                     y.z = t12_f32_to_bf16(v[gi][4] * rn * wb.x) | ((uint32_t)t12_f32_to_bf16(v[gi][5] * rn * wb.y) << 16);

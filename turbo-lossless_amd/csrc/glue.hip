@@ -123,6 +123,64 @@ __global__ __launch_bounds__(1024) void rms_norm_kernel(float* __restrict__ x, c
         y[off + i] = t12_f32_to_bf16(x[off + i] * r * w[i]);
 }
 
+// The same for rows of 4 n' <= 8192 values with 16-byte aligned operands: every thread owns one or two pieces of four
+// neighbouring values and requests everything it needs for them -- all partial rows, the residual, the norm weights --
+// in one go as 128-bit loads, so the row costs one memory round trip, a block sum and the stores.  NZ = most partial
+// rows the instance unrolls.  Sums per element are formed exactly as above (ascending partials, then the residual).
+template <bool ADD, bool PART, int NZ>
+__global__ __launch_bounds__(1024) void rms_norm_vec_kernel(float* __restrict__ x, const float* __restrict__ res,
+                                                            const float* __restrict__ w, uint16_t* __restrict__ y,
+                                                            int n, float eps, const float* __restrict__ part,
+                                                            int nsplit, size_t split_stride, int ld)
+{
+    __shared__ float red[17];
+    constexpr int NP = 2;
+    const size_t off = (size_t)blockIdx.x * n;
+    const float* prow = PART ? part + (size_t)blockIdx.x * ld : nullptr;
+    float4 v[NP], wv[NP];
+    float ss = 0.0f;
+#pragma unroll
+    for (int u = 0; u < NP; u++) {
+        const int i = (threadIdx.x + u * blockDim.x) * 4;
+        v[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        wv[u] = v[u];
+        if (i < n) {
+            float4 pz[PART ? NZ : 1], r4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f), t;
+            if (PART) {
+#pragma unroll
+                for (int z = 0; z < NZ; z++)
+                    pz[z] = z < nsplit ? *(const float4*)(prow + (size_t)z * split_stride + i) : r4;
+            } else {
+                pz[0] = *(const float4*)(x + off + i);
+            }
+            if (ADD) r4 = *(const float4*)(res + off + i);
+            wv[u] = *(const float4*)(w + i);
+            if (PART) {
+                t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+                for (int z = 0; z < NZ; z++)
+                    if (z < nsplit) { t.x += pz[z].x; t.y += pz[z].y; t.z += pz[z].z; t.w += pz[z].w; }
+            } else {
+                t = pz[0];
+            }
+            if (ADD) { t.x += r4.x; t.y += r4.y; t.z += r4.z; t.w += r4.w; }
+            if (ADD || PART) *(float4*)(x + off + i) = t;
+            v[u] = t;
+            ss += t.x * t.x + t.y * t.y + t.z * t.z + t.w * t.w;
+        }
+    }
+    ss = block_reduce<false>(ss, red);
+    const float r = rsqrtf(ss / (float)n + eps);
+#pragma unroll
+    for (int u = 0; u < NP; u++) {
+        const int i = (threadIdx.x + u * blockDim.x) * 4;
+        if (i < n)
+            *(uint2*)(y + off + i) =
+                make_uint2(t12_f32_to_bf16(v[u].x * r * wv[u].x) | ((uint32_t)t12_f32_to_bf16(v[u].y * r * wv[u].y) << 16),
+                           t12_f32_to_bf16(v[u].z * r * wv[u].z) | ((uint32_t)t12_f32_to_bf16(v[u].w * r * wv[u].w) << 16));
+    }
+}
+
 // ----------------------------------------------------------------- SiLU*mul
 // out = bf16( g / (1 + exp(-g)) * up )   (kernels.hip:447-459)
 __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
@@ -1395,6 +1453,20 @@ void launch_embed_lookup(const int16_t* embd_table, const int* token_ids, float*
     report("embed_lookup");
 }
 
+// Rows the 128-bit form takes: a multiple of 4 values, at most 8192, every operand 16-byte aligned.
+static bool norm_vec_ok(int n, const void* x, const void* res, const void* w, const void* y, const void* part,
+                        size_t split_stride, int ld)
+{
+    auto al = [](const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; };
+    return n >= 4 && n % 4 == 0 && n <= 8192 && al(x, 16) && al(res, 16) && al(w, 16) && al(y, 8) && al(part, 16) &&
+           split_stride % 4 == 0 && ld % 4 == 0;
+}
+static int norm_vec_threads(int n)
+{
+    const int t = (n / 4 + 63) / 64 * 64;
+    return t > 1024 ? 1024 : t;
+}
+
 static int norm_threads(int n)
 {
     int t = (n + 7) / 8;                   // 8 values per thread stay in registers
@@ -1405,16 +1477,25 @@ static int norm_threads(int n)
 void launch_rms_norm_bf16_batch(const float* x, const float* weight, int16_t* y, int n, float eps, int batch_size,
                                 hipStream_t stream)
 {
-    hipLaunchKernelGGL(rms_norm_kernel<false>, dim3(batch_size), dim3(norm_threads(n)), 0, stream, (float*)x,
-                       (const float*)nullptr, weight, (uint16_t*)y, n, eps);
+    if (norm_vec_ok(n, x, nullptr, weight, y, nullptr, 0, 0))
+        hipLaunchKernelGGL((rms_norm_vec_kernel<false, false, 1>), dim3(batch_size), dim3(norm_vec_threads(n)), 0, stream,
+                           (float*)x, (const float*)nullptr, weight, (uint16_t*)y, n, eps, (const float*)nullptr, 0,
+                           (size_t)0, 0);
+    else
+        hipLaunchKernelGGL(rms_norm_kernel<false>, dim3(batch_size), dim3(norm_threads(n)), 0, stream, (float*)x,
+                           (const float*)nullptr, weight, (uint16_t*)y, n, eps);
     report("rms_norm");
 }
 
 void launch_add_rms_norm_bf16_batch(float* x, const float* residual, const float* weight, int16_t* y, int n, float eps,
                                     int batch_size, hipStream_t stream)
 {
-    hipLaunchKernelGGL(rms_norm_kernel<true>, dim3(batch_size), dim3(norm_threads(n)), 0, stream, x, residual, weight,
-                       (uint16_t*)y, n, eps);
+    if (norm_vec_ok(n, x, residual, weight, y, nullptr, 0, 0))
+        hipLaunchKernelGGL((rms_norm_vec_kernel<true, false, 1>), dim3(batch_size), dim3(norm_vec_threads(n)), 0, stream, x,
+                           residual, weight, (uint16_t*)y, n, eps, (const float*)nullptr, 0, (size_t)0, 0);
+    else
+        hipLaunchKernelGGL(rms_norm_kernel<true>, dim3(batch_size), dim3(norm_threads(n)), 0, stream, x, residual, weight,
+                           (uint16_t*)y, n, eps);
     report("add_rms_norm");
 }
 
@@ -1427,6 +1508,20 @@ void launch_sum_add_rms_norm_bf16_batch(float* x, const float* partials, int nsp
     if (nsplit < 1 || nsplit > T12_MAX_KSPLIT || !partials) {
         t12_set_error("sum_add_rms_norm: nsplit %d outside 1..%d or null partials", nsplit, T12_MAX_KSPLIT);
         fprintf(stderr, "turbo12: %s\n", t12_last_error());
+        return;
+    }
+    if (norm_vec_ok(n, x, residual, weight, y, partials, split_stride, ld)) {
+        const dim3 g(batch_size), b(norm_vec_threads(n));
+        if (nsplit <= 4)
+            hipLaunchKernelGGL((rms_norm_vec_kernel<true, true, 4>), g, b, 0, stream, x, residual, weight, (uint16_t*)y, n,
+                               eps, partials, nsplit, split_stride, ld);
+        else if (nsplit <= 8)
+            hipLaunchKernelGGL((rms_norm_vec_kernel<true, true, 8>), g, b, 0, stream, x, residual, weight, (uint16_t*)y, n,
+                               eps, partials, nsplit, split_stride, ld);
+        else
+            hipLaunchKernelGGL((rms_norm_vec_kernel<true, true, T12_MAX_KSPLIT>), g, b, 0, stream, x, residual, weight,
+                               (uint16_t*)y, n, eps, partials, nsplit, split_stride, ld);
+        report("sum_add_rms_norm");
         return;
     }
     // one workgroup per row has every partial of the row to fetch: as many lanes as the row allows
