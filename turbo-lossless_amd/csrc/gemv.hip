@@ -269,8 +269,10 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
     if (!live) return;
 
     // escape entries: lane l takes entry beg + l of each row
+    // (kept as loaded until the row's sum is formed: arithmetic on a requested value right here would make the wave
+    // wait for it, a full memory latency, before it consumes its first tile)
     int pcol[R];
-    float pdelta[R];
+    int pcorrect[R], pwrong[R];              // (the arrays' own 16-bit integers, widened by the load itself)
     int pend[R], pnext[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -278,11 +280,11 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
         pend[r] = end;
         pnext[r] = beg + T12_WAVE;
         pcol[r] = -1;
-        pdelta[r] = 0.0f;
+        pcorrect[r] = pwrong[r] = 0;
         if (beg + lane < end) {                          // end > beg only when the tensor has a list
             pcol[r] = SEG(r).cols[beg + lane];
-            pdelta[r] = t12_bf16_to_f32((uint16_t)SEG(r).correct[beg + lane]) -
-                        t12_bf16_to_f32((uint16_t)SEG(r).wrong[beg + lane]);
+            pcorrect[r] = SEG(r).correct[beg + lane];
+            pwrong[r] = SEG(r).wrong[beg + lane];
         }
     }
 
@@ -323,7 +325,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
         tot[r] = 0.0f;
         if (ROW(r) < M) {                                // wave-uniform
             float v = acc[r];
-            if (pcol[r] >= 0) v += pdelta[r] * lds_act_at(lds_act, pcol[r]);
+            if (pcol[r] >= 0) v += (t12_bf16_to_f32((uint16_t)pcorrect[r]) - t12_bf16_to_f32((uint16_t)pwrong[r])) * lds_act_at(lds_act, pcol[r]);
             for (int q = pnext[r] + lane; q < pend[r]; q += T12_WAVE)     // rows with > 64 escapes
                 v += (t12_bf16_to_f32((uint16_t)SEG(r).correct[q]) - t12_bf16_to_f32((uint16_t)SEG(r).wrong[q])) *
                      lds_act_at(lds_act, SEG(r).cols[q]);
