@@ -731,14 +731,17 @@ int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, in
     }
     p.blk_start[nseg] = tiles;
     // K split: fill the chip.  A 256-row batch tile needs a whole CU (LDS, accumulators);
-    // smaller batch tiles fit 2-4 workgroups per CU.  Every split keeps >= 4 stages.
+    // smaller batch tiles fit 2-4 workgroups per CU.  Every split keeps >= 4 stages; with 256-row batch tiles
+    // >= 8: a 4096 x 4096 tensor then runs as 128 workgroups in the time 256 take, and leaves half the partial
+    // sums (4 x 4 MB instead of 8 x 4 MB at B = 256) for the kernel that adds them up.
     const int btiles = B > 128 ? (B + 255) / 256 : 1;
     const int per_cu = B > 64 ? 1 : 2;
     const int want = 256 * per_cu;
     int ks = 1;
+    const int min_stages = B > 128 ? 16 : 8;
     if (g_gemm_ksplit > 0) ks = g_gemm_ksplit < T12_MAX_KSPLIT ? g_gemm_ksplit : T12_MAX_KSPLIT;
     else
-        while (tiles * btiles * ks * 4 < want * 3 && K / (ks * 2) >= 8 * KC && ks < T12_MAX_KSPLIT) ks *= 2;
+        while (tiles * btiles * ks * 4 < want * 3 && K / (ks * 2) >= min_stages * KC && ks < T12_MAX_KSPLIT) ks *= 2;
     int kslice = (((K + 2 * KC - 1) / (2 * KC) + ks - 1) / ks) * 2 * KC;      // whole windows of two stages
     ks = (K + kslice - 1) / kslice;
     p.ksplit = ks;
