@@ -1593,9 +1593,9 @@ void launch_rope_store_attention(float* q, float* k, const float* v, int8_t* kv_
                                  hipStream_t stream)
 {
     // Fusing pays when every workgroup stores its own cache slot (one sequence, or per-sequence caches) and
-    // the launch is small enough to be a chain of latencies: the fused kernel stages a V tile in LDS and holds
-    // prefetched rows in registers, so only two or three of its workgroups fit a CU (measured at B = 256 on
-    // per-sequence caches: 221 us fused against 37 us + 9 us for the two launches at 150 positions).  Lock-step
+    // the launch is small enough to be a chain of latencies: the fused kernel holds prefetched rows in more
+    // registers, so only two of its workgroups fit a CU (measured at B = 256 on per-sequence caches: 35 us
+    // fused against 26 + 7 us for the two launches at 150 positions, 256 against 248 + 7 us at 2000).  Lock-step
     // copies on a shared cache (kv_stride = 0, batch > 1) would store the same slot from every workgroup.
     if (attn_has_fast(n_head, n_head_kv, head_dim) && (batch_size == 1 || (kv_stride != 0 && batch_size * n_head_kv <= 256))) {
         AttnFuse fz;
