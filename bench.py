@@ -360,10 +360,13 @@ def run_attention(args, t12, torch, dev):
     cur = torch.cuda.current_stream()
     g = torch.Generator(device=dev)
     g.manual_seed(77)
-    cases = [(256, 2048, 2000), (256, 2048, 150), (64, 8192, 8000), (16, 2048, 1000), (1, 8192, 8000), (1, 2048, 2000),
-             (1, 2048, 150)]
+    # (batch, positions per region, context, head-major regions): the first three per-sequence cases also in the layout
+    # the engine keeps its per-sequence caches in ([kv head][position][dim] instead of the reference's [position][kv head][dim])
+    cases = [(256, 2048, 2000, False), (256, 2048, 150, False), (64, 8192, 8000, False), (16, 2048, 1000, False),
+             (1, 8192, 8000, False), (1, 2048, 2000, False), (1, 2048, 150, False),
+             (256, 2048, 2000, True), (256, 2048, 150, True), (64, 8192, 8000, True)]
     out_cases = {}
-    for B, S, ctx in cases:
+    for B, S, ctx, head_major in cases:
         kc = torch.randint(-127, 128, (B, S, kv_dim), dtype=torch.int8, device=dev, generator=g)
         vc = torch.randint(-127, 128, (B, S, kv_dim), dtype=torch.int8, device=dev, generator=g)
         ks = torch.rand((B, S, nkv), device=dev, generator=g) / 127 + 0.004
@@ -375,15 +378,19 @@ def run_attention(args, t12, torch, dev):
         pos = torch.full((B,), ctx - 1, dtype=torch.int32, device=dev)
 
         def step():
-            t12.lib.launch_rope_store_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), kc.data_ptr(), vc.data_ptr(),
-                                                ks.data_ptr(), vs.data_ptr(), out.data_ptr(),
-                                                pos.data_ptr() if B > 1 else None, ctx - 1, nh, nkv, hd, theta,
-                                                1.0 / np.sqrt(hd), B, S * kv_dim if B > 1 else 0, cur.cuda_stream)
+            head = (q.data_ptr(), k.data_ptr(), v.data_ptr(), kc.data_ptr(), vc.data_ptr(), ks.data_ptr(), vs.data_ptr(),
+                    out.data_ptr(), pos.data_ptr() if B > 1 else None, ctx - 1, nh, nkv, hd, theta, 1.0 / np.sqrt(hd), B,
+                    S * kv_dim if B > 1 else 0)
+            if head_major:                       # (random contents: the same buffers serve as regions of either layout)
+                t12.lib.launch_rope_store_attention_regions(*head, S, cur.cuda_stream)
+            else:
+                t12.lib.launch_rope_store_attention(*head, cur.cuda_stream)
         for _ in range(max(args.warmup, 1)):
             step()
         _, ms = timed(torch, cur, step, args.steps)
         nbytes = B * ctx * (2 * kv_dim + 8 * nkv)            # INT8 K and V rows + their fp32 scales
-        out_cases["b%d_ctx%d" % (B, ctx)] = {"us": ms * 1e3, "cache_MB": nbytes / 1e6, "GBps": nbytes / ms / 1e6}
+        out_cases["b%d_ctx%d%s" % (B, ctx, "_headmajor" if head_major else "")] = {
+            "us": ms * 1e3, "cache_MB": nbytes / 1e6, "GBps": nbytes / ms / 1e6}
         del kc, vc, ks, vs
     head = out_cases["b256_ctx2000"]
     return {

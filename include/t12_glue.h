@@ -124,6 +124,24 @@ void launch_rope_store_attention_partials(float* q, float* k, const float* v, in
                                           float scale, int batch_size, const float* partials, int nsplit,
                                           size_t split_stride, int ld, int kv_stride, hipStream_t stream);
 
+/* The two launches above on HEAD-MAJOR cache regions: a region holds region_positions rows per KV head, laid out
+ * [kv head][region_positions][head_dim] (scales [kv head][region_positions]) instead of the reference's
+ * [position][kv head][head_dim] (engine/model.h:58-63, the layout every other launcher here keeps).  The workgroup of a
+ * (sequence, KV head) then reads one contiguous stream; in the reference's layout it reads 128-byte pieces of rows that
+ * it shares with the other KV heads' workgroups.  kv_stride: element distance between regions, as above (a region
+ * still has region_positions * n_head_kv * head_dim elements).  Positions must stay below region_positions.  The
+ * engine keeps its per-sequence caches this way.  No counterpart in the reference. */
+void launch_rope_store_attention_regions(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v, float* scale_k,
+                                         float* scale_v, int16_t* output, const int* positions, int position, int n_head,
+                                         int n_head_kv, int head_dim, float theta, float scale, int batch_size,
+                                         int kv_stride, int region_positions, hipStream_t stream);
+void launch_rope_store_attention_partials_regions(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v,
+                                                  float* scale_k, float* scale_v, int16_t* output, const int* positions,
+                                                  int position, int n_head, int n_head_kv, int head_dim, float theta,
+                                                  float scale, int batch_size, const float* partials, int nsplit,
+                                                  size_t split_stride, int ld, int kv_stride, int region_positions,
+                                                  hipStream_t stream);
+
 /* Benchmark switch.  0: always the general attention kernel.  1 (default): shapes with a specialised kernel
  * (head_dim 128 with GQA ratio 1/2/4/8, head_dim 64 with ratio 1/4) use it in its INT8 MFMA form (scores and P.V by
  * v_mfma_i32_32x32x32_i8: Q in three INT8 limbs, the softmax weights in two, K and V as stored), and a launch without a

@@ -306,6 +306,76 @@ def test_per_sequence_caches_fused_and_from_partial_sums(t12, oracle, attn_mode,
     assert not torch.equal(oa[0], oa[1])
 
 
+@pytest.mark.parametrize("nh,nkv,hd,B,pos", [(32, 8, 128, 3, [70, 5, 33]), (32, 8, 128, 40, None), (8, 2, 32, 3, [1, 90, 64]),
+                                             (4, 4, 64, 2, [300, 17]), (32, 8, 128, 1, [1290]), (32, 8, 128, 2, [700, 700])])
+def test_head_major_regions_equal_the_reference_layout(t12, oracle, attn_mode, nh, nkv, hd, B, pos):
+    """launch_rope_store_attention_regions / _partials_regions work on regions laid out [kv head][position][dim]
+    (scales [kv head][position]).  On the transposed data they give bit-identical outputs, rotated q / k, and --
+    transposed back -- bit-identical caches and scales, for per-sequence regions with a position array (fused form at
+    small batches, separate launches at B = 40), for the launch fed by K-split partial sums, and for one region without a
+    position array (the context-split form at long contexts, lock-step rows)."""
+    rng = np.random.default_rng(hd + B)
+    theta = 500000.0
+    shared = B <= 2 and pos[0] == pos[-1] and pos[0] >= 700          # one region, no position array
+    if pos is None:
+        pos = [int(x) for x in rng.integers(0, 280, size=B)]
+    max_seq = max(pos) + 9
+    R = 1 if shared else B                                          # regions
+    q, k, v = make_qkv(rng, B, nh, nkv, hd)
+    if shared:
+        q[1:], k[1:], v[1:] = q[0], k[0], v[0]
+    kc = rng.integers(-127, 128, size=(R, max_seq, nkv, hd)).astype(np.int8)
+    vc = rng.integers(-127, 128, size=(R, max_seq, nkv, hd)).astype(np.int8)
+    ks = (rng.random((R, max_seq, nkv)).astype(np.float32) + 0.5) / 127
+    vs = (rng.random((R, max_seq, nkv)).astype(np.float32) + 0.5) / 127
+    hm = lambda a: np.ascontiguousarray(np.swapaxes(a, 1, 2))       # [R, pos, head, ...] <-> [R, head, pos, ...]
+    pd = torch.tensor(pos, dtype=torch.int32, device=dev())
+    sc = 1.0 / np.sqrt(hd)
+    kv_stride = 0 if shared else max_seq * nkv * hd
+    pptr = None if shared else pd.data_ptr()
+    nq, nk = nh * hd, nkv * hd
+    row = np.concatenate([q.reshape(B, -1), k.reshape(B, -1), v.reshape(B, -1)], axis=1).astype(np.float32)
+    p0 = (rng.standard_normal(row.shape) * 0.5).astype(np.float32)
+    if shared:
+        p0[1:] = p0[0]                                              # lock-step rows store one slot: bit-identical rows
+    p1 = (row - p0).astype(np.float32)
+    row = (p0 + p1).astype(np.float32)
+    q, k, v = row[:, :nq].copy(), row[:, nq:nq + nk].copy(), row[:, nq + nk:].copy()
+    ws = torch.from_numpy(np.stack([p0, p1])).to(dev())
+
+    def run(head_major, partials):
+        arrs = (q, k, v, hm(kc), hm(vc), hm(ks), hm(vs)) if head_major else (q, k, v, kc, vc, ks, vs)
+        f = [torch.from_numpy(a.copy()).to(dev()) for a in arrs]
+        o = torch.zeros((B, nq), dtype=torch.int16, device=dev())
+        head = [f[i].data_ptr() for i in range(7)] + [o.data_ptr(), pptr, max(pos), nh, nkv, hd, theta, sc, B]
+        if partials:
+            f[0].zero_(); f[1].zero_(); f[2].zero_()
+            tail = [ws.data_ptr(), 2, B * row.shape[1], row.shape[1], kv_stride]
+            if head_major:
+                t12.lib.launch_rope_store_attention_partials_regions(*head, *tail, max_seq, st(t12))
+            else:
+                t12.lib.launch_rope_store_attention_partials(*head, *tail, st(t12))
+        elif head_major:
+            t12.lib.launch_rope_store_attention_regions(*head, kv_stride, max_seq, st(t12))
+        else:
+            t12.lib.launch_rope_store_attention(*head, kv_stride, st(t12))
+        torch.cuda.synchronize()
+        if head_major:
+            for i in (3, 4, 5, 6):
+                f[i] = f[i].transpose(1, 2).contiguous()
+        return f, o
+
+    for partials in (False, True):
+        if partials and shared and B == 1:
+            continue                                                # (the K-split launch is a batch path)
+        a, oa = run(False, partials)
+        b, ob = run(True, partials)
+        assert not torch.equal(a[3], torch.from_numpy(kc).to(dev()))
+        for i in range(7):
+            assert torch.equal(a[i], b[i]), (partials, i)
+        assert torch.equal(oa, ob), partials
+
+
 @pytest.mark.parametrize("nh,nkv,hd,B,pos", [(32, 8, 128, 1, 1290), (32, 8, 128, 2, 700), (16, 4, 64, 3, 333)])
 def test_context_split_equals_single_pass(t12, oracle, nh, nkv, hd, B, pos):
     """A launch without a position array at a long context is split along the context (partial softmax per

@@ -72,6 +72,9 @@ _SIGS = {
     "launch_rope_store_attention": (None, [_vp] * 9 + [_i, _i, _i, _i, C.c_float, C.c_float, _i, _i, _vp]),
     "launch_rope_store_attention_partials": (None, [_vp] * 9 + [_i, _i, _i, _i, C.c_float, C.c_float, _i, _vp, _i,
                                                     C.c_size_t, _i, _i, _vp]),
+    "launch_rope_store_attention_regions": (None, [_vp] * 9 + [_i, _i, _i, _i, C.c_float, C.c_float, _i, _i, _i, _vp]),
+    "launch_rope_store_attention_partials_regions": (None, [_vp] * 9 + [_i, _i, _i, _i, C.c_float, C.c_float, _i, _vp, _i,
+                                                            C.c_size_t, _i, _i, _i, _vp]),
     "launch_attention_all_heads": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _vp]),
     "launch_flash_attention": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _vp]),
     "launch_attention_all_heads_batch": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, C.c_float, _i, _i, _vp]),

@@ -41,6 +41,11 @@ void launch_rope_store_attention_partials(float*, float*, const float*, int8_t*,
 void launch_rope_scaling(float, float, float, float);
 void launch_rope_store_attention(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int16_t*, const int*,
                                  int, int, int, int, float, float, int, int, hipStream_t);
+void launch_rope_store_attention_regions(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int16_t*,
+                                         const int*, int, int, int, int, float, float, int, int, int, hipStream_t);
+void launch_rope_store_attention_partials_regions(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int16_t*,
+                                                  const int*, int, int, int, int, float, float, int, const float*, int,
+                                                  size_t, int, int, int, hipStream_t);
 }
 
 namespace {
@@ -78,7 +83,24 @@ struct KvView {
     size_t layer_kv, layer_sc;
     int kv_stride;      // 0: every row of the batch works on one region
     int max_seq;
+    // 0: a region is [position][kv head][head_dim], the reference's layout (engine/model.h:58-63) -- the model's own
+    // cache.  > 0: [kv head][head_major positions][head_dim], scales [kv head][head_major] -- the per-sequence caches,
+    // which only this engine reads: a (sequence, KV head) workgroup of the attention kernel then streams contiguous memory.
+    int head_major;
 };
+
+// RoPE + KV store + attention on either layout
+void rope_store_attention(const KvView& kv, float* q, float* k, const float* v, int8_t* ck, int8_t* cv, float* sk, float* sv,
+                          int16_t* out, const int* positions, int position, int n_head, int n_head_kv, int head_dim,
+                          float theta, float scale, int B, hipStream_t st)
+{
+    if (kv.head_major)
+        launch_rope_store_attention_regions(q, k, v, ck, cv, sk, sv, out, positions, position, n_head, n_head_kv, head_dim,
+                                            theta, scale, B, kv.kv_stride, kv.head_major, st);
+    else
+        launch_rope_store_attention(q, k, v, ck, cv, sk, sv, out, positions, position, n_head, n_head_kv, head_dim, theta,
+                                    scale, B, kv.kv_stride, st);
+}
 
 enum LogitsMode { LOGITS_ALL, LOGITS_LAST_ROW, LOGITS_NONE };
 
@@ -309,9 +331,11 @@ void forward_b1_fused(InferenceState* state, const int* token_ids, const KvView&
 
         const size_t kv_off = (size_t)layer * kv.layer_kv;
         const size_t sc_off = (size_t)layer * kv.layer_sc;
-        launch_rope_store_attention(state->q_buf, state->k_buf, state->v_buf, kv.k + kv_off, kv.v + kv_off,
-                                    kv.sk + sc_off, kv.sv + sc_off, bf16_a, nullptr, pos, c.n_head, c.n_head_kv,
-                                    head_dim, c.rope_theta, scale, 1, 0, st);
+        KvView one = kv;
+        one.kv_stride = 0;
+        rope_store_attention(one, state->q_buf, state->k_buf, state->v_buf, kv.k + kv_off, kv.v + kv_off, kv.sk + sc_off,
+                             kv.sv + sc_off, bf16_a, nullptr, pos, c.n_head, c.n_head_kv, head_dim, c.rope_theta, scale, 1,
+                             st);
 
         S.o[0] = seg_of(L.wo, h_alt, n);
         must(t12_gemv_add(S.o, bf16_a, n, h, st), "wo decode-GEMV");                  // h_alt = h + wo . attn
@@ -351,10 +375,10 @@ KvView kv_view(const InferenceState* state)
     if (impl->per_seq) {
         const size_t S = (size_t)impl->seq_len, B = (size_t)state->batch_size;
         kv = KvView{impl->pk, impl->pv, impl->psk, impl->psv, B * S * kv_dim, B * S * c.n_head_kv, (int)(S * kv_dim),
-                    impl->seq_len};
+                    impl->seq_len, impl->seq_len};
     } else {
         kv = KvView{m->kv_cache_k, m->kv_cache_v, m->kv_scale_k, m->kv_scale_v, (size_t)m->max_seq_len * kv_dim,
-                    (size_t)m->max_seq_len * c.n_head_kv, 0, m->max_seq_len};
+                    (size_t)m->max_seq_len * c.n_head_kv, 0, m->max_seq_len, 0};
     }
     return kv;
 }
@@ -403,15 +427,21 @@ void forward_rows(InferenceState* state, int R, const KvView& kv, int pos0, Logi
         const size_t kv_off = (size_t)layer * kv.layer_kv;
         const size_t sc_off = (size_t)layer * kv.layer_sc;
         // RoPE (Q, K) + INT8 KV store + GQA attention
-        if (qkv_part.nsplit > 1)
+        if (qkv_part.nsplit > 1 && kv.head_major)
+            launch_rope_store_attention_partials_regions(state->q_buf, state->k_buf, state->v_buf, kv.k + kv_off,
+                                                         kv.v + kv_off, kv.sk + sc_off, kv.sv + sc_off, bf16_a,
+                                                         state->d_positions, pos0, c.n_head, c.n_head_kv, head_dim,
+                                                         c.rope_theta, scale, B, qkv_part.ws, qkv_part.nsplit,
+                                                         qkv_part.split_stride, qkv_part.ld, kv.kv_stride, kv.head_major, st);
+        else if (qkv_part.nsplit > 1)
             launch_rope_store_attention_partials(state->q_buf, state->k_buf, state->v_buf, kv.k + kv_off, kv.v + kv_off,
                                                  kv.sk + sc_off, kv.sv + sc_off, bf16_a, state->d_positions, pos0,
                                                  c.n_head, c.n_head_kv, head_dim, c.rope_theta, scale, B, qkv_part.ws,
                                                  qkv_part.nsplit, qkv_part.split_stride, qkv_part.ld, kv.kv_stride, st);
         else
-            launch_rope_store_attention(state->q_buf, state->k_buf, state->v_buf, kv.k + kv_off, kv.v + kv_off,
-                                        kv.sk + sc_off, kv.sv + sc_off, bf16_a, B == 1 ? nullptr : state->d_positions,
-                                        pos0, c.n_head, c.n_head_kv, head_dim, c.rope_theta, scale, B, kv.kv_stride, st);
+            rope_store_attention(kv, state->q_buf, state->k_buf, state->v_buf, kv.k + kv_off, kv.v + kv_off, kv.sk + sc_off,
+                                 kv.sv + sc_off, bf16_a, B == 1 ? nullptr : state->d_positions, pos0, c.n_head, c.n_head_kv,
+                                 head_dim, c.rope_theta, scale, B, st);
 
         S.o[0] = seg_of(L.wo, res, n);
         if (B > 1) {
@@ -720,6 +750,18 @@ void shift_context(InferenceState* state, int seq, int current_pos, int discard)
         for (int done = 0; done < keep; done += discard) {
             const size_t rows = (size_t)std::min(discard, keep - done);
             const size_t to = (size_t)done, from = (size_t)done + discard;
+            if (kv.head_major) {                                  // every KV head's rows are a block of their own
+                const size_t S = (size_t)kv.head_major;
+                for (int h = 0; h < nkv; h++) {
+                    check_gpu(hipMemcpyAsync(k + (h * S + to) * hd, k + (h * S + from) * hd, rows * hd, hipMemcpyDeviceToDevice, st), "shift K");
+                    check_gpu(hipMemcpyAsync(v + (h * S + to) * hd, v + (h * S + from) * hd, rows * hd, hipMemcpyDeviceToDevice, st), "shift V");
+                    check_gpu(hipMemcpyAsync(sk + h * S + to, sk + h * S + from, rows * sizeof(float), hipMemcpyDeviceToDevice, st),
+                              "shift K scales");
+                    check_gpu(hipMemcpyAsync(sv + h * S + to, sv + h * S + from, rows * sizeof(float), hipMemcpyDeviceToDevice, st),
+                              "shift V scales");
+                }
+                continue;
+            }
             check_gpu(hipMemcpyAsync(k + to * kv_dim, k + from * kv_dim, rows * kv_dim, hipMemcpyDeviceToDevice, st), "shift K");
             check_gpu(hipMemcpyAsync(v + to * kv_dim, v + from * kv_dim, rows * kv_dim, hipMemcpyDeviceToDevice, st), "shift V");
             check_gpu(hipMemcpyAsync(sk + to * nkv, sk + from * nkv, rows * nkv * sizeof(float), hipMemcpyDeviceToDevice, st),

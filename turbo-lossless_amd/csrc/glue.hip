@@ -246,7 +246,7 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(float* __restrict__ q, floa
                                                      const int* __restrict__ positions, int position,
                                                      int head_dim, int n_head, int n_head_kv, int q_stride,
                                                      int k_stride, QkvPartials part = QkvPartials{nullptr, 0, 0, 0},
-                                                     size_t kv_stride = 0)
+                                                     size_t kv_stride = 0, int hm = 0)
 {
     const int b = blockIdx.y;
     const int pos = positions ? positions[b] : position;
@@ -311,12 +311,15 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(float* __restrict__ q, floa
         const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
         const size_t kv_dim = (size_t)n_head_kv * head_dim;
         // per-sequence caches: sequence b's region starts kv_stride elements (kv_stride / head_dim scales) further on
-        int8_t* row = dst + (size_t)b * kv_stride + (size_t)pos * kv_dim + (size_t)kvh * head_dim;
+        // hm != 0: head-major regions, [kv head][hm positions][head_dim] (scales [kv head][hm]); else [position][kv head][head_dim]
+        int8_t* row = dst + (size_t)b * kv_stride +
+                      (hm ? ((size_t)kvh * hm + pos) * head_dim : (size_t)pos * kv_dim + (size_t)kvh * head_dim);
         if (own) {
             row[lane] = (int8_t)(int)fminf(fmaxf(rintf(r0 * inv), -127.0f), 127.0f);
             row[lane + half] = (int8_t)(int)fminf(fmaxf(rintf(r1 * inv), -127.0f), 127.0f);
         }
-        if (lane == 0) sdst[(size_t)b * (kv_stride / head_dim) + (size_t)pos * n_head_kv + kvh] = amax / 127.0f;
+        if (lane == 0)
+            sdst[(size_t)b * (kv_stride / head_dim) + (hm ? (size_t)kvh * hm + pos : (size_t)pos * n_head_kv + kvh)] = amax / 127.0f;
     }
 }
 
@@ -336,7 +339,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
                                                           const float* __restrict__ sv, uint16_t* __restrict__ out,
                                                           const int* __restrict__ positions, int seq_len_arg,
                                                           int n_head, int n_head_kv, int head_dim, float scale,
-                                                          size_t kv_stride)
+                                                          size_t kv_stride, int hm)
 {
     extern __shared__ float smem[];
     const int ratio = n_head / n_head_kv;
@@ -347,12 +350,14 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
     const int kvh = blockIdx.x, b = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int seq_len = positions ? positions[b] + 1 : seq_len_arg;
-    const size_t kv_dim = (size_t)n_head_kv * head_dim;
-    const int8_t* kbase = ck + (size_t)b * kv_stride + (size_t)kvh * head_dim;
-    const int8_t* vbase = cv + (size_t)b * kv_stride + (size_t)kvh * head_dim;
+    const size_t kv_dim = hm ? (size_t)head_dim : (size_t)n_head_kv * head_dim;   // distance between the rows of consecutive positions
+    const size_t hoff = hm ? (size_t)kvh * hm * head_dim : (size_t)kvh * head_dim;
+    const int ssr = hm ? 1 : n_head_kv;                  // distance between the scales of consecutive positions
+    const int8_t* kbase = ck + (size_t)b * kv_stride + hoff;
+    const int8_t* vbase = cv + (size_t)b * kv_stride + hoff;
     const size_t sstride = kv_stride / head_dim;        // scale arrays: kv_stride / head_dim per sequence
-    const float* skb = sk + (size_t)b * sstride + kvh;
-    const float* svb = sv + (size_t)b * sstride + kvh;
+    const float* skb = sk + (size_t)b * sstride + (hm ? (size_t)kvh * hm : (size_t)kvh);
+    const float* svb = sv + (size_t)b * sstride + (hm ? (size_t)kvh * hm : (size_t)kvh);
     const float* qb = q + (size_t)b * n_head * head_dim + (size_t)kvh * ratio * head_dim;
 
     for (int i = tid; i < ratio * head_dim; i += 256) qs[i] = qb[i];
@@ -372,7 +377,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
         if (tid < tl) {
             const int t = t0 + tid;
             const int8_t* kr = kbase + (size_t)t * kv_dim;
-            const float kscale = skb[(size_t)t * n_head_kv] * scale;
+            const float kscale = skb[(size_t)t * ssr] * scale;
             float dot[ATT_MAX_RATIO];
 #pragma unroll
             for (int h = 0; h < ATT_MAX_RATIO; h++) dot[h] = 0.0f;
@@ -416,7 +421,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
                 if (lane < nd2) {
                     for (int t = 0; t < tl; t++) {
                         const float pv = ps[h * ATT_TILE + t];
-                        const float w = pv * svb[(size_t)(t0 + t) * n_head_kv];
+                        const float w = pv * svb[(size_t)(t0 + t) * ssr];
                         const uint16_t two = *(const uint16_t*)(vbase + (size_t)(t0 + t) * kv_dim + 2 * lane);
                         a0 += w * (float)(int8_t)(two & 0xFF);
                         a1 += w * (float)(int8_t)(two >> 8);
@@ -490,7 +495,7 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
                                                         const float* __restrict__ sv, uint16_t* __restrict__ out,
                                                         const int* __restrict__ positions, int seq_len_arg,
                                                         int n_head_kv, float scale, size_t kv_stride, AttnFuse fz,
-                                                        AttnSplit sp)
+                                                        AttnSplit sp, int hm)
 {
     constexpr int CH = HD / 16;                 // lanes per position in phase 3
     constexpr int PG = 64 / CH;                 // positions per load instruction
@@ -502,11 +507,14 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
     const int seq_len = positions ? positions[b] + 1 : seq_len_arg;
     const int n_head = n_head_kv * RATIO;
     const size_t kv_dim = (size_t)n_head_kv * HD;
-    const int8_t* kbase = ck + (size_t)b * kv_stride + (size_t)kvh * HD;
-    const int8_t* vbase = cv + (size_t)b * kv_stride + (size_t)kvh * HD;
+    const size_t rstride = hm ? (size_t)HD : kv_dim;     // distance between the cache rows of consecutive positions
+    const size_t hoff = hm ? (size_t)kvh * hm * HD : (size_t)kvh * HD;
+    const int ssr = hm ? 1 : n_head_kv;                  // distance between the scales of consecutive positions
+    const int8_t* kbase = ck + (size_t)b * kv_stride + hoff;
+    const int8_t* vbase = cv + (size_t)b * kv_stride + hoff;
     const size_t sstride = kv_stride / HD;
-    const float* skb = sk + (size_t)b * sstride + kvh;
-    const float* svb = sv + (size_t)b * sstride + kvh;
+    const float* skb = sk + (size_t)b * sstride + (hm ? (size_t)kvh * hm : (size_t)kvh);
+    const float* svb = sv + (size_t)b * sstride + (hm ? (size_t)kvh * hm : (size_t)kvh);
     const float* qb = q + (size_t)b * n_head * HD + (size_t)kvh * RATIO * HD;
     // this workgroup's share of the context
     const int nchunk = SPLIT ? gridDim.z : 1;
@@ -530,10 +538,10 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
     uint4 kk_pre_n[CH];
     float kscale_pre_n = 0.0f;
     if (kpre_n) {
-        const uint4* kr = (const uint4*)(kbase + (size_t)(c0 + tid) * kv_dim);
+        const uint4* kr = (const uint4*)(kbase + (size_t)(c0 + tid) * rstride);
 #pragma unroll
         for (int u = 0; u < CH; u++) kk_pre_n[u] = kr[u];
-        kscale_pre_n = skb[(size_t)(c0 + tid) * n_head_kv] * scale;
+        kscale_pre_n = skb[(size_t)(c0 + tid) * ssr] * scale;
     }
     // Phase 1 layout: wave w scores positions 64 w .. 64 w + 63 of a tile in two blocks of 32; lane (ln, lh) of
     // block nb holds half lh of the K row of position 64 w + 32 nb + ln: HD / 2 contiguous bytes = KS pieces
@@ -552,10 +560,10 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
             const int tp = wave * 64 + nb * 32 + ln;             // position inside the first tile
             kpre[nb] = tp < tl0 && c0 + tp != newpos;
             if (kpre[nb]) {
-                const uint4* kr = (const uint4*)(kbase + (size_t)(c0 + tp) * kv_dim + lh * (HD / 2));
+                const uint4* kr = (const uint4*)(kbase + (size_t)(c0 + tp) * rstride + lh * (HD / 2));
 #pragma unroll
                 for (int u = 0; u < KS; u++) kk_pre[nb][u] = kr[u];
-                kscale_pre[nb] = skb[(size_t)(c0 + tp) * n_head_kv];     // as stored; multiplied where it is used
+                kscale_pre[nb] = skb[(size_t)(c0 + tp) * ssr];     // as stored; multiplied where it is used
             }
         }
     }
@@ -566,9 +574,9 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
         for (int x = 0; x < VPRE; x++) {
             const int idx = tid + 256 * x, t = idx / CH, u = idx % CH;
             v_pre[x] = make_uint4(0, 0, 0, 0);
-            if (t < tl0 && c0 + t != newpos) v_pre[x] = *(const uint4*)(vbase + (size_t)(c0 + t) * kv_dim + u * 16);
+            if (t < tl0 && c0 + t != newpos) v_pre[x] = *(const uint4*)(vbase + (size_t)(c0 + t) * rstride + u * 16);
         }
-        if (tid < tl0 && c0 + tid != newpos) vs_pre = svb[(size_t)(c0 + tid) * n_head_kv];
+        if (tid < tl0 && c0 + tid != newpos) vs_pre = svb[(size_t)(c0 + tid) * ssr];
     }
 
     if (!FUSE) {
@@ -599,7 +607,7 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
             }
             const float amax = wave_max(fmaxf(fabsf(r0), fabsf(r1)));
             const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
-            int8_t* row = (wave == 0 ? fz.ck_w : fz.cv_w) + (size_t)b * kv_stride + (size_t)pos * kv_dim + (size_t)kvh * HD;
+            int8_t* row = (wave == 0 ? fz.ck_w : fz.cv_w) + (size_t)b * kv_stride + hoff + (size_t)pos * rstride;
             const int8_t q0 = (int8_t)(int)fminf(fmaxf(rintf(r0 * inv), -127.0f), 127.0f);
             const int8_t q1 = (int8_t)(int)fminf(fmaxf(rintf(r1 * inv), -127.0f), 127.0f);
             // the new row: to the cache, and (first tile) to LDS where this launch reads it
@@ -615,7 +623,7 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
                 }
             }
             if (lane == 0) {
-                (wave == 0 ? fz.sk_w : fz.sv_w)[(size_t)b * sstride + (size_t)pos * n_head_kv + kvh] = amax / 127.0f;
+                (wave == 0 ? fz.sk_w : fz.sv_w)[(size_t)b * sstride + (hm ? (size_t)kvh * hm + pos : (size_t)pos * n_head_kv + kvh)] = amax / 127.0f;
                 if (wave == 0) knew_scale = amax / 127.0f;
                 else if (VLDS && rel < ATT_TILE) vts[rel] = amax / 127.0f;
             }
@@ -715,10 +723,10 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
                     for (int u = 0; u < KS; u++) kk[nb][u] = ((const uint4*)(knew8 + lh * (HD / 2)))[u];
                     kscale[nb] = knew_scale;
                 } else {
-                    const uint4* kr = (const uint4*)(kbase + (size_t)t * kv_dim + lh * (HD / 2));
+                    const uint4* kr = (const uint4*)(kbase + (size_t)t * rstride + lh * (HD / 2));
 #pragma unroll
                     for (int u = 0; u < KS; u++) kk[nb][u] = kr[u];
-                    kscale[nb] = skb[(size_t)t * n_head_kv];
+                    kscale[nb] = skb[(size_t)t * ssr];
                 }
             }
         }
@@ -727,7 +735,7 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
 #pragma unroll
         for (int x = 0; x < VP; x++) {
             const int idx = tid + 256 * x, t = min(half * 128 + idx / CH, tlx - 1), u = idx % CH;
-            vreg[x] = *(const t12_u32x4*)(vbase + (size_t)(t0x + t) * kv_dim + u * 16);
+            vreg[x] = *(const t12_u32x4*)(vbase + (size_t)(t0x + t) * rstride + u * 16);
         }
     };
     auto issue_vsc = [&](int t0x, int tlx, float (&dst)[OWN][ATT_TILE / 64]) __attribute__((always_inline)) {
@@ -736,7 +744,7 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
 #pragma unroll
             for (int i = 0; i < ATT_TILE / 64; i++) {
                 const int t = lane + 64 * i;
-                dst[j][i] = (wave + 4 * j < RATIO && t < tlx) ? svb[(size_t)(t0x + t) * n_head_kv] : 0.0f;
+                dst[j][i] = (wave + 4 * j < RATIO && t < tlx) ? svb[(size_t)(t0x + t) * ssr] : 0.0f;
             }
     };
     if constexpr (WIDE) {
@@ -799,10 +807,10 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
                 for (int u = 0; u < CH; u++) kk[u] = ((const uint4*)knew8)[u];
                 kscale = knew_scale * scale;
             } else {
-                const uint4* kr = (const uint4*)(kbase + (size_t)t * kv_dim);
+                const uint4* kr = (const uint4*)(kbase + (size_t)t * rstride);
 #pragma unroll
                 for (int u = 0; u < CH; u++) kk[u] = kr[u];
-                kscale = skb[(size_t)t * n_head_kv] * scale;
+                kscale = skb[(size_t)t * ssr] * scale;
             }
             float dot[RATIO];
 #pragma unroll
@@ -835,22 +843,22 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
 #pragma unroll
                 for (int nb = 0; nb < 2; nb++) {
                     const int t = t0n + wave * 64 + nb * 32 + ln;
-                    const uint4* kr = (const uint4*)(kbase + (size_t)t * kv_dim + lh * (HD / 2));
+                    const uint4* kr = (const uint4*)(kbase + (size_t)t * rstride + lh * (HD / 2));
 #pragma unroll
                     for (int u = 0; u < KS; u++) kk[nb][u] = kr[u];
-                    kscale[nb] = skb[(size_t)t * n_head_kv];
+                    kscale[nb] = skb[(size_t)t * ssr];
                 }
 #pragma unroll
                 for (int j = 0; j < OWN; j++)
 #pragma unroll
                     for (int i = 0; i < ATT_TILE / 64; i++) {
-                        const float s = svb[(size_t)(t0n + lane + 64 * i) * n_head_kv];
+                        const float s = svb[(size_t)(t0n + lane + 64 * i) * ssr];
                         vsc_n[j][i] = (RATIO % 4 == 0 || wave + 4 * j < RATIO) ? s : 0.0f;
                     }
 #pragma unroll
                 for (int x = 0; x < VP; x++) {
                     const int idx = tid + 256 * x;
-                    vreg[x] = *(const t12_u32x4*)(vbase + (size_t)(t0 + 128 + idx / CH) * kv_dim + (idx % CH) * 16);
+                    vreg[x] = *(const t12_u32x4*)(vbase + (size_t)(t0 + 128 + idx / CH) * rstride + (idx % CH) * 16);
                 }
             } else {
                 if (has_next) {
@@ -937,7 +945,7 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
 #pragma unroll
                             for (int x = 0; x < VP; x++) {
                                 const int idx = tid + 256 * x;
-                                vreg[x] = *(const t12_u32x4*)(vbase + (size_t)(t0n + idx / CH) * kv_dim + (idx % CH) * 16);
+                                vreg[x] = *(const t12_u32x4*)(vbase + (size_t)(t0n + idx / CH) * rstride + (idx % CH) * 16);
                             }
                         } else if (has_next) issue_v(t0n, tln, 0);    // the next tile's first 128 V rows
                         __syncthreads();
@@ -1011,8 +1019,8 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
                                 vv[x] = ((const uint4*)vt)[tc * CH + c];
                                 w[x] = ok ? ph[tc] * vts[tc] : 0.0f;
                             } else {
-                                vv[x] = *(const uint4*)(vbase + (size_t)(t0 + tc) * kv_dim + c * 16);
-                                w[x] = ok ? ph[tc] * svb[(size_t)(t0 + tc) * n_head_kv] : 0.0f;
+                                vv[x] = *(const uint4*)(vbase + (size_t)(t0 + tc) * rstride + c * 16);
+                                w[x] = ok ? ph[tc] * svb[(size_t)(t0 + tc) * ssr] : 0.0f;
                             }
                         }
     #pragma unroll
@@ -1271,7 +1279,7 @@ template <int MODE>
 void launch_rope_kv(float* q, float* k, const float* v, int8_t* ck, int8_t* cv, float* sk, float* sv,
                     const int* positions, int position, int head_dim, int n_head, int n_head_kv, int q_stride,
                     int k_stride, float theta, int batch, hipStream_t st, QkvPartials part = QkvPartials{nullptr, 0, 0, 0},
-                    size_t kv_stride = 0)
+                    size_t kv_stride = 0, int hm = 0)
 {
     const float* f = nullptr;
     if (MODE & 1) {
@@ -1284,7 +1292,7 @@ void launch_rope_kv(float* q, float* k, const float* v, int8_t* ck, int8_t* cv, 
         return;
     }
     hipLaunchKernelGGL(rope_kv_kernel<MODE>, dim3(n_head + 2 * n_head_kv, batch), dim3(64), 0, st, q, k, v, ck, cv, sk,
-                       sv, f, positions, position, head_dim, n_head, n_head_kv, q_stride, k_stride, part, kv_stride);
+                       sv, f, positions, position, head_dim, n_head, n_head_kv, q_stride, k_stride, part, kv_stride, hm);
     report("rope/kv-store");
 }
 
@@ -1325,7 +1333,7 @@ bool attn_has_fast(int n_head, int n_head_kv, int head_dim)
 // fuse != nullptr: RoPE + INT8 KV store happen inside the attention kernel (fast shapes only).
 void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float* sk, const float* sv, int16_t* out,
                  const int* positions, int seq_len, int n_head, int n_head_kv, int head_dim, float scale, int batch,
-                 size_t kv_stride, hipStream_t st, const AttnFuse* fuse = nullptr)
+                 size_t kv_stride, hipStream_t st, const AttnFuse* fuse = nullptr, int hm = 0)
 {
     const int ratio = n_head / n_head_kv;
     if (ratio < 1 || ratio > ATT_MAX_RATIO || n_head % n_head_kv || head_dim % 16 || head_dim > 128) {
@@ -1360,7 +1368,7 @@ void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float
 #define T12_ATT_GO(HD_, R_, F_, S_, W_)                                                                         \
     hipLaunchKernelGGL((attn_fast_kernel<HD_, R_, F_, S_, W_>), dim3(n_head_kv, batch, S_ ? nchunk : 1), dim3(256), 0, \
                        st, q, ck, cv, sk, sv, (uint16_t*)out, positions, seq_len, n_head_kv, scale, kv_stride,   \
-                       fuse ? *fuse : AttnFuse(), sp)
+                       fuse ? *fuse : AttnFuse(), sp, hm)
 #define T12_ATT_FAST(HD_, R_)                                                                                   \
     if (head_dim == HD_ && ratio == R_) {                                                                       \
         const int sel = (fuse ? 4 : 0) | (nchunk > 1 ? 2 : 0) | (wide ? 1 : 0);                                 \
@@ -1389,7 +1397,7 @@ void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float
 #undef T12_ATT_GO
     const size_t smem = ((size_t)ratio * head_dim + (size_t)ratio * ATT_TILE + 17 + 2 * ratio) * sizeof(float);
     hipLaunchKernelGGL(attn_decode_kernel, dim3(n_head_kv, batch), dim3(256), smem, st, q, ck, cv, sk, sv,
-                       (uint16_t*)out, positions, seq_len, n_head, n_head_kv, head_dim, scale, kv_stride);
+                       (uint16_t*)out, positions, seq_len, n_head, n_head_kv, head_dim, scale, kv_stride, hm);
     report("attention");
 }
 
@@ -1587,10 +1595,10 @@ void launch_rope_store_kv_batch(float* q, float* k, const float* v, int8_t* kv_k
 // launch, for B >= 1.  positions: device array [batch] (NULL: every sequence is at `position`).
 // Shapes without a specialised kernel, and large batches, run the separate launches.  q is scratch: left as
 // it was by the fused kernel, rotated in place by the separate RoPE launch.
-void launch_rope_store_attention(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v, float* scale_k,
+static void rope_store_attention(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v, float* scale_k,
                                  float* scale_v, int16_t* output, const int* positions, int position, int n_head,
                                  int n_head_kv, int head_dim, float theta, float scale, int batch_size, int kv_stride,
-                                 hipStream_t stream)
+                                 int hm, hipStream_t stream)
 {
     // Fusing pays when every workgroup stores its own cache slot (one sequence, or per-sequence caches) and
     // the launch is small enough to be a chain of latencies: the fused kernel holds prefetched rows in more
@@ -1608,14 +1616,42 @@ void launch_rope_store_attention(float* q, float* k, const float* v, int8_t* kv_
         fz.freqs = rope_table(head_dim, theta);
         if (!fz.freqs) { t12_set_error("rope: cannot build the frequency table"); return; }
         launch_attn(q, kv_k, kv_v, scale_k, scale_v, output, positions, position + 1, n_head, n_head_kv, head_dim,
-                    scale, batch_size, (size_t)kv_stride, stream, &fz);
+                    scale, batch_size, (size_t)kv_stride, stream, &fz, hm);
         return;
     }
     launch_rope_kv<3>(q, k, v, kv_k, kv_v, scale_k, scale_v, positions, position, head_dim, n_head, n_head_kv,
                       n_head * head_dim, n_head_kv * head_dim, theta, batch_size, stream, QkvPartials{nullptr, 0, 0, 0},
-                      (size_t)kv_stride);
+                      (size_t)kv_stride, hm);
     launch_attn(q, kv_k, kv_v, scale_k, scale_v, output, positions, position + 1, n_head, n_head_kv, head_dim, scale,
-                batch_size, (size_t)kv_stride, stream);
+                batch_size, (size_t)kv_stride, stream, nullptr, hm);
+}
+
+void launch_rope_store_attention(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v, float* scale_k,
+                                 float* scale_v, int16_t* output, const int* positions, int position, int n_head,
+                                 int n_head_kv, int head_dim, float theta, float scale, int batch_size, int kv_stride,
+                                 hipStream_t stream)
+{
+    rope_store_attention(q, k, v, kv_k, kv_v, scale_k, scale_v, output, positions, position, n_head, n_head_kv, head_dim,
+                         theta, scale, batch_size, kv_stride, 0, stream);
+}
+
+// The same on head-major cache regions: region_positions > 0 rows per (region, KV head), a region laid out
+// [kv head][region_positions][head_dim] (scales [kv head][region_positions]) instead of the reference's
+// [position][kv head][head_dim].  Every workgroup then reads one contiguous stream instead of 128-byte pieces of rows
+// it shares with the other KV heads' workgroups (B = 256 at 2000 positions: 199 against 254 us).  kv_stride is the
+// distance between regions as before.
+void launch_rope_store_attention_regions(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v, float* scale_k,
+                                         float* scale_v, int16_t* output, const int* positions, int position, int n_head,
+                                         int n_head_kv, int head_dim, float theta, float scale, int batch_size,
+                                         int kv_stride, int region_positions, hipStream_t stream)
+{
+    if (region_positions < 1 || position >= region_positions) {
+        t12_set_error("rope_store_attention_regions: position %d outside a region of %d positions", position, region_positions);
+        fprintf(stderr, "turbo12: %s\n", t12_last_error());
+        return;
+    }
+    rope_store_attention(q, k, v, kv_k, kv_v, scale_k, scale_v, output, positions, position, n_head, n_head_kv, head_dim,
+                         theta, scale, batch_size, kv_stride, region_positions, stream);
 }
 
 // launch_rope_store_attention for a batch whose q | k | v projection was split along K (t12_gemm_deferred,
@@ -1624,11 +1660,11 @@ void launch_rope_store_attention(float* q, float* k, const float* v, int8_t* kv_
 // region (lock-step copies, or the rows of one sequence's prompt at consecutive positions -- every row's
 // K / V is stored before any row attends, so row t sees rows <= t: a causal prefill); otherwise the element
 // distance between the regions of consecutive sequences.
-void launch_rope_store_attention_partials(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v,
+static void rope_store_attention_partials(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v,
                                           float* scale_k, float* scale_v, int16_t* output, const int* positions,
                                           int position, int n_head, int n_head_kv, int head_dim, float theta,
                                           float scale, int batch_size, const float* partials, int nsplit,
-                                          size_t split_stride, int ld, int kv_stride, hipStream_t stream)
+                                          size_t split_stride, int ld, int kv_stride, int hm, hipStream_t stream)
 {
     if (!partials || nsplit < 1 || nsplit > T12_MAX_KSPLIT || ld < (n_head + 2 * n_head_kv) * head_dim) {
         t12_set_error("rope_store_attention_partials: nsplit %d outside 1..%d, null partials or ld %d too small", nsplit,
@@ -1638,9 +1674,37 @@ void launch_rope_store_attention_partials(float* q, float* k, const float* v, in
     }
     launch_rope_kv<3>(q, k, v, kv_k, kv_v, scale_k, scale_v, positions, position, head_dim, n_head, n_head_kv,
                       n_head * head_dim, n_head_kv * head_dim, theta, batch_size, stream,
-                      QkvPartials{partials, nsplit, ld, split_stride}, (size_t)kv_stride);
+                      QkvPartials{partials, nsplit, ld, split_stride}, (size_t)kv_stride, hm);
     launch_attn(q, kv_k, kv_v, scale_k, scale_v, output, positions, position + 1, n_head, n_head_kv, head_dim, scale,
-                batch_size, (size_t)kv_stride, stream);
+                batch_size, (size_t)kv_stride, stream, nullptr, hm);
+}
+
+void launch_rope_store_attention_partials(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v,
+                                          float* scale_k, float* scale_v, int16_t* output, const int* positions,
+                                          int position, int n_head, int n_head_kv, int head_dim, float theta,
+                                          float scale, int batch_size, const float* partials, int nsplit,
+                                          size_t split_stride, int ld, int kv_stride, hipStream_t stream)
+{
+    rope_store_attention_partials(q, k, v, kv_k, kv_v, scale_k, scale_v, output, positions, position, n_head, n_head_kv,
+                                  head_dim, theta, scale, batch_size, partials, nsplit, split_stride, ld, kv_stride, 0, stream);
+}
+
+// launch_rope_store_attention_partials on head-major cache regions (see launch_rope_store_attention_regions).
+void launch_rope_store_attention_partials_regions(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v,
+                                                  float* scale_k, float* scale_v, int16_t* output, const int* positions,
+                                                  int position, int n_head, int n_head_kv, int head_dim, float theta,
+                                                  float scale, int batch_size, const float* partials, int nsplit,
+                                                  size_t split_stride, int ld, int kv_stride, int region_positions,
+                                                  hipStream_t stream)
+{
+    if (region_positions < 1) {
+        t12_set_error("rope_store_attention_partials_regions: a region of %d positions", region_positions);
+        fprintf(stderr, "turbo12: %s\n", t12_last_error());
+        return;
+    }
+    rope_store_attention_partials(q, k, v, kv_k, kv_v, scale_k, scale_v, output, positions, position, n_head, n_head_kv,
+                                  head_dim, theta, scale, batch_size, partials, nsplit, split_stride, ld, kv_stride,
+                                  region_positions, stream);
 }
 
 void launch_attention_all_heads(const float* q, const int8_t* k_cache, const int8_t* v_cache, const float* scale_k,
