@@ -353,7 +353,9 @@ def run_moe(args, t12, torch, dev):
 def run_attention(args, t12, torch, dev):
     """The attention step of one Llama-3.1-8B decoder layer (RoPE of q and k, INT8 store of the new K / V
     row, GQA attention over the INT8 cache: launch_rope_store_attention), every sequence on its own cache
-    region, at several (batch, context) points; `value` is the B = 256, 2000-position case in GB/s of cache read."""
+    region, at several (batch, context) points; `value` is the B = 256, 2000-position case on head-major regions (the
+    layout of the engine's per-sequence caches) in GB/s of cache read; the same case in the reference's layout is among
+    the cases."""
     import numpy as np
     nh, nkv, hd, theta = LLAMA8B["n_head"], LLAMA8B["n_head_kv"], LLAMA8B["n_embd"] // LLAMA8B["n_head"], 500000.0
     kv_dim = nkv * hd
@@ -392,9 +394,10 @@ def run_attention(args, t12, torch, dev):
         out_cases["b%d_ctx%d%s" % (B, ctx, "_headmajor" if head_major else "")] = {
             "us": ms * 1e3, "cache_MB": nbytes / 1e6, "GBps": nbytes / ms / 1e6}
         del kc, vc, ks, vs
-    head = out_cases["b256_ctx2000"]
+    head = out_cases["b256_ctx2000_headmajor"]           # the layout of the engine's per-sequence caches
     return {
-        "metric": "GB/s of INT8 KV cache read by the decode-attention step of one Llama-3.1-8B layer, B=256 at 2000 positions",
+        "metric": "GB/s of INT8 KV cache read by the decode-attention step of one Llama-3.1-8B layer, B=256 at 2000 positions "
+                  "(head-major per-sequence regions)",
         "value": head["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["us"] / 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
