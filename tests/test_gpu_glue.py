@@ -39,8 +39,10 @@ def test_embed_lookup(t12, oracle):
     assert np.array_equal(out.cpu().numpy(), oracle.embed_lookup(embd, toks, V))
 
 
-@pytest.mark.parametrize("n,B", [(4096, 1), (4096, 5), (256, 3), (14336, 2), (100, 1)])
+@pytest.mark.parametrize("n,B", [(4096, 1), (4096, 5), (256, 3), (14336, 2), (100, 1), (8192, 2), (4100, 2), (6, 3), (1022, 2)])
 def test_rms_norm_and_add(t12, oracle, n, B):
+    """Rows of a multiple of 4 values up to 8192 take the 128-bit form of the kernel (one or two pieces per thread),
+    the others the scalar form."""
     rng = np.random.default_rng(n + B)
     x = rng.standard_normal((B, n)).astype(np.float32) * 3
     r = rng.standard_normal((B, n)).astype(np.float32)
@@ -55,6 +57,28 @@ def test_rms_norm_and_add(t12, oracle, n, B):
     torch.cuda.synchronize()
     s, yb = oracle.add_rms_norm_bf16(x, r, w, 1e-5)
     assert np.array_equal(xd.cpu().numpy(), s)          # x += residual, exact in fp32
+    bf16_close(y.cpu().numpy().view(np.uint16), yb.reshape(B, n))
+
+
+def test_rms_norm_unaligned_rows_take_the_scalar_form(t12, oracle):
+    """Operands that are not 16-byte aligned (a view one float into a buffer) still give the same result."""
+    rng = np.random.default_rng(5)
+    n, B = 512, 3
+    x = rng.standard_normal((B, n)).astype(np.float32) * 3
+    r = rng.standard_normal((B, n)).astype(np.float32)
+    w = (1 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+
+    def off(a):                                         # a device copy that starts 4 bytes past a 16-byte boundary
+        buf = torch.zeros(a.size + 1, dtype=torch.float32, device=dev())
+        buf[1:] = torch.from_numpy(a.reshape(-1)).to(dev())
+        return buf[1:]
+    xd, rd, wd = off(x), off(r), off(w)
+    assert xd.data_ptr() % 16 == 4
+    y = torch.zeros((B, n), dtype=torch.int16, device=dev())
+    t12.lib.launch_add_rms_norm_bf16_batch(xd.data_ptr(), rd.data_ptr(), wd.data_ptr(), y.data_ptr(), n, 1e-5, B, st(t12))
+    torch.cuda.synchronize()
+    s_, yb = oracle.add_rms_norm_bf16(x, r, w, 1e-5)
+    assert np.array_equal(xd.cpu().numpy().reshape(B, n), s_)
     bf16_close(y.cpu().numpy().view(np.uint16), yb.reshape(B, n))
 
 
