@@ -30,8 +30,9 @@ def run_gemv(t12, packs, x, patched=True):
 
 
 @pytest.mark.parametrize("M,K", [(4096, 4096), (1024, 4096), (256, 14336), (300, 1280), (77, 5120),
-                                 (1, 1024), (9, 16), (64, 1040), (5, 2064)])
+                                 (1, 1024), (9, 16), (64, 1040), (5, 2064), (16, 20480), (8, 28672), (3, 16400)])
 def test_gemv_llm_law(t12, oracle, synth, M, K):
+    """(Rows wider than 16384 columns stage the rest of the activations in a loop behind the pieces requested up front.)"""
     w = synth.weights_llm(M, K, seed=1001 + M + K, p_outlier=3e-4 if M * K > 1e5 else 2e-2)
     x = synth.activations(1, K, seed=1002)[0]
     p = oracle.pack(w)
