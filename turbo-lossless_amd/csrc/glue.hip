@@ -468,6 +468,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
 // RATIO query heads while loading them, rotates this KV head's new K, quantises K and V to
 // INT8 and stores them at position pos -- and only then attends over positions 0..pos.
 // (All B workgroups of a shared cache, kv_stride = 0, store identical values into one slot.)
+// hm (all cache-touching kernels): 0 = a cache region is [position][kv head][dim] with scales [position][kv head], the
+// reference's layout; hm > 0 = head-major regions of hm positions, [kv head][hm][dim] with scales [kv head][hm], in which
+// the rows one workgroup reads are contiguous.
 struct AttnFuse {
     const float* k_new;      // [B, n_head_kv * HD] fp32, unrotated
     const float* v_new;
