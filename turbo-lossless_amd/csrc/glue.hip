@@ -582,31 +582,47 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
         if (tid < tl0 && c0 + tid != newpos) vs_pre = svb[(size_t)(c0 + tid) * ssr];
     }
 
+    constexpr int QSTR = HD + 16;               // row pitch of qlimb, for the same reason as WSTR
+    __shared__ __attribute__((aligned(16))) int8_t qlimb[WIDE ? 32 * QSTR : 16];
+    __shared__ float qscale[RATIO];
+    if constexpr (WIDE)
+        for (int i = tid; i < 32 * QSTR / 16; i += 256) ((uint4*)qlimb)[i] = make_uint4(0, 0, 0, 0);
     if (!FUSE) {
         for (int i = tid; i < RATIO * HD; i += 256) qs[i] = qb[i];
     } else {
         constexpr int HALF = HD / 2;
+        static_assert(256 % HALF == 0, "a thread keeps one rotation angle");
         const int pos = seq_len - 1;
-        for (int i = tid; i < RATIO * HALF; i += 256) {              // rotate Q on the way into LDS
-            const int h = i / HALF, d = i % HALF;
-            float sn, cs;
-            sincosf((float)pos * fz.freqs[d], &sn, &cs);
+        // everything this part needs is requested in one go -- the frequency of the thread's dim pair d = tid % HALF
+        // (the same d in every pass of the Q loop, and the new K row's d in wave 0), the thread's first Q pair, the new
+        // K / V row -- and the angle is worked out once: one round trip instead of one per step
+        const int d = tid % HALF;
+        const float freq = fz.freqs[d];
+        const bool qfirst = tid < RATIO * HALF;
+        float qx0 = 0.0f, qx1 = 0.0f;
+        if (qfirst) {
+            qx0 = qb[(tid / HALF) * HD + d];
+            qx1 = qb[(tid / HALF) * HD + d + HALF];
+        }
+        const bool own = lane < HALF;
+        float r0 = 0.0f, r1 = 0.0f;
+        if (wave < 2 && store_new && own) {
+            const float* src = (wave == 0 ? fz.k_new : fz.v_new) + (size_t)b * kv_dim + (size_t)kvh * HD;
+            r0 = src[lane];
+            r1 = src[lane + HALF];
+        }
+        float sn, cs;
+        sincosf((float)pos * freq, &sn, &cs);
+        if (qfirst) rope_rotate(qx0, qx1, sn, cs, qs[(tid / HALF) * HD + d], qs[(tid / HALF) * HD + d + HALF]);
+        for (int i = tid + 256; i < RATIO * HALF; i += 256) {        // (more than 256 pairs: GQA ratios above 4 at head_dim 128)
+            const int h = i / HALF;
             const float x0 = qb[h * HD + d], x1 = qb[h * HD + d + HALF];
             rope_rotate(x0, x1, sn, cs, qs[h * HD + d], qs[h * HD + d + HALF]);
         }
         if (wave < 2 && store_new) {                                 // wave 0: K (rotated), wave 1: V
-            const bool own = lane < HALF;
-            const float* src = (wave == 0 ? fz.k_new : fz.v_new) + (size_t)b * kv_dim + (size_t)kvh * HD;
-            float r0 = 0.0f, r1 = 0.0f;
-            if (own) {
-                r0 = src[lane];
-                r1 = src[lane + HALF];
-                if (wave == 0) {
-                    float sn, cs;
-                    sincosf((float)pos * fz.freqs[lane], &sn, &cs);
-                    const float x0 = r0, x1 = r1;
-                    rope_rotate(x0, x1, sn, cs, r0, r1);
-                }
+            if (own && wave == 0) {
+                const float x0 = r0, x1 = r1;
+                rope_rotate(x0, x1, sn, cs, r0, r1);
             }
             const float amax = wave_max(fmaxf(fabsf(r0), fabsf(r1)));
             const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
@@ -649,12 +665,8 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
     // 6e-8 max|q_h|: fp32 level, also for heads with outlier dims), laid out as the A operand of the score MFMAs: row
     // 8 * limb + h (the 32 rows of the MFMA are there anyway).
     // INT8 x INT8 products accumulate exactly in int32, so K needs no conversion at all.
-    constexpr int QSTR = HD + 16;               // row pitch of qlimb, for the same reason as WSTR
-    __shared__ __attribute__((aligned(16))) int8_t qlimb[WIDE ? 32 * QSTR : 16];
-    __shared__ float qscale[RATIO];
+    // (qlimb was cleared ahead of the Q loads, under their latency; the barrier above covers it)
     if constexpr (WIDE) {
-    for (int i = tid; i < 32 * QSTR / 16; i += 256) ((uint4*)qlimb)[i] = make_uint4(0, 0, 0, 0);
-    __syncthreads();
     for (int h = wave; h < RATIO; h += 4) {
         float amax = 0.0f;
         for (int d = lane; d < HD; d += 64) amax = fmaxf(amax, fabsf(qs[h * HD + d]));
