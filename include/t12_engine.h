@@ -15,6 +15,10 @@ extern "C" {
 #endif
 
 void* t12_engine_load(const char* model_dir, int device);            /* load_model; NULL on failure (model.cpp:165-328) */
+/* check_model_dir: the host-only consistency check load_model starts with (files present, sizes, tensor shapes
+ * against config.bin, escape-list invariants).  0 = consistent; -1 = not, first finding in msg (cap bytes).
+ * No counterpart in the reference, which loads what it finds (model.cpp:203-242). */
+int   t12_engine_check_dir(const char* model_dir, char* msg, size_t cap);
 /* create_synthetic_model: a random-init model of the given shape, generated and packed on the GPU
  * (weights N(0, 0.02) with outliers N(0, 8) at rate p_outlier; norm weights 1).  No reference counterpart:
  * the reference loads converted checkpoints only. */
@@ -26,6 +30,11 @@ int   t12_engine_max_seq(void* model);                               /* Model::m
 /* which: 0 wq 1 wk 2 wv 3 wo 4 w_gate 5 w_up 6 w_down; layer -1 = output_proj.  Fills *seg (out = NULL), *K and the
  * escape count; returns 0, or -1 for a tensor that does not exist. */
 int   t12_engine_weight(void* model, int layer, int which, T12Segment* seg, int* K, int* num_patches);
+/* The derived escape tables load_compressed builds for the same tensor (engine/model.cpp:86-160), as device
+ * pointers: escape_row_base [M], escape_vals [num_patches] (correct values ordered row, col % 256, col),
+ * patch_nonempty_rows [*n_nonempty]. */
+int   t12_engine_weight_tables(void* model, int layer, int which, const int32_t** row_base, const int16_t** vals,
+                               const int32_t** nonempty_rows, int* n_nonempty);
 
 void* t12_engine_create_state(void* model, int batch, int max_seq);  /* create_inference_state (inference.cpp:94-166) */
 /* create_inference_state_per_sequence: batch INDEPENDENT sequences, each with its own KV-cache region of max_seq

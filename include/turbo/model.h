@@ -67,10 +67,19 @@ struct Model {
 
 // Reads a converted model directory (config.bin, tok_embd.bin, *_norm.bin and the
 // seven files of every tensor).  Returns nullptr when config.bin or tok_embd.bin is
-// missing (engine/model.cpp:173-178,198); a tensor whose planes are missing or whose
-// file sizes contradict its .dims is reported on stderr and left empty.
+// missing (engine/model.cpp:173-178,198) -- and, unlike the reference, which warns and
+// carries on with null pointers (model.cpp:203-242), also when check_model_dir finds
+// anything else wrong: the first forward would turn it into a device memory fault.
 // Context length: TURBO_CTX, else min(8192, what fits in free HBM) (model.cpp:248-269).
 Model* load_model(const std::string& model_path, int device_id = 0);
+
+// Not in the reference: the host-only consistency check load_model starts with (no GPU call).
+// Every norm file present with n_embd floats; every tensor's .dims equal to the shape its role
+// implies from config.bin (wq n x n, wk/wv kv x n, wo n x n, w_gate/w_up ff x n, w_down n x ff,
+// output_proj vocab x n), base_exp in -1..254, plane and list file sizes equal to what .dims
+// says, row_off[0] == 0, non-decreasing, row_off[M] == num_patches, escape columns inside the
+// row and ascending within it.  false + the first finding in err.
+bool check_model_dir(const std::string& model_path, std::string& err);
 void free_model(Model* model);
 
 // ---- not in the reference -----------------------------------------------------

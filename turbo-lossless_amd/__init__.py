@@ -83,6 +83,8 @@ _SIGS = {
     "launch_argmax_batch": (None, [_vp, _vp, _i, _i, _vp]),
     # engine (C face of model.h / inference.h / sampler.h)
     "t12_engine_load": (_vp, [C.c_char_p, _i]),
+    "t12_engine_check_dir": (_i, [C.c_char_p, C.c_char_p, C.c_size_t]),
+    "t12_engine_weight_tables": (_i, [_vp, _i, _i, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_i)]),
     "t12_engine_create_synthetic": (_vp, [_i, _i, _i, _i, _i, _i, _i, C.c_float, C.c_float, C.c_uint64, _i, C.c_float]),
     "t12_engine_save": (_i, [_vp, C.c_char_p]),
     "t12_engine_free_model": (None, [_vp]),
@@ -405,6 +407,13 @@ class Engine:
         check(lib.t12_engine_weight(self.model, layer, which, C.byref(seg), C.byref(K), C.byref(P)), "engine_weight")
         return seg, K.value, P.value
 
+    def weight_tables(self, layer, which):
+        """Device pointers (row_base, vals, nonempty_rows) and the number of non-empty rows."""
+        rb, vals, ne, n = _vp(), _vp(), _vp(), C.c_int()
+        check(lib.t12_engine_weight_tables(self.model, layer, which, C.byref(rb), C.byref(vals), C.byref(ne), C.byref(n)),
+              "engine_weight_tables")
+        return rb.value, vals.value, ne.value, n.value
+
     def close(self):
         if self.state:
             lib.t12_engine_free_state(self.state)
@@ -424,6 +433,12 @@ def _hip_memcpy_d2d(dst, src, nbytes):
         _hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
         _hip.hipMemcpy.restype = C.c_int
     return _hip.hipMemcpy(dst, src, nbytes, 3)   # hipMemcpyDeviceToDevice
+
+
+def check_model_dir(path) -> str:
+    """'' when the directory is consistent, else the loader's first finding (host only, no GPU)."""
+    buf = C.create_string_buffer(512)
+    return "" if lib.t12_engine_check_dir(os.fsencode(path), buf, 512) == 0 else (buf.value.decode() or "inconsistent")
 
 
 class Tokenizer:

@@ -12,6 +12,18 @@ extern "C" {
 
 void* t12_engine_load(const char* path, int device) { return load_model(path ? path : "", device); }
 
+// check_model_dir(); 0 = consistent, -1 = not (the first finding in msg, cut to cap bytes incl. the terminator).
+int t12_engine_check_dir(const char* path, char* msg, size_t cap)
+{
+    std::string err;
+    const bool ok = check_model_dir(path ? path : "", err);
+    if (msg && cap) {
+        strncpy(msg, err.c_str(), cap - 1);
+        msg[cap - 1] = 0;
+    }
+    return ok ? 0 : -1;
+}
+
 void* t12_engine_create_synthetic(int n_vocab, int n_embd, int n_head, int n_head_kv, int n_layer, int n_ff, int n_ctx,
                                   float rope_theta, float rms_eps, uint64_t seed, int max_seq, float p_outlier)
 {
@@ -147,6 +159,28 @@ int t12_engine_weight(void* model, int layer, int which, T12Segment* seg, int* K
     seg->out_stride = seg->reserved = 0;
     *K = w->K;
     *num_patches = w->num_patches;
+    return 0;
+}
+
+// The loader's derived escape tables of the same tensor (engine/model.cpp:86-160): device pointers to
+// escape_row_base [M], escape_vals [num_patches], patch_nonempty_rows [*n_nonempty]; all NULL / 0 for a tensor
+// without escapes.
+int t12_engine_weight_tables(void* model, int layer, int which, const int32_t** row_base, const int16_t** vals,
+                             const int32_t** nonempty_rows, int* n_nonempty)
+{
+    Model* m = (Model*)model;
+    const CompressedWeight* w = nullptr;
+    if (layer < 0) w = &m->output_proj;
+    else if (layer < (int)m->layers.size()) {
+        TransformerLayer& L = m->layers[layer];
+        const CompressedWeight* all[7] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.w_gate, &L.w_up, &L.w_down};
+        if (which >= 0 && which < 7) w = all[which];
+    }
+    if (!w || !w->split_sm) return -1;
+    *row_base = w->escape_row_base;
+    *vals = w->escape_vals;
+    *nonempty_rows = w->patch_nonempty_rows;
+    *n_nonempty = w->num_nonempty_rows;
     return 0;
 }
 

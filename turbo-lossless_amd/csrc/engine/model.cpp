@@ -9,6 +9,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <fstream>
+#include <sys/stat.h>
 
 #include "t12_abi.h"
 
@@ -91,6 +92,99 @@ void build_escape_tables(CompressedWeight& w, const int32_t* row_off, const int3
     w.patch_nonempty_rows = upload<int32_t>(nonempty.data(), nonempty.size());
 }
 
+
+// ---------------------------------------------------------------- directory check (host only)
+long long file_size(const std::string& path)
+{
+    struct stat st;
+    if (stat(path.c_str(), &st) != 0 || !S_ISREG(st.st_mode)) return -1;
+    return (long long)st.st_size;
+}
+
+bool fail(std::string& err, const std::string& what)
+{
+    err = what;
+    return false;
+}
+
+// One tensor: .dims against the shape its role implies, the seven file sizes against .dims, and the CSR list's
+// own invariants (row_off[0] == 0, non-decreasing, row_off[M] == P; columns inside the row and ascending in it).
+bool check_tensor(const std::string& dir, const std::string& prefix, int want_M, int want_K, std::string& err)
+{
+    const std::string base = dir + "/" + prefix;
+    std::ifstream df(base + ".dims");
+    if (!df) return fail(err, prefix + ".dims is missing");
+    long long M = 0, K = 0, P = 0, be = 0;
+    if (!(df >> M >> K >> P) || M <= 0 || K <= 0 || P < 0 || M > 0x7FFFFFFF || K > 0x7FFFFFFF || P > 0x7FFFFFFF)
+        return fail(err, prefix + ".dims is malformed");
+    if (!(df >> be)) be = 0;                       // 4th field optional (engine/model.cpp:38-42)
+    if (M != want_M || K != want_K)
+        return fail(err, prefix + ": dims " + std::to_string(M) + " x " + std::to_string(K) + " but config.bin implies " +
+                             std::to_string(want_M) + " x " + std::to_string(want_K));
+    if (be < -1 || be > 254) return fail(err, prefix + ": base_exp " + std::to_string(be) + " outside -1..254");
+    const long long n = M * K;
+    if (file_size(base + ".sm.bin") != n || file_size(base + ".gr.bin") != (n + 1) / 2)
+        return fail(err, prefix + ": .sm.bin / .gr.bin missing or not the size of " + std::to_string(M) + " x " + std::to_string(K));
+    if (P == 0) return true;                       // the three list files may be empty or absent (model.cpp:47-68)
+    if (file_size(base + ".row_off.bin") != (M + 1) * 4 || file_size(base + ".patch_cols.bin") != P * 4 ||
+        file_size(base + ".patch_correct.bin") != P * 2 || file_size(base + ".patch_wrong.bin") != P * 2)
+        return fail(err, prefix + ": escape list files do not match num_patches " + std::to_string(P));
+    std::vector<uint8_t> ro, pc;
+    if (!read_file(base + ".row_off.bin", ro, true) || !read_file(base + ".patch_cols.bin", pc, true))
+        return fail(err, prefix + ": escape list files unreadable");
+    const int32_t* r = (const int32_t*)ro.data();
+    const int32_t* c = (const int32_t*)pc.data();
+    if (r[0] != 0) return fail(err, prefix + ": row_off[0] is not 0");
+    if (r[M] != P) return fail(err, prefix + ": row_off[M] is not num_patches");
+    for (long long i = 0; i < M; i++)
+        if (r[i + 1] < r[i]) return fail(err, prefix + ": row_off is not monotone");
+    for (long long i = 0; i < M; i++)
+        for (int32_t q = r[i]; q < r[i + 1]; q++) {
+            if (c[q] < 0 || c[q] >= K) return fail(err, prefix + ": escape column out of range");
+            if (q > r[i] && c[q] <= c[q - 1]) return fail(err, prefix + ": escape columns of a row do not ascend");
+        }
+    return true;
+}
+
+bool read_config(const std::string& model_path, ModelConfig& c, std::string& err)
+{
+    std::vector<uint8_t> buf;
+    if (!read_file(model_path + "/config.bin", buf, true) || buf.size() < 36)
+        return fail(err, "No config.bin found in " + model_path);
+    struct { int32_t v[7]; float theta, eps; } raw;
+    static_assert(sizeof raw == 36, "config.bin is 36 bytes");
+    memcpy(&raw, buf.data(), sizeof raw);
+    c.n_vocab = raw.v[0]; c.n_embd = raw.v[1]; c.n_head = raw.v[2]; c.n_head_kv = raw.v[3];
+    c.n_layer = raw.v[4]; c.n_ff = raw.v[5]; c.n_ctx = raw.v[6];
+    c.rope_theta = raw.theta; c.rms_norm_eps = raw.eps;
+    c.rope_scaling[0] = c.rope_scaling[1] = c.rope_scaling[2] = c.rope_scaling[3] = 0.0f;
+    std::vector<uint8_t> rs;
+    if (read_file(model_path + "/rope_scaling.bin", rs, true)) {
+        if (rs.size() != 16) return fail(err, "rope_scaling.bin in " + model_path + " is not 4 floats");
+        memcpy(c.rope_scaling, rs.data(), 16);
+        if (!(c.rope_scaling[0] > 0.0f) || !(c.rope_scaling[2] > c.rope_scaling[1]) || !(c.rope_scaling[3] > 0.0f))
+            return fail(err, "rope_scaling.bin in " + model_path + " holds impossible values");
+    }
+    if (c.n_vocab <= 0 || c.n_embd <= 0 || c.n_head <= 0 || c.n_head_kv <= 0 || c.n_layer < 0 || c.n_ff <= 0 ||
+        c.n_embd % c.n_head || c.n_head % c.n_head_kv)
+        return fail(err, "config.bin in " + model_path + " holds an impossible shape");
+    return true;
+}
+
+const char* const kTensorNames[7] = {"wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down"};
+
+// (rows, columns) of layer tensor `which` (order of kTensorNames) for a configuration
+void tensor_shape(const ModelConfig& c, int which, int& M, int& K)
+{
+    const int n = c.n_embd, kv = c.n_head_kv * (c.n_embd / c.n_head);
+    switch (which) {
+        case 1: case 2: M = kv; K = n; break;
+        case 4: case 5: M = c.n_ff; K = n; break;
+        case 6: M = n; K = c.n_ff; break;
+        default: M = n; K = n; break;
+    }
+}
+
 bool load_compressed(const std::string& dir, const std::string& prefix, CompressedWeight& w)
 {
     clear_weight(w);
@@ -125,7 +219,7 @@ bool load_compressed(const std::string& dir, const std::string& prefix, Compress
     if (P > 0) {
         const bool sizes_ok = ro.size() == (size_t)(M + 1) * 4 && pc.size() == (size_t)P * 4 &&
                               pv.size() == (size_t)P * 2 && pw.size() == (size_t)P * 2;
-        if (!sizes_ok || ((const int32_t*)ro.data())[M] != P) {
+        if (!sizes_ok || ((const int32_t*)ro.data())[M] != P || ((const int32_t*)ro.data())[0] != 0) {
             fprintf(stderr, "ERROR: %s: escape list files do not match num_patches %d\n", prefix.c_str(), P);
             return false;
         }
@@ -192,80 +286,82 @@ int default_context(const ModelConfig& c)
 
 }  // namespace
 
-Model* load_model(const std::string& model_path, int device_id)
+bool check_model_dir(const std::string& model_path, std::string& err)
 {
-    if (!gpu_ok(hipSetDevice(device_id), "hipSetDevice")) return nullptr;
-    std::vector<uint8_t> buf;
-    if (!read_file(model_path + "/config.bin", buf, true) || buf.size() < 36) {
-        fprintf(stderr, "No config.bin found in %s\n", model_path.c_str());
-        return nullptr;
-    }
-    Model* m = new Model();
-    struct { int32_t v[7]; float theta, eps; } raw;
-    static_assert(sizeof raw == 36, "config.bin is 36 bytes");
-    memcpy(&raw, buf.data(), sizeof raw);
-    ModelConfig& c = m->config;
-    c.n_vocab = raw.v[0]; c.n_embd = raw.v[1]; c.n_head = raw.v[2]; c.n_head_kv = raw.v[3];
-    c.n_layer = raw.v[4]; c.n_ff = raw.v[5]; c.n_ctx = raw.v[6];
-    c.rope_theta = raw.theta; c.rms_norm_eps = raw.eps;
-    c.rope_scaling[0] = c.rope_scaling[1] = c.rope_scaling[2] = c.rope_scaling[3] = 0.0f;
-    {
-        std::vector<uint8_t> rs;
-        if (read_file(model_path + "/rope_scaling.bin", rs, true)) {
-            if (rs.size() != 16) {
-                fprintf(stderr, "rope_scaling.bin in %s is not 4 floats\n", model_path.c_str());
-                delete m;
-                return nullptr;
-            }
-            memcpy(c.rope_scaling, rs.data(), 16);
-            if (!(c.rope_scaling[0] > 0.0f) || !(c.rope_scaling[2] > c.rope_scaling[1]) || !(c.rope_scaling[3] > 0.0f)) {
-                fprintf(stderr, "rope_scaling.bin in %s holds impossible values\n", model_path.c_str());
-                delete m;
-                return nullptr;
-            }
+    ModelConfig c;
+    if (!read_config(model_path, c, err)) return false;
+    if (file_size(model_path + "/tok_embd.bin") != (long long)c.n_vocab * c.n_embd * 2)
+        return fail(err, "Missing tok_embd.bin (or wrong size)");
+    auto norm_ok = [&](const std::string& name) {
+        if (file_size(model_path + "/" + name) == (long long)c.n_embd * 4) return true;
+        return fail(err, name + " missing or not n_embd floats");
+    };
+    if (!norm_ok("output_norm.bin")) return false;
+    if (!check_tensor(model_path, "output_proj", c.n_vocab, c.n_embd, err)) return false;
+    for (int i = 0; i < c.n_layer; i++) {
+        const std::string p = "layer." + std::to_string(i) + ".";
+        if (!norm_ok(p + "attn_norm.bin") || !norm_ok(p + "ffn_norm.bin")) return false;
+        for (int t = 0; t < 7; t++) {
+            int M, K;
+            tensor_shape(c, t, M, K);
+            if (!check_tensor(model_path, p + kTensorNames[t], M, K, err)) return false;
         }
     }
-    if (c.n_vocab <= 0 || c.n_embd <= 0 || c.n_head <= 0 || c.n_head_kv <= 0 || c.n_layer < 0 || c.n_ff <= 0 ||
-        c.n_embd % c.n_head || c.n_head % c.n_head_kv) {
-        fprintf(stderr, "config.bin in %s holds an impossible shape\n", model_path.c_str());
-        delete m;
+    return true;
+}
+
+Model* load_model(const std::string& model_path, int device_id)
+{
+    // Everything that can be wrong with the directory is found on the host first: a norm that is missing, a tensor
+    // whose shape is not its role's, a list that points outside its row would each become a device memory fault in
+    // the first forward.  (The reference warns and carries on, engine/model.cpp:203-242.)
+    std::string err;
+    if (!check_model_dir(model_path, err)) {
+        fprintf(stderr, "%s\n", err.c_str());
         return nullptr;
     }
+    if (!gpu_ok(hipSetDevice(device_id), "hipSetDevice")) return nullptr;
+    Model* m = new Model();
+    ModelConfig& c = m->config;
+    read_config(model_path, c, err);
     printf("  Config: vocab=%d embd=%d heads=%d/%d layers=%d ff=%d\n", c.n_vocab, c.n_embd, c.n_head, c.n_head_kv,
            c.n_layer, c.n_ff);
 
-    if (!read_file(model_path + "/tok_embd.bin", buf, true) || buf.size() != (size_t)c.n_vocab * c.n_embd * 2) {
-        fprintf(stderr, "Missing tok_embd.bin (or wrong size)\n");
-        delete m;
-        return nullptr;
-    }
-    m->token_embd = upload<int16_t>(buf.data(), buf.size() / 2);
+    std::vector<uint8_t> buf;
+    bool ok = read_file(model_path + "/tok_embd.bin", buf, true) && buf.size() == (size_t)c.n_vocab * c.n_embd * 2;
+    if (ok) m->token_embd = upload<int16_t>(buf.data(), buf.size() / 2);
+    buf.clear();
+    buf.shrink_to_fit();
 
     auto load_norm = [&](const std::string& name) -> float* {
         std::vector<uint8_t> nb;
         if (!read_file(model_path + "/" + name, nb, true) || nb.size() != (size_t)c.n_embd * 4) {
-            fprintf(stderr, "Warning: %s missing or wrong size\n", name.c_str());
+            fprintf(stderr, "%s missing or wrong size\n", name.c_str());
+            ok = false;
             return nullptr;
         }
         return upload<float>(nb.data(), c.n_embd);
     };
-    m->output_norm = load_norm("output_norm.bin");
-    if (!load_compressed(model_path, "output_proj", m->output_proj)) fprintf(stderr, "Warning: no output_proj\n");
+    if (ok) m->output_norm = load_norm("output_norm.bin");
+    ok = ok && load_compressed(model_path, "output_proj", m->output_proj);
 
     m->layers.resize(c.n_layer);
-    for (int i = 0; i < c.n_layer; i++) {
+    for (auto& L : m->layers) {
+        L.attn_norm = L.ffn_norm = nullptr;
+        for (CompressedWeight* w : {&L.wq, &L.wk, &L.wv, &L.wo, &L.w_gate, &L.w_up, &L.w_down}) clear_weight(*w);
+    }
+    for (int i = 0; ok && i < c.n_layer; i++) {
         TransformerLayer& L = m->layers[i];
         const std::string p = "layer." + std::to_string(i) + ".";
         L.attn_norm = load_norm(p + "attn_norm.bin");
         L.ffn_norm = load_norm(p + "ffn_norm.bin");
-        load_compressed(model_path, p + "wq", L.wq);
-        load_compressed(model_path, p + "wk", L.wk);
-        load_compressed(model_path, p + "wv", L.wv);
-        load_compressed(model_path, p + "wo", L.wo);
-        load_compressed(model_path, p + "w_gate", L.w_gate);
-        load_compressed(model_path, p + "w_up", L.w_up);
-        load_compressed(model_path, p + "w_down", L.w_down);
-        if ((i + 1) % 8 == 0 || i == c.n_layer - 1) printf("  Loaded layer %d/%d\n", i + 1, c.n_layer);
+        CompressedWeight* all[7] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.w_gate, &L.w_up, &L.w_down};
+        for (int t = 0; ok && t < 7; t++) ok = load_compressed(model_path, p + kTensorNames[t], *all[t]);
+        if (ok && ((i + 1) % 8 == 0 || i == c.n_layer - 1)) printf("  Loaded layer %d/%d\n", i + 1, c.n_layer);
+    }
+    if (!ok) {                                      // a file changed under the check, or could not be read
+        free_model(m);
+        return nullptr;
     }
     alloc_kv_cache(m, default_context(c));
     printf("  Context length: %d\n  Model loaded.\n", m->max_seq_len);
