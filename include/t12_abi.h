@@ -144,6 +144,17 @@ int t12_gemm_swiglu(const T12Segment* gate, const T12Segment* up, const void* ac
                     int K, int B, void* out_bf16, int out_stride, void* stream);
 int t12_tune_gemm(int ksplit);
 
+/* t12_gemm for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference (its GEMM never splits K and so has no
+ * workspace).  Same operands, kernels, K split and results as t12_gemm, bit for bit; the partial sums of a
+ * K-split launch go to a fixed array of T12_GEMM_NOALLOC_WS_BYTES inside the library's device image (every GPU
+ * the library runs on holds one until the process ends) and the call never calls hipMalloc / hipFree.  A launch
+ * whose partial sums (nsplit * B * sum of M * 4 bytes) exceed the array is refused with T12_EINVAL.  All calls on
+ * one GPU share the array: calls that overlap in time on one GPU, on any streams, race. */
+#define T12_GEMM_NOALLOC_WS_BYTES (32u << 20)
+int t12_gemm_noalloc(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride,
+                     int out_stride, int K, int B, void* stream);
+
 /* ---- (c) standalone decompress --------------------------------------------
  * out_bf16[m*K + k] = decoded weight bits.  patched != 0: escapes take
  * `correct` (lossless, bit-exact with the tensor that was packed).

@@ -129,6 +129,7 @@ _SIGS = {
     "nv_launch_split12_cublas_batch_async": (_i, [_vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_gemm": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_tune_gemm": (_i, [_i]),
+    "t12_gemm_noalloc": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_gemm_swiglu": (_i, [C.POINTER(Segment), C.POINTER(Segment), _vp, _i, _i, _i, _vp, _i, _vp]),
     "t12_gemm_deferred": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, C.POINTER(GemmPartials), _vp]),
     "launch_sum_add_rms_norm_bf16_batch": (None, [_vp, _vp, _i, C.c_size_t, _i, _vp, _vp, _vp, _i, C.c_float, _i, _vp]),

@@ -580,6 +580,27 @@ float* workspace(size_t bytes, hipStream_t st)
     return w.ptr;
 }
 
+// ---- the same workspace for callers that may not allocate: a fixed array in the code object's own device
+//      memory.  Every GPU the library runs on holds its own copy at its own address; the name below is only a
+//      host-side handle for hipGetSymbolAddress, never a pointer a kernel could use.
+constexpr size_t STATIC_WS_BYTES = (size_t)T12_GEMM_NOALLOC_WS_BYTES;
+static __device__ __align__(256) float g_static_ws[STATIC_WS_BYTES / sizeof(float)];
+std::mutex g_static_ws_mutex;
+float* g_static_ws_ptr[16] = {};                       // per device, filled on the first call on that device
+
+float* static_workspace()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
+    std::lock_guard<std::mutex> lock(g_static_ws_mutex);
+    if (!g_static_ws_ptr[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_ws)) != hipSuccess || !ptr) return nullptr;
+        g_static_ws_ptr[dev] = (float*)ptr;
+    }
+    return g_static_ws_ptr[dev];
+}
+
 int g_gemm_ksplit = 0;   // 0 = choose by shape
 
 template <int WB, int WM, int FB, int FM, bool SWI = false>
@@ -667,10 +688,14 @@ int t12_gemm_swiglu(const T12Segment* gate, const T12Segment* up, const void* ac
     return launch_mfma<4, 2, 2, 2, true>(p, tiles, (hipStream_t)stream);
 }
 
-// t12_gemm whose K-split partial sums may be left in the workspace for the caller's next kernel to add
-// up (part != NULL): part->nsplit == 1 means the outputs are complete in segs[].out.
-int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride, int out_stride, int K,
-                      int B, T12GemmPartials* part, void* stream)
+}  // extern "C"
+
+namespace {
+
+// The body of t12_gemm / t12_gemm_deferred / t12_gemm_noalloc.  static_ws: the K-split partial sums go to the
+// library's fixed device array instead of a grown hipMalloc buffer, and a launch that needs more is refused.
+int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride, int out_stride, int K,
+              int B, T12GemmPartials* part, void* stream, bool static_ws)
 {
     if (part) {
         part->ws = nullptr;
@@ -746,7 +771,18 @@ int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, in
     ks = (K + kslice - 1) / kslice;
     p.ksplit = ks;
     p.kslice = kslice;
-    if (ks > 1) {
+    if (ks > 1 && static_ws) {
+        const size_t need = (size_t)ks * B * m_total * sizeof(float);
+        T12_REQUIRE(need <= STATIC_WS_BYTES,
+                    "t12_gemm_noalloc: this shape splits K %d ways and needs %zu bytes of partial sums, the fixed "
+                    "workspace holds %zu (B %d x %d rows): use t12_gemm, or a smaller batch", ks, need, STATIC_WS_BYTES, B,
+                    m_total);
+        p.ws = static_workspace();
+        if (!p.ws) {
+            t12_set_error("t12_gemm_noalloc: hipGetSymbolAddress of the fixed workspace failed");
+            return T12_ELAUNCH;
+        }
+    } else if (ks > 1) {
         p.ws = workspace((size_t)ks * B * m_total * sizeof(float), st);
         if (!p.ws) {
             t12_set_error("t12_gemm: cannot allocate %zu bytes of K-split workspace",
@@ -770,6 +806,29 @@ int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, in
         T12_CHECK_LAUNCH("t12_gemm(reduce)");
     }
     return T12_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+// t12_gemm whose K-split partial sums may be left in the workspace for the caller's next kernel to add
+// up (part != NULL): part->nsplit == 1 means the outputs are complete in segs[].out.
+int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride, int out_stride, int K,
+                      int B, T12GemmPartials* part, void* stream)
+{
+    return gemm_impl(segs, nseg, act_bf16, act_stride, out_stride, K, B, part, stream, false);
+}
+
+// t12_gemm for callers that may not allocate device memory (HIP graph capture, serving loops, harnesses that forbid
+// it): same kernels, same K split, same results bit for bit; the partial sums of a split launch live in a fixed
+// T12_GEMM_NOALLOC_WS_BYTES array inside the library's device image instead of a buffer grown with hipMalloc.
+// Every launch writes each partial sum it later adds, so the array needs no clearing between calls; all calls on
+// one GPU share it, whatever their stream: calls that overlap in time on one GPU race.
+int t12_gemm_noalloc(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride, int out_stride, int K,
+                     int B, void* stream)
+{
+    return gemm_impl(segs, nseg, act_bf16, act_stride, out_stride, K, B, nullptr, stream, true);
 }
 
 }  // extern "C"
