@@ -217,3 +217,46 @@ def test_pipelined_decode_equals_step_by_step(t12, small_model, B):
     finally:
         os.environ.pop("TURBO_NO_PIPELINE", None)
         eng.close()
+
+
+def test_two_states_on_their_own_streams_do_not_share_scratch(t12, small_model):
+    """Two states of one model (own cache regions, own streams) decode past 256 positions -- where a B = 1 launch
+    splits the context across workgroups and keeps partial results and arrival counters in library-owned scratch --
+    with their forwards and argmax launches enqueued alternately and no synchronisation in between.  The scratch is
+    per (device, stream), so each state's logits and tokens equal those of the same steps run alone."""
+    path, _ = small_model
+    rng = np.random.default_rng(21)
+    n_prompt, n_steps = 300, 24
+    prompts = [[int(t) for t in rng.integers(3, SMALL["n_vocab"], size=n_prompt)] for _ in range(2)]
+    base = t12.Engine.load(path, batch=1)
+    states = [base.new_state(1, per_sequence=400) for _ in range(2)]
+    try:
+        # alone: prompt, then greedy steps one state after the other
+        alone_tokens, alone_logits = [], []
+        for st, prompt in zip(states, prompts):
+            st.set_positions([0])
+            st.prefill_rows(prompt, 64)
+            toks = []
+            for _ in range(n_steps):
+                t = st.sample()[0]
+                toks.append(t)
+                st.forward([t])
+            alone_tokens.append(toks)
+            alone_logits.append(st.logits(SMALL["n_vocab"]).clone())
+        # together: the same steps, enqueued alternately
+        for st, prompt in zip(states, prompts):
+            st.set_positions([0])
+            st.prefill_rows(prompt, 64)
+        both = [[], []]
+        for _ in range(n_steps):
+            toks = [st.sample()[0] for st in states]        # (sample synchronises its own stream only)
+            for i, st in enumerate(states):
+                both[i].append(toks[i])
+                st.forward([toks[i]])
+        for i, st in enumerate(states):
+            assert both[i] == alone_tokens[i]
+            assert torch.equal(st.logits(SMALL["n_vocab"]), alone_logits[i])
+    finally:
+        for st in states:
+            st.close()
+        base.close()

@@ -16,8 +16,10 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <type_traits>
+#include <utility>
 #include <vector>
 
 #include "t12_device.h"
@@ -1235,50 +1237,77 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const ArgPair* __restr
     if (threadIdx.x == 0) result[blockIdx.x] = p.i == 0x7FFFFFFF ? 0 : p.i;
 }
 
-// ---- library-owned device state: RoPE table (keyed by head_dim AND theta) and the
-//      argmax partial buffer.  Guarded for use from several host threads.
+// ---- library-owned device state.  RoPE tables: one per (device, head_dim, theta, scaling rule), built on first
+//      use and kept until the process ends (a table is 256 bytes; none is ever freed, so a pointer handed to a launch
+//      stays valid whatever other threads do).  Scratch of the argmax and of the context-split attention: one set per
+//      (device, stream) -- launches on different streams may overlap and must not share partial results or arrival
+//      counters; launches on one stream are ordered.  Guarded for use from several host threads; two host threads
+//      that launch on the SAME stream still share that stream's scratch, like any other buffer they would share.
 std::mutex g_mu;
-float* g_freqs = nullptr;
-int g_freqs_dim = 0;
-float g_freqs_theta = 0.0f;
-ArgPair* g_part = nullptr;
-int g_part_rows = 0;
+struct RopeKey {
+    int dev, head_dim;
+    float theta, scale[4];
+    bool operator<(const RopeKey& o) const { return memcmp(this, &o, sizeof(RopeKey)) < 0; }
+};
+std::map<RopeKey, float*> g_rope_tables;
+struct StreamScratch {
+    ArgPair* part = nullptr;       // argmax partials [part_rows][ARG_CHUNKS]
+    int part_rows = 0;
+    float* split_ws = nullptr;     // context-split attention: partial results
+    int* split_cnt = nullptr;      //   and arrival counters (zero between launches)
+};
+std::map<std::pair<int, hipStream_t>, StreamScratch> g_scratch;
 
 // Frequency scaling of the "llama3" kind (factor <= 0: none); set by launch_rope_scaling
 float g_rope_scale[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-float g_freqs_scale[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+
+int current_device()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    return dev;
+}
 
 const float* rope_table(int head_dim, float theta)
 {
     std::lock_guard<std::mutex> lock(g_mu);
-    if (g_freqs && g_freqs_dim == head_dim && g_freqs_theta == theta &&
-        memcmp(g_freqs_scale, g_rope_scale, sizeof g_rope_scale) == 0)
-        return g_freqs;
+    RopeKey key;
+    memset(&key, 0, sizeof key);
+    key.dev = current_device();
+    key.head_dim = head_dim;
+    key.theta = theta;
+    memcpy(key.scale, g_rope_scale, sizeof key.scale);
+    auto it = g_rope_tables.find(key);
+    if (it != g_rope_tables.end()) return it->second;
     const int half = head_dim / 2;
+    if (half < 1) return nullptr;
     std::vector<float> h(half);
     t12_rope_freqs(head_dim, theta, g_rope_scale[0], g_rope_scale[1], g_rope_scale[2], g_rope_scale[3], h.data());
-    if (g_freqs) (void)hipFree(g_freqs);
-    g_freqs = nullptr;
-    if (hipMalloc((void**)&g_freqs, half * sizeof(float)) != hipSuccess) return nullptr;
-    if (hipMemcpy(g_freqs, h.data(), half * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) return nullptr;
-    g_freqs_dim = head_dim;
-    g_freqs_theta = theta;
-    memcpy(g_freqs_scale, g_rope_scale, sizeof g_rope_scale);
-    return g_freqs;
+    float* d = nullptr;
+    if (hipMalloc((void**)&d, half * sizeof(float)) != hipSuccess) return nullptr;
+    if (hipMemcpy(d, h.data(), half * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipFree(d);
+        return nullptr;
+    }
+    g_rope_tables[key] = d;
+    return d;
 }
 
-ArgPair* argmax_scratch(int rows)
+// The argmax partial buffer of this (device, stream), grown on demand (the old one is freed: hipFree waits for
+// the device, and only launches on this very stream ever read it).
+ArgPair* argmax_scratch(int rows, hipStream_t st)
 {
     std::lock_guard<std::mutex> lock(g_mu);
-    if (g_part_rows < rows) {
-        if (g_part) (void)hipFree(g_part);
-        g_part = nullptr;
-        g_part_rows = 0;
+    StreamScratch& sc = g_scratch[{current_device(), st}];
+    if (sc.part_rows < rows) {
+        if (sc.part) (void)hipFree(sc.part);
+        sc.part = nullptr;
+        sc.part_rows = 0;
         const int want = rows < 256 ? 256 : rows;
-        if (hipMalloc((void**)&g_part, (size_t)want * ARG_CHUNKS * sizeof(ArgPair)) != hipSuccess) return nullptr;
-        g_part_rows = want;
+        if (hipMalloc((void**)&sc.part, (size_t)want * ARG_CHUNKS * sizeof(ArgPair)) != hipSuccess) return nullptr;
+        sc.part_rows = want;
     }
-    return g_part;
+    return sc.part;
 }
 
 void report(const char* what)
@@ -1320,22 +1349,26 @@ int g_attn_wide = 0;    // contexts from this length on take the INT8 MFMA form 
 constexpr int ATT_SPLIT_WGS = 512;     // also: at most ATT_TILE / 2 chunks per (sequence, KV head)
 constexpr int ATT_SPLIT_HEADS = 4096;
 constexpr int ATT_SPLIT_TARGET = 256;  // workgroups a split launch aims for
-float* g_split_ws = nullptr;
-int* g_split_cnt = nullptr;
 
-bool attn_split_scratch()
+// The context-split scratch of this (device, stream); nullptr when it cannot be allocated.
+StreamScratch* attn_split_scratch(hipStream_t st)
 {
     std::lock_guard<std::mutex> lock(g_mu);
-    if (g_split_ws) return true;
+    StreamScratch& sc = g_scratch[{current_device(), st}];
+    if (sc.split_ws) return &sc;
     const size_t ws_bytes = (size_t)ATT_SPLIT_WGS * 8 * (128 + 4) * sizeof(float);     // RATIO <= 8, HD <= 128
-    if (hipMalloc((void**)&g_split_ws, ws_bytes) != hipSuccess) { g_split_ws = nullptr; return false; }
-    if (hipMalloc((void**)&g_split_cnt, ATT_SPLIT_HEADS * sizeof(int)) != hipSuccess ||
-        hipMemset(g_split_cnt, 0, ATT_SPLIT_HEADS * sizeof(int)) != hipSuccess) {
-        (void)hipFree(g_split_ws);
-        g_split_ws = nullptr;
-        return false;
+    float* ws = nullptr;
+    int* cnt = nullptr;
+    if (hipMalloc((void**)&ws, ws_bytes) != hipSuccess) return nullptr;
+    if (hipMalloc((void**)&cnt, ATT_SPLIT_HEADS * sizeof(int)) != hipSuccess ||
+        hipMemset(cnt, 0, ATT_SPLIT_HEADS * sizeof(int)) != hipSuccess) {
+        (void)hipFree(ws);
+        if (cnt) (void)hipFree(cnt);
+        return nullptr;
     }
-    return true;
+    sc.split_ws = ws;
+    sc.split_cnt = cnt;
+    return &sc;
 }
 
 bool attn_has_fast(int n_head, int n_head_kv, int head_dim)
@@ -1366,11 +1399,12 @@ void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float
         // (4 sequences at 4000 positions: 18.8 us with 256 workgroups, 22.3 us with 512)
         const int room = ATT_SPLIT_TARGET / (batch * n_head_kv);
         int want = std::min(std::min(room, ATT_TILE / 2), (seq_len + g_attn_chunk - 1) / g_attn_chunk);
-        if (want > 1 && attn_split_scratch()) {
+        StreamScratch* sc = want > 1 ? attn_split_scratch(st) : nullptr;
+        if (sc) {
             sp.chunk_len = (((seq_len + want - 1) / want) + 63) & ~63;
             nchunk = (seq_len + sp.chunk_len - 1) / sp.chunk_len;
-            sp.ws = g_split_ws;
-            sp.counter = g_split_cnt;
+            sp.ws = sc->split_ws;
+            sp.counter = sc->split_cnt;
         }
     }
     // Two forms of the kernel.  First form: scores by fp32 FMAs with one thread per position, P.V with one wave per
@@ -1760,7 +1794,7 @@ void launch_flash_attention_batch(const float* q, const int8_t* kv_k, const int8
 
 void launch_argmax_batch(const float* logits, int* results, int n_vocab, int batch_size, hipStream_t stream)
 {
-    ArgPair* part = argmax_scratch(batch_size);
+    ArgPair* part = argmax_scratch(batch_size, stream);
     if (!part) { t12_set_error("argmax: cannot allocate scratch"); return; }
     hipLaunchKernelGGL(argmax_part_kernel, dim3(ARG_CHUNKS, batch_size), dim3(256), 0, stream, logits, n_vocab, part);
     hipLaunchKernelGGL(argmax_final_kernel, dim3(batch_size), dim3(64), 0, stream, part, results);
