@@ -59,6 +59,8 @@ int   t12_engine_generate(void* state, const int* prompt, int n_prompt, int max_
 /* decode_greedy: the decode half of generate, from the logits the state holds: up to max_tokens steps of
  * (sample, forward), the next step enqueued before the host has read the token.  out may be NULL. */
 int   t12_engine_decode(void* state, int max_tokens, int stop_on_eos, int* out);
+/* decode_greedy_until: decode_greedy with the stop id named by the caller (-1: none). */
+int   t12_engine_decode_until(void* state, int max_tokens, int stop_id, int* out);
 /* decode_greedy_all: the same loop without the stop rule, every sequence's ids: out[t * batch + b] (host, room
  * for max_tokens * batch ints, may be NULL); returns the number of steps. */
 int   t12_engine_decode_all(void* state, int max_tokens, int* out);

@@ -76,8 +76,14 @@ std::vector<int> generate(InferenceState* state, const std::vector<int>& prompt_
 // The decode half of generate (extension): up to max_tokens greedy steps from the logits the state
 // holds, each a sample followed by a forward on the sampled ids; returns the ids of sequence 0.
 // forward(state, nullptr) runs on the ids already in state->d_tokens (device) -- what lets the loop
-// enqueue step t + 1 before the host has seen token t.
+// enqueue step t + 1 before the host has seen token t.  The loop alternates state->logits between two buffers
+// (the pointer may differ after the call); when a stop id ends the stream, state->logits are the logits it was
+// sampled from, as in the reference's sample-wait-forward order (TURBO_NO_PIPELINE, read when the state is created).
 std::vector<int> decode_greedy(InferenceState* state, int max_tokens, bool stop_on_eos);
+
+// decode_greedy with the stop id named by the caller (-1: none): sequence 0 sampling it ends the stream; it is not
+// returned, the positions do not count it, and state->logits are the logits it was sampled from.
+std::vector<int> decode_greedy_until(InferenceState* state, int max_tokens, int stop_id);
 
 // decode_greedy without the stop rule, returning every sequence's ids: element [t * batch_size + b].
 std::vector<int> decode_greedy_all(InferenceState* state, int max_tokens);

@@ -185,6 +185,17 @@ def test_synthetic_model_save_load_roundtrip(t12, tmp_path):
         b.close()
 
 
+def _state_with_order(base, B, sequential):
+    """A state on base's model whose greedy loop runs pipelined, or in the reference's sample-wait-forward order
+    (TURBO_NO_PIPELINE, read when the state is created)."""
+    if sequential:
+        os.environ["TURBO_NO_PIPELINE"] = "1"
+    try:
+        return base.new_state(B)
+    finally:
+        os.environ.pop("TURBO_NO_PIPELINE", None)
+
+
 @pytest.mark.parametrize("B", [1, 3])
 def test_pipelined_decode_equals_step_by_step(t12, small_model, B):
     """decode_greedy enqueues step t + 1 on the device-resident ids before the host has read token t;
@@ -193,30 +204,90 @@ def test_pipelined_decode_equals_step_by_step(t12, small_model, B):
     path, _ = small_model
     rng = np.random.default_rng(11)
     prompts = [[int(t) for t in rng.integers(3, SMALL["n_vocab"], size=5)] for _ in range(12)]
-    eng = t12.Engine.load(path, batch=B)
+    base = t12.Engine.load(path, batch=1)
+    engs = [_state_with_order(base, B, True), _state_with_order(base, B, False)]     # (they share the model's cache region)
     try:
         saw_eos = False
         for prompt in prompts:
             runs = []
-            for env in ("1", None):
-                if env:
-                    os.environ["TURBO_NO_PIPELINE"] = env
-                else:
-                    os.environ.pop("TURBO_NO_PIPELINE", None)
+            for eng in engs:
                 toks = eng.generate(prompt, 40)
                 runs.append((toks, eng.positions()))
             assert runs[0] == runs[1]
             saw_eos = saw_eos or len(runs[0][0]) < 40
             assert runs[0][1] == [len(prompt) + len(runs[0][0])] * B
         # decode() continues from the logits left behind, without the stop rule
-        os.environ["TURBO_NO_PIPELINE"] = "1"
-        a = eng.generate(prompts[0], 8) + eng.decode(8)
-        os.environ.pop("TURBO_NO_PIPELINE", None)
-        b = eng.generate(prompts[0], 8) + eng.decode(8)
+        a = engs[0].generate(prompts[0], 8) + engs[0].decode(8)
+        b = engs[1].generate(prompts[0], 8) + engs[1].decode(8)
         assert a == b and (len(a) == 16 or 2 in a or saw_eos)
     finally:
-        os.environ.pop("TURBO_NO_PIPELINE", None)
-        eng.close()
+        for e in engs:
+            e.close()
+        base.close()
+
+
+@pytest.mark.parametrize("B", [1, 2])
+def test_stop_leaves_the_state_as_the_sequential_order_does(t12, small_model, B):
+    """When a stop id ends the stream, the pipelined loop has already enqueued the forward on that id: positions are
+    stepped back AND state->logits are the logits the stop id was sampled from (the loop alternates two logits
+    buffers), so whatever the caller does next -- look at the logits, decode again -- matches the reference's order."""
+    path, _ = small_model
+    rng = np.random.default_rng(12)
+    prompt = [int(t) for t in rng.integers(3, SMALL["n_vocab"], size=6)]
+    base = t12.Engine.load(path, batch=1)
+    seq, pipe = _state_with_order(base, B, True), _state_with_order(base, B, False)
+    try:
+        def prompt_in(e):
+            for i, t in enumerate(prompt):
+                e.set_positions([i] * B)
+                e.forward([t] * B)
+        prompt_in(seq)
+        free_run = seq.decode(12)
+        assert len(free_run) == 12
+        stop = free_run[7]                                   # the stream must stop before its 8th token
+        k = free_run.index(stop)
+        results = []
+        for e in (seq, pipe):
+            prompt_in(e)
+            got = e.decode_until(12, stop)
+            lg = e.logits(SMALL["n_vocab"]).clone()
+            again = e.decode_until(5, stop)                  # the same logits: the stop id comes first again
+            results.append((got, e.positions(), lg, again, e.decode_until(3, -1)))
+        assert results[0][0] == free_run[:k] and results[0][3] == []
+        assert int(results[0][2][0].argmax()) == stop
+        for a, b in zip(results[0], results[1]):
+            assert torch.equal(a, b) if torch.is_tensor(a) else a == b
+    finally:
+        seq.close()
+        pipe.close()
+        base.close()
+
+
+def test_stop_id_with_the_cache_exactly_full(t12, small_model):
+    """The last cache row is written, the next sampled id is the stop id: the loop ends cleanly in both orders (the
+    pipelined one must not enqueue a forward past the cache before it has looked at the id)."""
+    path, _ = small_model
+    rng = np.random.default_rng(13)
+    base = t12.Engine.load(path, batch=1)
+    seq, pipe = _state_with_order(base, 1, True), _state_with_order(base, 1, False)
+    try:
+        max_seq = t12.lib.t12_engine_max_seq(base.model)
+        start = max_seq - 6
+        tok0 = int(rng.integers(3, SMALL["n_vocab"]))
+        seq.set_positions([start]); seq.forward([tok0])
+        stream = seq.decode(5)                               # fills positions start+1 .. max_seq-1
+        assert seq.positions() == [max_seq]
+        stop = seq.sample()[0]                               # what comes next with the cache full
+        outs = []
+        for e in (seq, pipe):
+            e.set_positions([start]); e.forward([tok0])
+            outs.append((e.decode_until(8, stop), e.positions()))
+        assert outs[0] == outs[1]
+        assert outs[0][0] == stream[:stream.index(stop)] if stop in stream else outs[0] == (stream, [max_seq])
+    finally:
+        seq.close()
+        pipe.close()
+        base.close()
 
 
 def test_two_states_on_their_own_streams_do_not_share_scratch(t12, small_model):

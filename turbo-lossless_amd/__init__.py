@@ -102,6 +102,7 @@ _SIGS = {
     "t12_engine_sample": (_i, [_vp, C.POINTER(C.c_int)]),
     "t12_engine_generate": (_i, [_vp, C.POINTER(C.c_int), _i, _i, C.POINTER(C.c_int)]),
     "t12_engine_decode": (_i, [_vp, _i, _i, C.POINTER(C.c_int)]),
+    "t12_engine_decode_until": (_i, [_vp, _i, _i, C.POINTER(C.c_int)]),
     "t12_engine_sync": (_i, [_vp]),
     "t12_engine_shift_context": (_i, [_vp, _i, _i, _i]),
     "t12_engine_chat_turn": (_i, [_vp, C.POINTER(C.c_int), C.POINTER(C.c_int), _i, _i, _i, _i, _i, C.POINTER(C.c_int),
@@ -383,6 +384,12 @@ class Engine:
         """Up to max_tokens greedy steps (sample, forward) from the current logits; ids of sequence 0."""
         out = (C.c_int * max(max_tokens, 1))()
         n = lib.t12_engine_decode(self.state, max_tokens, int(stop_on_eos), out)
+        return list(out[:n])
+
+    def decode_until(self, max_tokens, stop_id):
+        """Greedy steps until sequence 0 samples stop_id (not returned; -1: never) or max_tokens."""
+        out = (C.c_int * max(max_tokens, 1))()
+        n = lib.t12_engine_decode_until(self.state, max_tokens, int(stop_id), out)
         return list(out[:n])
 
     def shift_context(self, current_pos, discard, seq=0):

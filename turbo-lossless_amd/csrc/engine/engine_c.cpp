@@ -95,6 +95,14 @@ int t12_engine_decode(void* state, int max_tokens, int stop_on_eos, int* out)
     return (int)r.size();
 }
 
+int t12_engine_decode_until(void* state, int max_tokens, int stop_id, int* out)
+{
+    std::vector<int> r = decode_greedy_until((InferenceState*)state, max_tokens, stop_id);
+    if (out)
+        for (size_t i = 0; i < r.size(); i++) out[i] = r[i];
+    return (int)r.size();
+}
+
 // decode_greedy_all(); out is a host array [max_tokens][batch]; returns the number of steps.
 int t12_engine_decode_all(void* state, int max_tokens, int* out)
 {

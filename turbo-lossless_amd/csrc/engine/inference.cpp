@@ -71,6 +71,11 @@ struct Impl {
     float* psv = nullptr;
     // prefill_rows: a state of that many rows on the same model, whose buffers carry a batch-1 state's prompt passes
     InferenceState* helper = nullptr;
+    // pipelined decoding: the second logits buffer (the forward enqueued ahead of the host's look at a token writes
+    // there, so the logits that produced an end-of-stream token are still in place when the loop stops)
+    float* logits_alt = nullptr;
+    // read once, when the state is created
+    bool no_pipeline = false;
 };
 
 // Where a forward reads and writes the KV cache: layer l of sequence b starts at
@@ -205,6 +210,7 @@ InferenceState* create_inference_state(Model* model, int batch_size, int max_seq
     impl->layers.resize(c.n_layer);
     const char* nofuse = getenv("TURBO_NO_FUSE");     // debugging aid: one kernel per reference kernel
     impl->fused_b1 = !(nofuse && nofuse[0] == '1');   // confirmed against the tensors at the first forward
+    impl->no_pipeline = getenv("TURBO_NO_PIPELINE") != nullptr;   // the reference's order: sample, wait, forward
     s->impl = impl;
     init_sampler(batch_size);
     return s;
@@ -261,7 +267,7 @@ void free_inference_state(InferenceState* state)
             if (impl->h_tokens[i]) (void)hipHostFree(impl->h_tokens[i]);
             if (impl->sampled[i]) (void)hipEventDestroy(impl->sampled[i]);
         }
-        for (void* p : {(void*)impl->pk, (void*)impl->pv, (void*)impl->psk, (void*)impl->psv})
+        for (void* p : {(void*)impl->pk, (void*)impl->pv, (void*)impl->psk, (void*)impl->psv, (void*)impl->logits_alt})
             if (p) (void)hipFree(p);
         free_inference_state(impl->helper);
     }
@@ -655,8 +661,8 @@ std::vector<int> decode_loop(InferenceState* state, int max_tokens, int stop_a, 
     const int n_vocab = state->model->config.n_vocab;
     const int bs = state->batch_size;
     hipStream_t st = state->stream;
-    const bool no_pipeline = getenv("TURBO_NO_PIPELINE") != nullptr;
-    if (no_pipeline) {
+    Impl* impl = (Impl*)state->impl;
+    if (impl->no_pipeline) {
         std::vector<int> tokens(bs);
         for (int t = 0; t < max_tokens; t++) {
             if (bs == 1) tokens[0] = sample_greedy(state->logits, n_vocab, st);
@@ -669,7 +675,8 @@ std::vector<int> decode_loop(InferenceState* state, int max_tokens, int stop_a, 
         }
         return output;
     }
-    Impl* impl = (Impl*)state->impl;
+    if (!impl->logits_alt)
+        check_gpu(hipMalloc((void**)&impl->logits_alt, (size_t)bs * n_vocab * sizeof(float)), "hipMalloc");
     for (int i = 0; i < 2; i++) {
         if (!impl->h_tokens[i]) check_gpu(hipHostMalloc((void**)&impl->h_tokens[i], bs * sizeof(int)), "hipHostMalloc");
         if (!impl->sampled[i]) check_gpu(hipEventCreateWithFlags(&impl->sampled[i], hipEventDisableTiming), "hipEventCreate");
@@ -681,19 +688,35 @@ std::vector<int> decode_loop(InferenceState* state, int max_tokens, int stop_a, 
         must(t12_util_copy_i32(impl->h_tokens[slot], state->d_tokens, bs, st), "token copy");
         (void)hipEventRecord(impl->sampled[slot], st);
     };
+    const int max_seq = kv_view(state).max_seq;
     if (max_tokens > 0) enqueue_sample(0);
     for (int t = 0; t < max_tokens; t++) {
-        forward(state, nullptr);                                  // on the ids the argmax left in d_tokens
-        if (t + 1 < max_tokens) enqueue_sample((t + 1) & 1);
+        // The forward on token t is enqueued before the host has seen token t -- unless the cache is full: then the
+        // host looks first, as the reference's order does, and a stop id ends the stream without an error.
+        int max_pos = 0;
+        for (int b = 0; b < bs; b++) max_pos = std::max(max_pos, state->positions[b]);
+        const bool ahead = max_pos < max_seq;
+        if (ahead) {
+            std::swap(state->logits, impl->logits_alt);           // keep the logits token t came from
+            forward(state, nullptr);                              // on the ids the argmax left in d_tokens
+            if (t + 1 < max_tokens) enqueue_sample((t + 1) & 1);
+        }
         check_gpu(hipEventSynchronize(impl->sampled[t & 1]), "hipEventSynchronize");
         const int tok = impl->h_tokens[t & 1][0];
         if (is_stop(tok)) {
-            for (int b = 0; b < bs; b++) state->positions[b]--;   // the forward on the end-of-stream id does not count
+            if (ahead) {
+                for (int b = 0; b < bs; b++) state->positions[b]--;   // the forward on the end-of-stream id does not count
+                std::swap(state->logits, impl->logits_alt);           // state->logits: those that produced the stop id
+            }
             break;
         }
         if (all_rows) output.insert(output.end(), impl->h_tokens[t & 1], impl->h_tokens[t & 1] + bs);
         else output.push_back(tok);
         if (on_token) on_token(tok);
+        if (!ahead) {
+            forward(state, nullptr);                              // reports the full cache like the sequential order
+            if (t + 1 < max_tokens) enqueue_sample((t + 1) & 1);
+        }
     }
     check_gpu(hipStreamSynchronize(st), "hipStreamSynchronize");
     return output;
@@ -703,6 +726,11 @@ std::vector<int> decode_loop(InferenceState* state, int max_tokens, int stop_a, 
 std::vector<int> decode_greedy(InferenceState* state, int max_tokens, bool stop_on_eos)
 {
     return decode_loop(state, max_tokens, stop_on_eos ? 2 : -1, -1, false, nullptr);
+}
+
+std::vector<int> decode_greedy_until(InferenceState* state, int max_tokens, int stop_id)
+{
+    return decode_loop(state, max_tokens, stop_id, -1, false, nullptr);
 }
 
 std::vector<int> decode_greedy_all(InferenceState* state, int max_tokens)
