@@ -142,6 +142,17 @@ def cpu_baseline(torch, launches, cfg, runs=3, n_weights_model=None):
     }
 
 
+def calibration_copy(torch, dev):
+    """One plain device-to-device copy kernel of exactly 1 GiB (torch's elementwise copy of an int32 tensor): the
+    launch of known size that the profiler's FETCH_SIZE / WRITE_SIZE readings are scaled by."""
+    src = torch.empty(2**28, dtype=torch.int32, device=dev).random_(0, 1 << 30)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
+
 def ext_stream(torch, ptr):
     return torch.cuda.ExternalStream(ptr)
 
@@ -518,11 +529,7 @@ def run_gemm_layers(args, t12, torch, dev):
     g.manual_seed(2100)
     cur = torch.cuda.current_stream()
     if args.calibrate:
-        src = torch.empty(2**30, dtype=torch.uint8, device=dev).random_(0, 255)
-        dst = torch.empty_like(src)
-        t12.check(t12.lib.t12_util_copy(dst.data_ptr(), src.data_ptr(), src.numel(), 8192, cur.cuda_stream), "t12_util_copy")
-        torch.cuda.synchronize()
-        del src, dst
+        calibration_copy(torch, dev)
     layers = gemm_layer_leg(t12, torch, dev, cfg, weight_of, 3, cur, g, iters=max(args.steps, 10))
     us256 = sum(layers["%s_b256" % k]["us"] for k in ("qkv", "o", "gate_up", "down"))
     fl256 = sum(layers["%s_b256" % k]["flops"] for k in ("qkv", "o", "gate_up", "down"))
@@ -563,7 +570,7 @@ def main():
     ap.add_argument("--layers", type=int, default=LLAMA8B["n_layer"], help="debug: fewer layers (invalid as a result)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
-                    help="also launch one plain 1 GiB copy kernel (t12_util_copy) before the steps: the known-size "
+                    help="also launch one plain 1 GiB copy kernel (a torch tensor copy) before the steps: the known-size "
                          "yardstick for the profiler's FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -617,11 +624,7 @@ def main():
                 t12.check(rc, "t12_gemv")
 
     if args.calibrate:
-        src = torch.empty(2**30, dtype=torch.uint8, device=dev).random_(0, 255)
-        dst = torch.empty_like(src)
-        t12.check(t12.lib.t12_util_copy(dst.data_ptr(), src.data_ptr(), src.numel(), 8192, stream), "t12_util_copy")
-        torch.cuda.synchronize()
-        del src, dst
+        calibration_copy(torch, dev)
 
     for _ in range(args.warmup):
         step()

@@ -61,17 +61,9 @@ typedef struct T12Segment {
 const char* t12_version(void);
 const char* t12_last_error(void);      /* text of the last failure on this thread */
 
-/* ---- calibration kernels (no counterpart in the reference) ------------------
- * Plain streaming read / copy of `bytes` (a multiple of 16) with `blocks`
- * workgroups of 256 lanes: the yardstick for achieved HBM bandwidth and for the
- * profiler's FETCH_SIZE / WRITE_SIZE counters.  `sink` holds blocks x u32. */
-int t12_util_read(const void* src, size_t bytes, void* sink, int blocks, void* stream);
-int t12_util_copy(void* dst, const void* src, size_t bytes, int blocks, void* stream);
-/* dst[0..n) = src[0..n) (32-bit words) by a kernel; dst may be pinned host memory. */
+/* dst[0..n) = src[0..n) (32-bit words) by a kernel; dst may be pinned host memory (the engine's sampled ids reach the
+ * host this way, without a DMA-engine hand-over in the middle of the stream).  No counterpart in the reference. */
 int t12_util_copy_i32(void* dst, const void* src, int n, void* stream);
-/* Pins the B = 1 kernel variant (100*waves + 10*rows_per_wave + ring depth);
- * 0 restores the choice by shape.  For benchmark sweeps. */
-int t12_tune_gemv(int variant);
 
 /* ---- (a) decode-GEMV, one activation vector ------------------------------
  * out_s[m] = sum_k dec(W_s[m,k]) * x[k] for every segment s, escapes exact.
@@ -119,7 +111,6 @@ int t12_gemv_batch(const T12Segment* segs, int nseg, const void* act_bf16, int a
 int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride,
              int out_stride, int K, int B, void* stream);
 
-/* Pins the number of K splits of the MFMA path; 0 restores the choice by shape. */
 /* t12_gemm with the last step left to the caller: when the launch splits K across workgroups, the
  * partial sums stay in the library's per-device workspace and *part describes them,
  *   value[b, m] = sum over z < nsplit (ascending) of ws[z * split_stride + b * ld + (segment's first column) + m],
@@ -142,7 +133,6 @@ int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, in
  * then; negative on bad operands. */
 int t12_gemm_swiglu(const T12Segment* gate, const T12Segment* up, const void* act_bf16, int act_stride,
                     int K, int B, void* out_bf16, int out_stride, void* stream);
-int t12_tune_gemm(int ksplit);
 
 /* t12_gemm for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  No counterpart in the reference (its GEMM never splits K and so has no

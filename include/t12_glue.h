@@ -142,12 +142,14 @@ void launch_rope_store_attention_partials_regions(float* q, float* k, const floa
                                                   size_t split_stride, int ld, int kv_stride, int region_positions,
                                                   hipStream_t stream);
 
-/* Benchmark switch.  0: always the general attention kernel.  1 (default): shapes with a specialised kernel
+/* Process-wide choice of the decode-attention kernel form, for comparisons (set it before launching; it is read at
+ * every launch, atomically, and is not a per-call argument because the reference-named launchers have fixed
+ * signatures).  0: always the general attention kernel.  1 (default): shapes with a specialised kernel
  * (head_dim 128 with GQA ratio 1/2/4/8, head_dim 64 with ratio 1/4) use it in its INT8 MFMA form (scores and P.V by
  * v_mfma_i32_32x32x32_i8: Q in three INT8 limbs, the softmax weights in two, K and V as stored), and a launch without a
  * position array whose batch * n_head_kv workgroups would leave the chip idle is split along the context into
  * chunks of at least 256 positions (partial softmax per chunk, folded by the workgroup that finishes last; the
- * partial results live in a library-owned buffer, so two such launches on different streams must not overlap).
+ * partial results live in a buffer the library keeps per device and stream).
  * 2: never split.  3: the specialised kernels in their fp32 FMA form.  4: same as 1.  n >= 16: chunks of at least n
  * positions. */
 int t12_tune_attention(int mode);

@@ -51,18 +51,38 @@ def test_gemm_shapes(t12, oracle, synth, M, K, B):
     assert rel_err(un, oracle.gemm(p, X, patched=False)) < TOL
 
 
-def test_gemm_ksplit_values_agree(t12, oracle, synth):
-    M, K, B = 256, 4096, 96
-    p = oracle.pack(synth.weights_llm(M, K, seed=5, p_outlier=1e-3))
-    X = synth.activations(B, K, seed=6)
-    ref = oracle.gemm(p, X)
-    try:
-        for ks in (1, 2, 3, 4, 8, 16):
-            t12.check(t12.lib.t12_tune_gemm(ks))
-            (got,) = run_gemm(t12, [p], X)
-            assert rel_err(got, ref) < TOL, ks
-    finally:
-        t12.lib.t12_tune_gemm(0)
+def test_gemm_every_k_split(t12, oracle, synth):
+    """One row tile (M = 128): the launch splits K across workgroups as far as its rule allows, so the length of K
+    picks the number of splits.  The number the library chose is read back through t12_gemm_deferred; every count from
+    1 to 16 that is a power of two must occur among the cases, and chunks that are not a power of two (K = 1088,
+    6272).  The summed result is checked against the oracle both through t12_gemm (its own reduction launch) and
+    through the deferred partial sums added up on the host."""
+    import ctypes as C
+    M = 128
+    seen = set()
+    for K, B in [(256, 96), (512, 96), (1024, 96), (2048, 96), (4096, 96), (8192, 96), (16384, 96), (4096, 200),
+                 (8192, 200), (16384, 40), (1088, 40), (6272, 96), (64, 33)]:
+        p = oracle.pack(synth.weights_llm(M, K, seed=K + B, p_outlier=1e-3))
+        X = synth.activations(B, K, seed=6)
+        ref = oracle.gemm(p, X)
+        (got,) = run_gemm(t12, [p], X)
+        assert rel_err(got, ref) < TOL, (K, B)
+        dt = t12.DeviceTensor12.from_packed(p, dev())
+        Xd = to_dev_bits(X).reshape(X.shape)
+        out = torch.full((B, M), float("nan"), device=dev())
+        part = t12.GemmPartials()
+        segs = t12._seg_array([dt.segment(out)])
+        t12.check(t12.lib.t12_gemm_deferred(segs, 1, Xd.data_ptr(), K, M, K, B, C.byref(part), t12.current_stream()))
+        torch.cuda.synchronize()
+        seen.add(part.nsplit)
+        if part.nsplit > 1:
+            ws = torch.empty(part.nsplit * part.split_stride, dtype=torch.float32, device=dev())
+            assert t12._hip_memcpy_d2d(ws.data_ptr(), part.ws, ws.numel() * 4) == 0
+            tot = ws.view(part.nsplit, B, part.ld)[:, :, :M].sum(dim=0)
+            assert rel_err(tot.cpu().numpy(), ref) < TOL, (K, B, part.nsplit)
+        else:
+            assert rel_err(out.cpu().numpy(), ref) < TOL, (K, B)
+    assert {1, 2, 4, 8, 16} <= seen, seen
 
 
 def test_gemm_fused_segments_and_strides(t12, oracle, synth):
@@ -173,19 +193,20 @@ def test_deferred_reduction_into_add_rms_norm(t12, oracle, synth, M, K, B):
 def test_gemm_more_escapes_than_the_lds_list_holds(t12, oracle, synth, B):
     """A 128-row tile with ~10 k escapes overflows the in-LDS escape list (1536 / 2048 entries): the kernel then
     multiplies the unpatched values and adds (correct - wrong) * x per entry in its epilogue -- still exact to
-    fp32 rounding, with and without a K split."""
+    fp32 rounding, with a K split (few row tiles) and without one (many)."""
     M, K = 256, 4096
     p = oracle.pack(synth.weights_llm(M, K, seed=77, p_outlier=3e-2))
     assert p.P > 2 * 4096                       # > 2048 entries in every 128-row tile
     X = synth.activations(B, K, seed=B + 1)
     ref = oracle.gemm(p, X)
-    try:
-        for ks in (0, 1, 4):
-            t12.lib.t12_tune_gemm(ks)
-            (got,) = run_gemm(t12, [p], X)
-            assert rel_err(got, ref) < TOL, ks
-    finally:
-        t12.lib.t12_tune_gemm(0)
+    (got,) = run_gemm(t12, [p], X)                      # two row tiles: K is split 4 ways (B <= 128: 8)
+    assert rel_err(got, ref) < TOL
+    # without a K split: the same rows as the first 256 of a tensor with enough row tiles to fill the chip
+    M2 = 128 * 200
+    w2 = np.tile(oracle.decode(p), (M2 // M, 1))
+    p2 = oracle.pack(w2, p.base_exp)
+    (got2,) = run_gemm(t12, [p2], X)
+    assert rel_err(got2[:, :M], ref) < TOL and rel_err(got2[:, M2 - M:], ref) < TOL
 
 
 @pytest.mark.parametrize("M,K,B,p_out", [(14336, 4096, 256, 3e-4), (12300, 512, 129, 2e-3), (12352, 256, 300, 5e-2),

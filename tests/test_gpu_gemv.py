@@ -133,21 +133,6 @@ def test_gemv_nonfinite(t12, oracle, synth):
     assert rel_err(got[mask], ref[mask]) < TOL
 
 
-def test_all_variants_agree(t12, oracle, synth):
-    M, K = 520, 4096
-    w = synth.weights_llm(M, K, seed=31, p_outlier=1e-3)
-    x = synth.activations(1, K, seed=32)[0]
-    p = oracle.pack(w)
-    ref = oracle.gemv(p, x)
-    try:
-        for v in [810, 811, 812, 814, 411, 412, 414, 421, 422, 424, 442, 99]:
-            t12.check(t12.lib.t12_tune_gemv(v))
-            (got,) = run_gemv(t12, [p], x)
-            assert rel_err(got, ref) < TOL, v
-    finally:
-        t12.lib.t12_tune_gemv(0)
-
-
 def test_reference_named_launchers(t12, oracle, synth):
     """launch_split12_v2_async (+dual) give the UNPATCHED product; the patch launchers add
     (correct - wrong) * x -- the call sequence of the reference's forward_b1."""

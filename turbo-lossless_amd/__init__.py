@@ -44,9 +44,6 @@ _vp, _i = C.c_void_p, C.c_int
 _SIGS = {
     "t12_version": (C.c_char_p, []),
     "t12_last_error": (C.c_char_p, []),
-    "t12_tune_gemv": (_i, [_i]),
-    "t12_util_read": (_i, [_vp, C.c_size_t, _vp, _i, _vp]),
-    "t12_util_copy": (_i, [_vp, _vp, C.c_size_t, _i, _vp]),
     "t12_pack_histogram": (_i, [_vp, C.c_size_t, _vp, _vp]),
     "t12_pack_base_exp": (_i, [C.POINTER(C.c_uint64)]),
     "t12_pack_planes": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
@@ -129,7 +126,6 @@ _SIGS = {
     "nv_launch_patches_batch_async": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _i, _vp]),
     "nv_launch_split12_cublas_batch_async": (_i, [_vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_gemm": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
-    "t12_tune_gemm": (_i, [_i]),
     "t12_gemm_noalloc": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_gemm_swiglu": (_i, [C.POINTER(Segment), C.POINTER(Segment), _vp, _i, _i, _i, _vp, _i, _vp]),
     "t12_gemm_deferred": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, C.POINTER(GemmPartials), _vp]),

@@ -601,7 +601,6 @@ float* static_workspace()
     return g_static_ws_ptr[dev];
 }
 
-int g_gemm_ksplit = 0;   // 0 = choose by shape
 
 template <int WB, int WM, int FB, int FM, bool SWI = false>
 int launch_mfma(GemmParams& p, int tiles, hipStream_t st)
@@ -631,13 +630,6 @@ int launch_mfma(GemmParams& p, int tiles, hipStream_t st)
 }  // namespace
 
 extern "C" {
-
-// Pins the number of K splits of the MFMA path (benchmark sweeps); 0 = by shape.
-int t12_tune_gemm(int ksplit)
-{
-    g_gemm_ksplit = ksplit;
-    return T12_OK;
-}
 
 int t12_gemm(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride, int out_stride, int K, int B,
              void* stream)
@@ -764,9 +756,7 @@ int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_st
     const int want = 256 * per_cu;
     int ks = 1;
     const int min_stages = B > 128 ? 16 : 8;
-    if (g_gemm_ksplit > 0) ks = g_gemm_ksplit < T12_MAX_KSPLIT ? g_gemm_ksplit : T12_MAX_KSPLIT;
-    else
-        while (tiles * btiles * ks * 4 < want * 3 && K / (ks * 2) >= min_stages * KC && ks < T12_MAX_KSPLIT) ks *= 2;
+    while (tiles * btiles * ks * 4 < want * 3 && K / (ks * 2) >= min_stages * KC && ks < T12_MAX_KSPLIT) ks *= 2;
     int kslice = (((K + 2 * KC - 1) / (2 * KC) + ks - 1) / ks) * 2 * KC;      // whole windows of two stages
     ks = (K + kslice - 1) / kslice;
     p.ksplit = ks;

@@ -384,8 +384,6 @@ __global__ __launch_bounds__(256) void patches_kernel(const GemvParams p)
     if (lane == 0 && c != 0.0f) sg.out[row] += c;
 }
 
-int g_gemv_variant = 0;   // 0 = choose by shape; see t12_tune_gemv
-
 template <int NW, int R, int D, int MINB = 1>
 int launch_stream(GemvParams& p, const T12Segment* segs, int nseg, hipStream_t st)
 {
@@ -476,13 +474,6 @@ int gemv_impl(const T12Segment* segs, int nseg, const void* act_bf16, int K, con
 
 extern "C" {
 
-// Selects the B = 1 kernel variant (benchmark sweeps): 0 = by shape.
-int t12_tune_gemv(int variant)
-{
-    g_gemv_variant = variant;
-    return T12_OK;
-}
-
 int t12_gemv(const T12Segment* segs, int nseg, const void* act_bf16, int K, void* stream)
 {
     return gemv_impl(segs, nseg, act_bf16, K, nullptr, stream);
@@ -516,7 +507,7 @@ int gemv_impl(const T12Segment* segs, int nseg, const void* act_bf16, int K, con
         p.seg[i] = segs[i];
         if (segs[i].base_exp < 0 || segs[i].base_exp > 240) fast = false;
     }
-    if (!fast || g_gemv_variant == 99) {
+    if (!fast) {
         int total = 0;
         for (int i = 0; i < nseg; i++) {
             p.blk_start[i] = total;
@@ -527,34 +518,14 @@ int gemv_impl(const T12Segment* segs, int nseg, const void* act_bf16, int K, con
         T12_CHECK_LAUNCH("t12_gemv(general)");
         return T12_OK;
     }
-    // variant = 100*NW + 10*R + D ; 0 = by shape.  The ring depth may not exceed the
-    // number of whole 1024-column tiles.  Measured on MI355X (Llama-3.1-8B layer
-    // shapes): 8 waves x 1 row x depth 2 is the fastest everywhere -- the chip
-    // hides HBM latency better with many light waves (62 VGPRs, 8 waves/SIMD)
-    // than with deep per-wave rings.
+    // 8 waves x 1 row per wave x a ring two tiles deep (as deep as the row has whole 1024-column tiles): measured on
+    // MI355X over the Llama-3.1-8B layer shapes against 4-wave workgroups, two and four rows per wave and rings of
+    // depth 4, this is the fastest everywhere -- the chip hides HBM latency better with many light waves (62 VGPRs,
+    // 8 waves per SIMD) than with deep per-wave rings.
     const int T = K / 1024;
-    int v = g_gemv_variant ? g_gemv_variant : 812;
-    const int dmax = T >= 4 ? 4 : (T >= 2 ? 2 : T);
-    if (v % 10 > dmax) v = v - v % 10 + dmax;
-    if (v % 10 == 0 && T > 0) v += 1;               // depth 0 only exists for K < 1024
-    switch (v) {
-        case 810: return launch_stream<8, 1, 0>(p, segs, nseg, st);
-        case 811: return launch_stream<8, 1, 1>(p, segs, nseg, st);
-        case 812: return launch_stream<8, 1, 2>(p, segs, nseg, st);
-        case 814: return launch_stream<8, 1, 4>(p, segs, nseg, st);
-        case 410: return launch_stream<4, 1, 0>(p, segs, nseg, st);
-        case 411: return launch_stream<4, 1, 1>(p, segs, nseg, st);
-        case 412: return launch_stream<4, 1, 2>(p, segs, nseg, st);
-        case 414: return launch_stream<4, 1, 4>(p, segs, nseg, st);
-        case 420: return launch_stream<4, 2, 0>(p, segs, nseg, st);
-        case 421: return launch_stream<4, 2, 1>(p, segs, nseg, st);
-        case 422: return launch_stream<4, 2, 2>(p, segs, nseg, st);
-        case 424: return launch_stream<4, 2, 4>(p, segs, nseg, st);
-        case 442: return launch_stream<4, 4, 2>(p, segs, nseg, st);
-        default:
-            t12_set_error("t12_gemv: unknown kernel variant %d", v);
-            return T12_EINVAL;
-    }
+    if (T >= 2) return launch_stream<8, 1, 2>(p, segs, nseg, st);
+    if (T == 1) return launch_stream<8, 1, 1>(p, segs, nseg, st);
+    return launch_stream<8, 1, 0>(p, segs, nseg, st);
 }
 
 }  // namespace

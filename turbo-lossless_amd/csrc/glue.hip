@@ -14,6 +14,7 @@
 // float_to_bf16 (kernels.hip:21-27).
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstring>
 #include <map>
@@ -1340,9 +1341,13 @@ void launch_rope_kv(float* q, float* k, const float* v, int8_t* ck, int8_t* cv, 
     report("rope/kv-store");
 }
 
-int g_attn_fast = 1;   // 0: always the general kernel (tests compare the two)
-int g_attn_chunk = 256; // context split: fewest positions per chunk; 0 = never split
-int g_attn_wide = 0;    // contexts from this length on take the INT8 MFMA form (measured faster at every length)
+// The kernel form in use (t12_tune_attention); one word, read once per launch.
+//   bits 0..23: context split, fewest positions per chunk (0 = never split); bit 24: specialised kernels allowed;
+//   bit 25: their fp32 FMA form instead of the INT8 MFMA form
+std::atomic<int> g_attn_mode{256 | (1 << 24)};
+#define g_attn_fast ((attn_mode_now & (1 << 24)) != 0)
+#define g_attn_chunk (attn_mode_now & 0xFFFFFF)
+#define g_attn_wide ((attn_mode_now & (1 << 25)) ? 0x7FFFFFFF : 0)
 
 // Scratch of the context split: partial results of at most ATT_SPLIT_WGS workgroups and one
 // counter per (sequence, KV head); the counters start at zero and every launch leaves them there.
@@ -1373,6 +1378,7 @@ StreamScratch* attn_split_scratch(hipStream_t st)
 
 bool attn_has_fast(int n_head, int n_head_kv, int head_dim)
 {
+    const int attn_mode_now = g_attn_mode.load(std::memory_order_relaxed);
     if (!g_attn_fast || n_head_kv <= 0 || n_head % n_head_kv) return false;
     const int r = n_head / n_head_kv;
     return (head_dim == 128 && (r == 1 || r == 2 || r == 4 || r == 8)) || (head_dim == 64 && (r == 1 || r == 4));
@@ -1383,6 +1389,7 @@ void launch_attn(const float* q, const int8_t* ck, const int8_t* cv, const float
                  const int* positions, int seq_len, int n_head, int n_head_kv, int head_dim, float scale, int batch,
                  size_t kv_stride, hipStream_t st, const AttnFuse* fuse = nullptr, int hm = 0)
 {
+    const int attn_mode_now = g_attn_mode.load(std::memory_order_relaxed);
     const int ratio = n_head / n_head_kv;
     if (ratio < 1 || ratio > ATT_MAX_RATIO || n_head % n_head_kv || head_dim % 16 || head_dim > 128) {
         t12_set_error("attention: unsupported heads %d/%d or head_dim %d (needs ratio <= %d, head_dim %% 16 == 0, <= 128)",
@@ -1496,9 +1503,8 @@ void launch_rope_scaling(float factor, float low_freq_factor, float high_freq_fa
 // kernels in their fp32 FMA form (one wave per head); 4: same as 1; n >= 16: chunks of at least n positions.
 int t12_tune_attention(int mode)
 {
-    g_attn_fast = mode != 0;
-    g_attn_chunk = mode >= 16 ? mode : (mode == 2 ? 0 : 256);
-    g_attn_wide = mode == 3 ? 0x7FFFFFFF : 0;
+    const int chunk = mode >= 16 ? (mode & 0xFFFFFF) : (mode == 2 ? 0 : 256);
+    g_attn_mode.store(chunk | (mode != 0 ? 1 << 24 : 0) | (mode == 3 ? 1 << 25 : 0), std::memory_order_relaxed);
     return 0;
 }
 
