@@ -122,23 +122,35 @@ def cpu_baseline(torch, launches, cfg, runs=3, n_weights_model=None):
             packs.append(p)
     rng = np.random.default_rng(7)
     xs = {K: oracle.f32_to_bf16_bits(rng.standard_normal(K).astype(np.float32)) for K in {p.K for p in packs}}
-    times = []
-    t_begin = time.perf_counter()
-    while len(times) < runs or (time.perf_counter() - t_begin < 10.0 and len(times) < 2000):   # ~10 s of CPU work
-        t0 = time.perf_counter()
-        for p in packs:
-            oracle.gemv(p, xs[p.K])
-        times.append(time.perf_counter() - t0)
-    runs = len(times)
-    t_layer = sorted(times)[len(times) // 2]
     w_layer = sum(p.M * p.K for p in packs)
     w_model = n_weights_model or sum(t.M * t.K for tensors, _ in launches for t in tensors)
+
+    def leg(seconds):
+        times = []
+        t_begin = time.perf_counter()
+        while len(times) < runs or (time.perf_counter() - t_begin < seconds and len(times) < 2000):
+            t0 = time.perf_counter()
+            for p in packs:
+                oracle.gemv(p, xs[p.K])
+            times.append(time.perf_counter() - t0)
+        return sorted(times)[len(times) // 2], len(times)
+
+    oracle.set_num_threads(0)                      # every host core the process may use
+    threads = oracle.num_threads()
+    t_layer, n_all = leg(10.0)                     # ~10 s of CPU work
+    oracle.set_num_threads(1)
+    t_one, n_one = leg(8.0)                        # ~8 s more on one thread
+    oracle.set_num_threads(0)
     t_model = t_layer * w_model / w_layer
     return {
-        "value": 1.0 / t_model, "unit": "tok/s", "cores": oracle.num_threads(), "kind": "port",
-        "sample": "decoder layer 0 (wq,wk,wv,wo,gate,up,down = %d weights) x%d runs (~10 s), median %.4f s, scaled by weight "
-                  "count to the %d-weight model; %.2f GB/s compressed" % (w_layer, runs, t_layer, w_model,
-                                                                          1.5 * w_layer / t_layer / 1e9),
+        "value": 1.0 / t_model, "unit": "tok/s", "cores": threads, "kind": "port",
+        "nproc": os.cpu_count(),
+        "one_thread": {"value": 1.0 / (t_one * w_model / w_layer), "unit": "tok/s", "cores": 1,
+                       "GBps_compressed": 1.5 * w_layer / t_one / 1e9, "runs": n_one},
+        "sample": "decoder layer 0 (wq,wk,wv,wo,gate,up,down = %d weights) x%d runs (~10 s) on %d threads, median %.4f s, "
+                  "scaled by weight count to the %d-weight model; %.2f GB/s compressed; then the same layer x%d runs on "
+                  "one thread (median %.4f s)" % (w_layer, n_all, threads, t_layer, w_model,
+                                                  1.5 * w_layer / t_layer / 1e9, n_one, t_one),
     }
 
 
@@ -288,7 +300,10 @@ def run_decode(args, t12, torch, dev):
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["gemv_stack_b1"] if n_l == LLAMA8B["n_layer"] else None,
                      "kernel": "gemv_stream_kernel", "bytes_per_launch": alg_bytes / len(tabs),
-                     "us_per_launch": ms_gemv * 1e3 / len(tabs)},
+                     "us_per_launch": ms_gemv * 1e3 / len(tabs),
+                     # the other target of the path: decode+GEMM at B = 256 over the four linear layers of a decoder
+                     # layer, against the dense bf16 MFMA peak (median launch times of gemm_layers above)
+                     "gemm_b256": gemm_b256_roofline(gemm_layers)},
         "setup_s": t_build,
     }
     if not args.no_cpu_baseline:
@@ -421,10 +436,13 @@ def run_attention(args, t12, torch, dev):
     }
 
 
-def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(16, 64, 256), iters=10):
+def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(4, 8, 16, 64, 256), iters=50):
     """decode+GEMM per layer shape: for each B, each of QKV (3 segments), O, gate|up
     (2 segments), down is timed over `n_rot` distinct weight copies in rotation, so that neither L2 nor
-    the 256 MB last-level cache holds a tensor between launches.  weight_of(copy, which) -> (segment, K, P)."""
+    the 256 MB last-level cache holds a tensor between launches.  weight_of(copy, which) -> (segment, K, P).
+    Per case: 5 untimed rounds, then `iters` (>= 50) rounds each bracketed by its own pair of HIP events on the
+    launch stream; the figure is the MEDIAN round divided by the launches in it."""
+    iters = max(iters, 50)
     out = {}
     groups = [(0, 1, 2), (3,), (4, 5), (6,)]
     names = ["qkv", "o", "gate_up", "down"]
@@ -448,13 +466,30 @@ def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(16, 
                     rc = t12.lib.t12_gemm(segs, n, act, K, 2 * cfg["n_ff"], K, B, cur.cuda_stream)
                     if rc:
                         t12.check(rc, "t12_gemm")
-            gemm_pass()
-            _, ms = timed(torch, cur, gemm_pass, iters)
-            us = ms * 1e3 / n_rot
+            for _ in range(5):
+                gemm_pass()
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+            torch.cuda.synchronize()
+            for e0, e1 in evs:
+                e0.record(cur)
+                gemm_pass()
+                e1.record(cur)
+            torch.cuda.synchronize()
+            rounds = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+            us = rounds[len(rounds) // 2] * 1e3 / n_rot
             out["%s_b%d" % (name, B)] = {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
                                          "mfma_frac": round(flops / us / 1e6 / 2500.0, 4),
                                          "weight_GBps": round(wbytes / us / 1e3, 1), "flops": flops}
     return out
+
+
+def gemm_b256_roofline(layers):
+    names = ("qkv", "o", "gate_up", "down")
+    us = sum(layers["%s_b256" % k]["us"] for k in names)
+    fl = sum(layers["%s_b256" % k]["flops"] for k in names)
+    return {"bound": "mfma", "achieved": fl / us / 1e6, "peak": 2500.0, "unit": "TFLOP/s", "frac": fl / us / 1e6 / 2500.0,
+            "traffic": None, "kernel": "gemm_mfma_kernel, QKV + O + gate|up + down at B=256", "flops_per_step": fl,
+            "us_per_step": us, "gate_up_frac": layers["gate_up_b256"]["mfma_frac"]}
 
 
 def run_tokenizer(args, t12):
@@ -530,13 +565,13 @@ def run_gemm_layers(args, t12, torch, dev):
     cur = torch.cuda.current_stream()
     if args.calibrate:
         calibration_copy(torch, dev)
-    layers = gemm_layer_leg(t12, torch, dev, cfg, weight_of, 3, cur, g, iters=max(args.steps, 10))
+    layers = gemm_layer_leg(t12, torch, dev, cfg, weight_of, 3, cur, g, iters=max(args.steps, 50))
     us256 = sum(layers["%s_b256" % k]["us"] for k in ("qkv", "o", "gate_up", "down"))
     fl256 = sum(layers["%s_b256" % k]["flops"] for k in ("qkv", "o", "gate_up", "down"))
     gu = layers["gate_up_b256"]
     return {
         "metric": "decode+GEMM TFLOP/s at B=256 over the linear layers of one Llama-3.1-8B decoder layer (split-12 weights)",
-        "value": fl256 / us256 / 1e6, "unit": "TFLOP/s", "n_gpus": 1, "steps": max(args.steps, 10), "warmup": 1,
+        "value": fl256 / us256 / 1e6, "unit": "TFLOP/s", "n_gpus": 1, "steps": max(args.steps, 50), "warmup": 5,
         "ms_per_step": us256 / 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "gemm_layers: QKV 4096->6144 (3 segments), O 4096->4096, gate|up 4096->28672 (2 segments), "

@@ -60,6 +60,8 @@ def lib():
         L.t12o_apply_patches.argtypes = [i32p, i32p, i16p, i16p, u16p, f32p, C.c_int]
         L.t12o_apply_patches.restype = None
         L.t12o_num_threads.restype = C.c_int
+        L.t12o_set_num_threads.argtypes = [C.c_int]
+        L.t12o_set_num_threads.restype = None
         _lib = L
     return _lib
 
@@ -173,6 +175,11 @@ def apply_patches(p: Packed, x_bits: np.ndarray, out: np.ndarray) -> None:
 
 def num_threads() -> int:
     return int(lib().t12o_num_threads())
+
+
+def set_num_threads(n: int) -> None:
+    """Threads of the C oracle's parallel loops from now on (n < 1: the OpenMP default)."""
+    lib().t12o_set_num_threads(int(n))
 
 
 # ------------------------------------------------------------------ engine glue

@@ -48,6 +48,12 @@ static inline uint32_t nibble_at(const uint8_t *gr, int64_t i)
     return (i & 1) ? (uint32_t)(b >> 4) : (uint32_t)(b & 0xF);
 }
 
+/* threads the parallel loops below use from now on (n < 1: back to the OpenMP default) */
+void t12o_set_num_threads(int n)
+{
+    omp_set_num_threads(n >= 1 ? n : omp_get_num_procs());
+}
+
 int t12o_num_threads(void)
 {
 #ifdef _OPENMP

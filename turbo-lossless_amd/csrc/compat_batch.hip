@@ -8,9 +8,11 @@
 // The position of an escape inside esc_vals is therefore defined by the
 // reference's thread mapping (256 lanes, lane t owns columns t, t+256, ...), so
 // this kernel keeps that column ownership; everything else is this library's:
-// esc_counts may be NULL (each lane then counts its own group-0 nibbles), the
-// K loop reads 4 columns per lane and step when K % 1024 == 0, and any batch
-// size 1..8 is one template.
+// esc_counts may be NULL (each lane then counts its own group-0 nibbles) and any
+// batch size 1..8 is one template.  That ownership (one column per lane and step,
+// byte loads) is also what bounds this kernel; it exists for callers that hold the
+// derived tables -- the engine itself sends batches of 2..8 through t12_gemm, which
+// reads the CSR list and streams 16 columns per lane.
 #include "t12_device.h"
 #include "t12_host.h"
 
