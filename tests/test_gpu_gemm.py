@@ -295,3 +295,46 @@ def test_reference_named_batch_entry_points(t12, oracle, synth, M, K, B):
     torch.cuda.synchronize()
     assert rel_err(un.cpu().numpy(), ref) < TOL
     assert t12.lib.nv_launch_patches_batch_async(None, None, None, None, None, 0, None, K, None, M, B, st) == 0   # nothing to do
+
+
+@pytest.mark.parametrize("B", [2, 4, 5, 8, 9, 16])
+@pytest.mark.parametrize("M,K,law", [(4096, 4096, "llm"), (1000, 1280, "diffusion"), (37, 128, "llm"), (2560, 10240, "diffusion"),
+                                     (28672, 256, "llm"), (16, 14336, "llm")])
+def test_gemm_small_batches_dense_sweep(t12, oracle, synth, M, K, law, B):
+    """B <= 16 with K % 128 == 0 takes the kernel that sweeps whole rows (16 rows per workgroup, the waves of a
+    workgroup interleaved over the 128-column blocks, activations straight from memory): ragged row counts, one
+    block per row, rows with far more escapes than waves (the diffusion law: ~50-100 per row at K = 10240), row
+    counts that make it share activation loads across two and four row groups, padded batches."""
+    w = synth.weights_diffusion(M, K, seed=M + K) if law == "diffusion" else synth.weights_llm(M, K, seed=M + K, p_outlier=1e-3)
+    p = oracle.pack(w)
+    X = synth.activations(B, K, seed=B)
+    (got,) = run_gemm(t12, [p], X)
+    assert rel_err(got, oracle.gemm(p, X)) < TOL
+    (un,) = run_gemm(t12, [p], X, patched=False)
+    assert rel_err(un, oracle.gemm(p, X, patched=False)) < TOL
+
+
+def test_gemm_small_batch_segments_and_strides(t12, oracle, synth):
+    """Three tensors with three base_exp in one small-batch launch; activation rows with a padded stride; outputs in
+    column slices of one buffer; enough rows (2 x 14336 + 100) that the launch shares activation loads across row
+    groups and a segment ends inside a shared group."""
+    K, B = 512, 12
+    ps = [oracle.pack(synth.weights_llm(14336, K, seed=1, sigma=0.02)), oracle.pack(synth.weights_llm(100, K, seed=2, sigma=0.3)),
+          oracle.pack(synth.weights_llm(14336, K, seed=3, sigma=0.002))]
+    X = synth.activations(B, K, seed=4)
+    Xpad = torch.zeros((B, K + 64), dtype=torch.int16, device=dev())
+    Xpad[:, :K] = to_dev_bits(X).reshape(B, K)
+    dts = [t12.DeviceTensor12.from_packed(p, dev()) for p in ps]
+    total = sum(p.M for p in ps)
+    big = torch.full((B, total), float("nan"), device=dev())
+    outs, off = [], 0
+    for p in ps:
+        outs.append(big[:, off:off + p.M])
+        off += p.M
+    t12.gemm(dts, Xpad[:, :K], outs=outs)
+    torch.cuda.synchronize()
+    h = big.cpu().numpy()
+    off = 0
+    for p in ps:
+        assert rel_err(h[:, off:off + p.M], oracle.gemm(p, X)) < TOL
+        off += p.M

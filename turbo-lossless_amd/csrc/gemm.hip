@@ -555,6 +555,170 @@ __global__ __launch_bounds__(256) void gemm_general_kernel(const GemmParams p)
     }
 }
 
+// ---------------------------------------------------------------------------
+// Small batches (B <= 16): the dense-sweep kernel.  At these sizes the product is bound by the weight stream, and
+// what the memory system streams fastest is what the B = 1 kernel gives it: workgroups in launch order, each
+// sweeping a few whole rows quickly, so that the chip as a whole reads one dense window of the planes.  (Kernels
+// whose waves walk many rows slowly in parallel -- a K-split grid of 128-row tiles, a wave per 16 rows -- measure
+// 3.5-4.5 TB/s on the same bytes.)
+//   * a workgroup owns 16 consecutive weight rows and all of K; its NW waves take the 128-column blocks of the rows
+//     in turn (wave w: blocks w, w + NW, ...), so the workgroup as a whole reads its rows' planes front to back;
+//   * v_mfma_f32_16x16x32_bf16, activations = A operand (rows = batch), weights = B operand: lane (n, g) =
+//     (lane % 16, lane / 16) holds row n, so the planes go straight from HBM into the operand registers -- per
+//     block a lane loads 2 x 16 bytes of sign/mantissa (columns 32g .. 32g+15 and 32g+16 .. 32g+31: the four lanes
+//     of a row cover its 128-byte line in two back-to-back instructions) and 16 bytes of nibbles, rebuilds them
+//     with t12_decode8 and feeds four MFMAs;
+//   * the activations are not staged: lane (b, g) reads the 8 columns an MFMA needs straight from memory (they are
+//     B x K bf16, resident in L2) and pairs them in registers to match t12_decode8's order;
+//   * no barrier until the end, where the waves' partial 16 x 16 tiles are added through LDS in wave order;
+//   * escapes: the streamed value of a group-0 weight is its "wrong" value; wave w adds (correct - wrong) * x[b, col]
+//     for the entries w, w + NW, ... of each row (the four lanes of a row each for their four batch rows).
+// Requires K % 128 == 0, 0 <= base_exp <= 240, B <= 16.  blk_start counts 16-row groups per segment.
+// ---------------------------------------------------------------------------
+template <int NW, int D, int RG>
+__global__ __launch_bounds__(NW * 64) void gemm_dense16_kernel(const GemmParams p)
+{
+    __shared__ t12_f32x4 red[RG][NW][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, g = lane >> 4;
+
+    const int blk = blockIdx.x;
+    const int s = find_segment(p, blk);
+    const T12Segment& sg = p.seg[s];
+    const int M = sg.M, K = p.K, B = p.B;
+    const int m0 = (blk - p.blk_start[s]) * (16 * RG);               // RG groups of 16 rows share every activation load
+    const int nblk = K >> 7;                          // 128-column blocks per row
+    const int mine = nblk > wave ? (nblk - wave + NW - 1) / NW : 0;      // blocks of this wave
+    // A wave without a block (K < NW * 128) still issues the first D fetches below and drops them: it aims them at
+    // block 0, because its own first block would lie past the end of the row -- and, in the last rows of a plane or
+    // of the activations, past the end of the allocation.
+    const int wblk = mine > 0 ? wave : 0;
+    const uint32_t be2 = t12_opaque(((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23));
+
+    // CSR pointers of this lane's rows (used after the stream)
+    int e_beg[RG], e_end[RG];
+    const uint8_t* smp[RG];
+    const uint8_t* grp[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+        const int row = m0 + 16 * rg + n;
+        e_beg[rg] = e_end[rg] = 0;
+        if (sg.row_off && row < M) {
+            e_beg[rg] = sg.row_off[row];
+            e_end[rg] = sg.row_off[row + 1];
+        }
+        const size_t e0 = (size_t)min(row, M - 1) * K;              // rows past the end are clamped, never stored
+        smp[rg] = sg.sm + e0 + 32 * g + (size_t)wblk * 128;
+        grp[rg] = sg.gr + (e0 >> 1) + 16 * g + (size_t)wblk * 64;
+    }
+    const uint16_t* xp = p.act + (size_t)min(n, B - 1) * p.act_stride + 32 * g + (size_t)wblk * 128;
+    uint4 rS[D][RG][2], rG[D][RG], rX[D][4];
+#define T12_DS_FETCH(slot, j)                                                              \
+    {                                                                                      \
+        _Pragma("unroll") for (int q = 0; q < 4; q++)                                      \
+            rX[slot][q] = *(const uint4*)(xp + (size_t)(j) * (NW * 128) + 8 * q);          \
+        _Pragma("unroll") for (int rg = 0; rg < RG; rg++) {                                \
+            rS[slot][rg][0] = *(const uint4*)(smp[rg] + (size_t)(j) * (NW * 128));         \
+            rS[slot][rg][1] = *(const uint4*)(smp[rg] + (size_t)(j) * (NW * 128) + 16);    \
+            rG[slot][rg] = *(const uint4*)(grp[rg] + (size_t)(j) * (NW * 64));             \
+        }                                                                                  \
+    }
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+        T12_DS_FETCH(d, min(d, max(mine - 1, 0)))     // (fewer blocks than slots: the last one again, in bounds)
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // the first escape entries of the rows: wave w takes entry e_beg + w, requested now and used after the stream
+    int pcol[RG], pcorrect[RG], pwrong[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+        pcol[rg] = -1;
+        pcorrect[rg] = pwrong[rg] = 0;
+        if (e_beg[rg] + wave < e_end[rg]) {
+            pcol[rg] = sg.cols[e_beg[rg] + wave];
+            pcorrect[rg] = sg.correct[e_beg[rg] + wave];
+            pwrong[rg] = sg.wrong[e_beg[rg] + wave];
+        }
+    }
+
+    t12_f32x4 acc[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) acc[rg] = t12_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#define T12_DS_CONSUME(slot)                                                                                 \
+    _Pragma("unroll") for (int q = 0; q < 4; q++) {                                                          \
+        const uint4 xa = t12_pair_acts(rX[slot][q]);                                                         \
+        _Pragma("unroll") for (int rg = 0; rg < RG; rg++) {                                                  \
+            const uint4 sv = rS[slot][rg][q >> 1];                                                           \
+            const uint32_t gq = q == 0 ? rG[slot][rg].x : (q == 1 ? rG[slot][rg].y : (q == 2 ? rG[slot][rg].z : rG[slot][rg].w)); \
+            uint32_t w_[4];                                                                                  \
+            if (q & 1) t12_decode8(sv.z, sv.w, gq, be2, w_);                                                 \
+            else t12_decode8(sv.x, sv.y, gq, be2, w_);                                                       \
+            const uint4 wv = make_uint4(w_[0], w_[1], w_[2], w_[3]);                                         \
+            acc[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(t12_bf16x8, xa),            \
+                                                              __builtin_bit_cast(t12_bf16x8, wv), acc[rg], 0, 0, 0); \
+        }                                                                                                    \
+    }
+    int j = 0;
+    for (; j + 2 * D <= mine; j += D) {               // every slot is refilled
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            T12_DS_CONSUME(d)
+            T12_DS_FETCH(d, j + d + D)
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    for (; j < mine; j += D) {                        // the last (up to 2D - 1) blocks
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            if (j + d < mine) {
+                T12_DS_CONSUME(d)
+                if (j + d + D < mine) T12_DS_FETCH(d, j + d + D)
+            }
+        }
+    }
+#undef T12_DS_FETCH
+#undef T12_DS_CONSUME
+
+    // ---- escapes.  Accumulator register r of lane (n, g) is D[batch 4g + r][row n].
+    {
+        const uint16_t* xrow[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) xrow[r] = p.act + (size_t)min(4 * g + r, B - 1) * p.act_stride;
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            if (pcol[rg] >= 0) {
+                const float delta = t12_bf16_to_f32((uint16_t)pcorrect[rg]) - t12_bf16_to_f32((uint16_t)pwrong[rg]);
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[rg][r] += delta * t12_bf16_to_f32(xrow[r][pcol[rg]]);
+            }
+            for (int e = e_beg[rg] + wave + NW; e < e_end[rg]; e += NW) {        // rows with more than NW escapes
+                const int col = sg.cols[e];
+                const float delta = t12_bf16_to_f32((uint16_t)sg.correct[e]) - t12_bf16_to_f32((uint16_t)sg.wrong[e]);
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[rg][r] += delta * t12_bf16_to_f32(xrow[r][col]);
+            }
+        }
+    }
+
+    // ---- the waves' partial tiles, added in wave order; thread (r, l) = (tid / 64, tid % 64) of the first four waves
+    //      finishes element D[batch 4 (l / 16) + r][row l % 16] of every row group
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) red[rg][wave][lane] = acc[rg];
+    __syncthreads();
+    if (tid < 256) {
+        const int r = tid >> 6, l = tid & 63;
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            float v = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NW; w++) v += red[rg][w][l][r];
+            const int b = 4 * (l >> 4) + r, row = m0 + 16 * rg + (l & 15);
+            if (b < B && row < M) sg.out[(size_t)b * sg.out_stride + row] = v;
+        }
+    }
+}
+
 // ---- workspace for the K-split partial sums: one per (device, stream), grown on demand.  Launches on different
 //      streams may overlap, so they must not share partial sums; launches on one stream are ordered.
 struct Workspace {
@@ -747,6 +911,28 @@ int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_st
         tiles += (segs[i].M + TM - 1) / TM;
     }
     p.blk_start[nseg] = tiles;
+    if (B <= 16 && K % 128 == 0) {
+        // row groups that share an activation load: as many as leave the launch >= 448 workgroups
+        int groups16 = 0;
+        for (int i = 0; i < nseg; i++) groups16 += (segs[i].M + 15) / 16;
+        // (measured on 28672 x 4096: at B = 16 four groups per load 49 us against 56 with one; at B = 4 45 against 42:
+        // rows of a padded batch cost no activation traffic, more rows per wave cost registers)
+        const int want = B > 8 ? 4 : (B > 4 ? 2 : 1);
+        const int rg = groups16 >= 4 * 448 && want >= 4 ? 4 : (groups16 >= 2 * 448 && want >= 2 ? 2 : 1);
+        int groups = 0;
+        for (int i = 0; i < nseg; i++) {
+            p.blk_start[i] = groups;
+            groups += (segs[i].M + 16 * rg - 1) / (16 * rg);
+        }
+        p.blk_start[nseg] = groups;
+        p.ksplit = 1;
+        p.kslice = K;
+        if (rg == 4) hipLaunchKernelGGL((gemm_dense16_kernel<8, 2, 4>), dim3(groups), dim3(512), 0, st, p);
+        else if (rg == 2) hipLaunchKernelGGL((gemm_dense16_kernel<8, 2, 2>), dim3(groups), dim3(512), 0, st, p);
+        else hipLaunchKernelGGL((gemm_dense16_kernel<8, 2, 1>), dim3(groups), dim3(512), 0, st, p);
+        T12_CHECK_LAUNCH("t12_gemm(dense16)");
+        return T12_OK;
+    }
     // K split: fill the chip.  A 256-row batch tile needs a whole CU (LDS, accumulators);
     // smaller batch tiles fit 2-4 workgroups per CU.  Every split keeps >= 4 stages; with 256-row batch tiles
     // >= 8: a 4096 x 4096 tensor then runs as 128 workgroups in the time 256 take, and leaves half the partial
