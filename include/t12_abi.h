@@ -32,6 +32,7 @@ extern "C" {
 #define T12_OK          0
 #define T12_EINVAL     (-1)   /* bad shape / null pointer / unsupported size */
 #define T12_ELAUNCH    (-2)   /* HIP reported a launch or runtime error      */
+#define T12_EENGINE    (-3)   /* a t12_engine_* call failed (EngineError)    */
 #define T12_MAX_SEGMENTS 8
 #define T12_MAX_KSPLIT 16      /* most K splits a decode+GEMM launch uses (T12GemmPartials.nsplit) */
 

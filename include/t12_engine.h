@@ -2,6 +2,11 @@
  * include/turbo/{model,inference,sampler}.h: ctypes, cgo, JNI.  Each function forwards to the C++
  * function named beside it, which keeps the reference's name and meaning (engine/model.h:79-82,
  * engine/inference.h:43-55, engine/sampler.h:5-11).  Handles are the C++ objects as void*.
+ *
+ * Errors: where the reference ends the process (GPU_CHECK, gpu_compat.h:94-101; exit(1), inference.cpp:73,223,306)
+ * the C++ functions throw EngineError (include/turbo/model.h).  No exception crosses this interface: a function
+ * that returns int returns T12_EENGINE (counts are >= 0), one that returns a handle returns NULL, and
+ * t12_last_error() has the text.  A state whose call failed is good only for t12_engine_free_state.
  */
 #ifndef T12_ENGINE_H
 #define T12_ENGINE_H

@@ -6,8 +6,20 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <cstdint>
+#include <stdexcept>
 #include <string>
 #include <vector>
+
+// What the engine throws where the reference ends the process (its GPU_CHECK, gpu_compat.h:94-101, and the
+// `exit(1)` of inference.cpp:73,223,306): a failed GPU call, a launch the library refused, a position past the
+// cache, an argument outside the batch.  The message has already gone to stderr, as the reference prints it.  A
+// caller that does not catch it still ends (std::terminate); the C face (t12_engine_*) catches it and returns a
+// negative code with the text in t12_last_error().  The state the call worked on is not usable afterwards.
+struct EngineError : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+// Prints "ERROR: <text>" to stderr and throws EngineError(<text>).
+[[noreturn]] void engine_fail(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 
 // Model hyperparameters (config.bin: 7 x int32 + 2 x float32, engine/model.cpp:181-191)
 struct ModelConfig {

@@ -331,3 +331,38 @@ def test_two_states_on_their_own_streams_do_not_share_scratch(t12, small_model):
         for st in states:
             st.close()
         base.close()
+
+
+def test_errors_come_back_as_codes_not_as_a_dead_process(t12, small_model):
+    """Where the reference ends the process (a position past the cache: engine/inference.cpp:73,223,306 and its
+    GPU_CHECK), the C face returns T12_EENGINE with the text in t12_last_error(), and the Python wrapper raises.
+    Every condition here is found on the host before any kernel is launched."""
+    path, _ = small_model
+    base = t12.Engine.load(path, batch=1)
+    two = base.new_state(2)
+    try:
+        max_seq = t12.lib.t12_engine_max_seq(base.model)
+        base.set_positions([max_seq])
+        arr = (t12.C.c_int * 1)(5)
+        assert t12.lib.t12_engine_forward(base.state, arr) == -3
+        assert b"exceeds the KV cache" in t12.lib.t12_last_error()
+        with pytest.raises(t12.T12Error, match="exceeds the KV cache"):
+            base.forward([5])
+        base.set_positions([0])
+        with pytest.raises(t12.T12Error, match="outside the cache"):
+            base.shift_context(current_pos=4, discard=9)
+        with pytest.raises(t12.T12Error, match="outside the batch"):
+            two.prefill(2, [3, 4, 5])
+        with pytest.raises(t12.T12Error, match="batch size 1"):
+            two.prefill_rows([3, 4, 5], 4)
+        with pytest.raises(t12.T12Error, match="batch size 1"):
+            two.chat_turn(0, [3, 4], 4, 1, 2)
+        with pytest.raises(t12.T12Error, match="exceeds the KV cache"):
+            base.prefill_rows(list(range(3, 3 + max_seq + 1)), 8)
+        # the refusals above launched nothing: the state still decodes
+        base.set_positions([0])
+        base.forward([7])
+        assert len(base.decode(4)) == 4
+    finally:
+        two.close()
+        base.close()

@@ -152,6 +152,13 @@ def check(rc: int, what: str = "") -> None:
         raise T12Error("%s failed (%d): %s" % (what, rc, lib.t12_last_error().decode()))
 
 
+def _count(n: int, what: str) -> int:
+    """A t12_engine_* result that is a count when >= 0 and a T12_E* code otherwise."""
+    if n < 0:
+        raise T12Error("%s failed (%d): %s" % (what, n, lib.t12_last_error().decode()))
+    return n
+
+
 def _torch():
     import torch
     return torch
@@ -301,7 +308,10 @@ class Engine:
             if not st:
                 raise T12Error("per-sequence KV cache could not be created")
             return st
-        return lib.t12_engine_create_state(self.model, batch, 0)
+        st = lib.t12_engine_create_state(self.model, batch, 0)
+        if not st:
+            raise T12Error("inference state could not be created: %s" % lib.t12_last_error().decode())
+        return st
 
     @classmethod
     def load(cls, path, batch=1, device=0, per_sequence=0):
@@ -331,7 +341,7 @@ class Engine:
     def decode_all(self, max_tokens):
         """max_tokens greedy steps from the current logits; ids of every sequence as [steps][batch]."""
         out = (C.c_int * max(max_tokens * self.batch, 1))()
-        n = lib.t12_engine_decode_all(self.state, max_tokens, out)
+        n = _count(lib.t12_engine_decode_all(self.state, max_tokens, out), "decode_all")
         return [list(out[t * self.batch:(t + 1) * self.batch]) for t in range(n)]
 
     def save(self, path):
@@ -348,7 +358,7 @@ class Engine:
 
     def forward(self, tokens):
         arr = (C.c_int * self.batch)(*[int(t) for t in tokens])
-        lib.t12_engine_forward(self.state, arr)
+        check(lib.t12_engine_forward(self.state, arr), "forward")
 
     def sync(self):
         check(lib.t12_engine_sync(self.state), "stream sync")
@@ -367,25 +377,25 @@ class Engine:
 
     def sample(self):
         arr = (C.c_int * self.batch)()
-        lib.t12_engine_sample(self.state, arr)
+        check(lib.t12_engine_sample(self.state, arr), "sample")
         return list(arr)
 
     def generate(self, prompt, max_tokens):
         p = (C.c_int * len(prompt))(*[int(t) for t in prompt])
         out = (C.c_int * max(max_tokens, 1))()
-        n = lib.t12_engine_generate(self.state, p, len(prompt), max_tokens, out)
+        n = _count(lib.t12_engine_generate(self.state, p, len(prompt), max_tokens, out), "generate")
         return list(out[:n])
 
     def decode(self, max_tokens, stop_on_eos=False):
         """Up to max_tokens greedy steps (sample, forward) from the current logits; ids of sequence 0."""
         out = (C.c_int * max(max_tokens, 1))()
-        n = lib.t12_engine_decode(self.state, max_tokens, int(stop_on_eos), out)
+        n = _count(lib.t12_engine_decode(self.state, max_tokens, int(stop_on_eos), out), "decode")
         return list(out[:n])
 
     def decode_until(self, max_tokens, stop_id):
         """Greedy steps until sequence 0 samples stop_id (not returned; -1: never) or max_tokens."""
         out = (C.c_int * max(max_tokens, 1))()
-        n = lib.t12_engine_decode_until(self.state, max_tokens, int(stop_id), out)
+        n = _count(lib.t12_engine_decode_until(self.state, max_tokens, int(stop_id), out), "decode_until")
         return list(out[:n])
 
     def shift_context(self, current_pos, discard, seq=0):
@@ -402,8 +412,8 @@ class Engine:
         pos, dropped = C.c_int(int(current_pos)), C.c_int(0)
         arr = (C.c_int * max(len(tokens), 1))(*[int(t) for t in tokens])
         out = (C.c_int * max(max_tokens, 1))()
-        n = lib.t12_engine_chat_turn(self.state, C.byref(pos), arr, len(tokens), int(max_tokens), int(bos_id), int(eos_id),
-                                     int(prompt_rows), C.byref(dropped), out)
+        n = _count(lib.t12_engine_chat_turn(self.state, C.byref(pos), arr, len(tokens), int(max_tokens), int(bos_id),
+                                            int(eos_id), int(prompt_rows), C.byref(dropped), out), "chat_turn")
         return list(out[:n]), pos.value, dropped.value
 
     def weight(self, layer, which):

@@ -112,16 +112,14 @@ enum LogitsMode { LOGITS_ALL, LOGITS_LAST_ROW, LOGITS_NONE };
 void check_gpu(hipError_t e, const char* what)
 {
     if (e != hipSuccess) {
-        fprintf(stderr, "GPU error (%s): %s\n", what, hipGetErrorString(e));
-        exit(1);
+        engine_fail("GPU error (%s): %s", what, hipGetErrorString(e));
     }
 }
 
 T12Segment seg_of(const CompressedWeight& w, float* out, int out_stride)
 {
-    if (!w.split_sm) {   // same failure mode as the reference (inference.cpp:73,223,306)
-        fprintf(stderr, "ERROR: split12 data missing for weight %dx%d\n", w.M, w.K);
-        exit(1);
+    if (!w.split_sm) {   // where the reference ends the process (inference.cpp:73,223,306)
+        engine_fail("split12 data missing for weight %dx%d", w.M, w.K);
     }
     T12Segment s;
     s.sm = w.split_sm;
@@ -145,8 +143,7 @@ void run_linear(const T12Segment* segs, int nseg, const int16_t* act, int K, int
     if (B == 1) rc = t12_gemv(segs, nseg, act, K, st);
     else rc = t12_gemm(segs, nseg, act, K, segs[0].out_stride, K, B, st);
     if (rc != T12_OK) {
-        fprintf(stderr, "ERROR: split-12 linear launch failed: %s\n", t12_last_error());
-        exit(1);
+        engine_fail("split-12 linear launch failed: %s", t12_last_error());
     }
 }
 
@@ -157,8 +154,7 @@ void run_linear_add_norm(const T12Segment* seg, const int16_t* act, int K, int B
 {
     T12GemmPartials part;
     if (t12_gemm_deferred(seg, 1, act, K, seg->out_stride, K, B, &part, st) != T12_OK) {
-        fprintf(stderr, "ERROR: split-12 linear launch failed: %s\n", t12_last_error());
-        exit(1);
+        engine_fail("split-12 linear launch failed: %s", t12_last_error());
     }
     if (part.nsplit > 1)
         launch_sum_add_rms_norm_bf16_batch(seg->out, part.ws, part.nsplit, part.split_stride, part.ld, residual, norm_w,
@@ -294,8 +290,7 @@ bool fused_b1_eligible(const Model* m)
 void must(int rc, const char* what)
 {
     if (rc != T12_OK) {
-        fprintf(stderr, "ERROR: %s failed: %s\n", what, t12_last_error());
-        exit(1);
+        engine_fail("%s failed: %s", what, t12_last_error());
     }
 }
 
@@ -423,8 +418,7 @@ void forward_rows(InferenceState* state, int R, const KvView& kv, int pos0, Logi
         if (B > 1) {
             // a K-split q | k | v projection leaves its partial sums to the RoPE / KV-store kernel
             if (t12_gemm_deferred(S.qkv, 3, bf16_a, n, n, n, B, &qkv_part, st) != T12_OK) {
-                fprintf(stderr, "ERROR: split-12 linear launch failed: %s\n", t12_last_error());
-                exit(1);
+                engine_fail("split-12 linear launch failed: %s", t12_last_error());
             }
         } else {
             run_linear(S.qkv, 3, bf16_a, n, B, st);
@@ -463,15 +457,13 @@ void forward_rows(InferenceState* state, int R, const KvView& kv, int pos0, Logi
                                  L.w_up.base_exp >= 0 && L.w_up.base_exp <= 240;
         if (fuse_swiglu) {      // gate|up decode-GEMV with the SiLU*mul epilogue: one launch, no fp32 round trip
             if (t12_gemv_swiglu(&S.gateup[0], &S.gateup[1], bf16_a, n, bf16_b, st) != T12_OK) {
-                fprintf(stderr, "ERROR: fused gate|up launch failed: %s\n", t12_last_error());
-                exit(1);
+                engine_fail("fused gate|up launch failed: %s", t12_last_error());
             }
         } else {
             // gate|up decode+GEMM with the SiLU*mul in its epilogue where the shape has such a kernel
             const int rc = B > 1 ? t12_gemm_swiglu(&S.gateup[0], &S.gateup[1], bf16_a, n, n, B, bf16_b, n_ff, st) : 1;
             if (rc < 0) {
-                fprintf(stderr, "ERROR: fused gate|up launch failed: %s\n", t12_last_error());
-                exit(1);
+                engine_fail("fused gate|up launch failed: %s", t12_last_error());
             }
             if (rc == 1) {
                 run_linear(S.gateup, 2, bf16_a, n, B, st);
@@ -516,8 +508,7 @@ void forward(InferenceState* state, const int* token_ids)
     int max_pos = 0;
     for (int b = 0; b < B; b++) max_pos = std::max(max_pos, state->positions[b]);
     if (max_pos >= kv.max_seq) {
-        fprintf(stderr, "ERROR: position %d exceeds the KV cache (%d)\n", max_pos, kv.max_seq);
-        exit(1);
+        engine_fail("position %d exceeds the KV cache (%d)", max_pos, kv.max_seq);
     }
     if (B == 1 && impl->fused_b1) {
         if (!impl->checked) {
@@ -550,8 +541,7 @@ void prefill(InferenceState* state, int seq, const int* token_ids, int n_tokens)
     const int B = state->batch_size;
     Impl* impl = (Impl*)state->impl;
     if (seq < 0 || seq >= B || n_tokens < 0) {
-        fprintf(stderr, "ERROR: prefill: sequence %d outside the batch of %d, or negative length\n", seq, B);
-        exit(1);
+        engine_fail("prefill: sequence %d outside the batch of %d, or negative length", seq, B);
     }
     if (n_tokens == 0) return;
     if (B == 1) {                                   // nothing to batch over: the decode path, token by token
@@ -563,8 +553,7 @@ void prefill(InferenceState* state, int seq, const int* token_ids, int n_tokens)
     const int head_dim = c.n_embd / c.n_head;
     const int p0 = state->positions[seq];
     if (p0 + n_tokens > kv.max_seq) {
-        fprintf(stderr, "ERROR: position %d exceeds the KV cache (%d)\n", p0 + n_tokens - 1, kv.max_seq);
-        exit(1);
+        engine_fail("position %d exceeds the KV cache (%d)", p0 + n_tokens - 1, kv.max_seq);
     }
     // the rows of a chunk share this sequence's region
     kv.k += (size_t)seq * kv.kv_stride;
@@ -601,8 +590,7 @@ void prefill(InferenceState* state, int seq, const int* token_ids, int n_tokens)
 void prefill_rows(InferenceState* state, const int* token_ids, int n_tokens, int rows)
 {
     if (state->batch_size != 1) {
-        fprintf(stderr, "ERROR: prefill_rows is for states of batch size 1 (got %d): use prefill\n", state->batch_size);
-        exit(1);
+        engine_fail("prefill_rows is for states of batch size 1 (got %d): use prefill", state->batch_size);
     }
     if (rows <= 1 || n_tokens <= 1) {
         prefill(state, 0, token_ids, n_tokens);
@@ -622,8 +610,7 @@ void prefill_rows(InferenceState* state, const int* token_ids, int n_tokens, int
     kv.kv_stride = 0;
     const int p0 = state->positions[0];
     if (p0 + n_tokens > kv.max_seq) {
-        fprintf(stderr, "ERROR: position %d exceeds the KV cache (%d)\n", p0 + n_tokens - 1, kv.max_seq);
-        exit(1);
+        engine_fail("position %d exceeds the KV cache (%d)", p0 + n_tokens - 1, kv.max_seq);
     }
     check_gpu(hipEventRecord(state->sync_event, state->stream), "hipEventRecord");
     check_gpu(hipStreamWaitEvent(h->stream, state->sync_event, 0), "hipStreamWaitEvent");
@@ -762,9 +749,8 @@ void shift_context(InferenceState* state, int seq, int current_pos, int discard)
     const ModelConfig& c = state->model->config;
     const int hd = c.n_embd / c.n_head, nkv = c.n_head_kv, kv_dim = nkv * hd;
     if (seq < 0 || seq >= state->batch_size || discard < 0 || discard > current_pos || current_pos > kv.max_seq) {
-        fprintf(stderr, "ERROR: shift_context(seq %d, current_pos %d, discard %d) outside the cache (%d sequences, %d positions)\n",
+        engine_fail("shift_context(seq %d, current_pos %d, discard %d) outside the cache (%d sequences, %d positions)",
                 seq, current_pos, discard, state->batch_size, kv.max_seq);
-        exit(1);
     }
     const int keep = current_pos - discard;
     if (discard == 0 || keep == 0) return;
@@ -806,8 +792,7 @@ std::vector<int> chat_turn(InferenceState* state, int* current_pos, const std::v
 {
     if (discarded) *discarded = 0;
     if (state->batch_size != 1) {
-        fprintf(stderr, "ERROR: chat_turn needs a state of batch size 1 (got %d)\n", state->batch_size);
-        exit(1);
+        engine_fail("chat_turn needs a state of batch size 1 (got %d)", state->batch_size);
     }
     std::vector<int> tokens = turn_tokens;
     int pos = *current_pos;

@@ -5,6 +5,7 @@
 #include "turbo/model.h"
 
 #include <algorithm>
+#include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -15,6 +16,17 @@
 
 extern "C" int t12_synth_normal_bf16(void*, size_t, uint64_t, float, float, float, void*);
 extern "C" int t12_fill_f32(void*, size_t, float, void*);
+
+void engine_fail(const char* fmt, ...)
+{
+    char text[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(text, sizeof text, fmt, ap);
+    va_end(ap);
+    fprintf(stderr, "ERROR: %s\n", text);
+    throw EngineError(text);
+}
 
 namespace {
 
@@ -40,15 +52,15 @@ bool gpu_ok(hipError_t e, const char* what)
     return false;
 }
 
-// Device copy of a host array; an allocation failure ends the process like the
-// reference's GPU_CHECK (gpu_compat.h:94-101).
+// Device copy of a host array; an allocation failure throws EngineError where the
+// reference's GPU_CHECK (gpu_compat.h:94-101) ends the process.
 template <typename T>
 T* upload(const void* host, size_t count)
 {
     if (count == 0) return nullptr;
     T* d = nullptr;
-    if (!gpu_ok(hipMalloc((void**)&d, count * sizeof(T)), "hipMalloc")) exit(1);
-    if (!gpu_ok(hipMemcpy(d, host, count * sizeof(T), hipMemcpyHostToDevice), "hipMemcpy")) exit(1);
+    if (!gpu_ok(hipMalloc((void**)&d, count * sizeof(T)), "hipMalloc")) engine_fail("cannot allocate %zu bytes of device memory", count * sizeof(T));
+    if (!gpu_ok(hipMemcpy(d, host, count * sizeof(T), hipMemcpyHostToDevice), "hipMemcpy")) engine_fail("copy of %zu bytes to the device failed", count * sizeof(T));
     return d;
 }
 
@@ -56,7 +68,8 @@ template <typename T>
 T* device_alloc(size_t count)
 {
     T* d = nullptr;
-    if (!gpu_ok(hipMalloc((void**)&d, std::max<size_t>(count, 1) * sizeof(T)), "hipMalloc")) exit(1);
+    if (!gpu_ok(hipMalloc((void**)&d, std::max<size_t>(count, 1) * sizeof(T)), "hipMalloc"))
+        engine_fail("cannot allocate %zu bytes of device memory", std::max<size_t>(count, 1) * sizeof(T));
     return d;
 }
 

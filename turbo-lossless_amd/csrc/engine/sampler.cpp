@@ -1,6 +1,7 @@
 // Greedy sampler (engine/sampler.cpp:11-32): device argmax, one D2H copy and
 // one stream synchronisation per step.
 #include "turbo/sampler.h"
+#include "turbo/model.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -16,8 +17,7 @@ void init_sampler(int max_batch)
     if (max_batch <= s_d_result_size) return;
     if (s_d_result) (void)hipFree(s_d_result);
     if (hipMalloc((void**)&s_d_result, (size_t)max_batch * sizeof(int)) != hipSuccess) {
-        fprintf(stderr, "GPU error: sampler buffer allocation failed\n");
-        exit(1);
+        engine_fail("GPU error: sampler buffer allocation failed");
     }
     s_d_result_size = max_batch;
 }
