@@ -354,9 +354,11 @@ def run_moe(args, t12, torch, dev):
     X = torch.randn((T, n), generator=g, device=dev).to(torch.bfloat16).view(torch.int16)
     ids, w = moe.route_top_k(torch.randn((T, E), generator=g, device=dev), 2)
     cur = torch.cuda.current_stream()
+    layer = moe.MoeLayer(experts)
+    out = torch.empty((T, n), dtype=torch.float32, device=dev)
 
     def step():
-        moe.moe_ffn(experts, X, ids, w, stream=cur.cuda_stream)
+        layer(X, ids, w, out=out, stream=cur.cuda_stream)
     for _ in range(args.warmup):
         step()
     ms_step, ms = timed(torch, cur, step, args.steps)

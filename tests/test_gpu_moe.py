@@ -103,3 +103,73 @@ def test_moe_mixtral_shape_b256(t12, synth, moe):
         del dec
     err = float((got - ref).abs().max() / ref.abs().max())
     assert err < 1e-2, err
+
+
+@pytest.mark.parametrize("batches", [[40, 0, 64, 7, 1, 33], [130, 64, 65, 3], [300, 20], [16, 9, 2, 5]])
+@pytest.mark.parametrize("M,K", [(384, 1024), (1000, 4096), (128, 14336), (100, 192)])
+def test_grouped_gemm_vs_oracle(t12, oracle, synth, moe, M, K, batches):
+    """t12_gemm_grouped: every group its own tensor (own base_exp), activations and batch in one launch -- batch
+    tiles of 64 / 128 / 256 rows by the largest group, empty groups, K splits (few row tiles) with the per-group
+    workspace layout, K = 192 (three stages: an odd window), M not a multiple of the row tile."""
+    rng = np.random.default_rng(M + K + len(batches))
+    packs, Xs, items, outs = [], [], [], []
+    for i, B in enumerate(batches):
+        p = oracle.pack(synth.weights_llm(M, K, seed=300 + i, sigma=float(rng.choice([0.002, 0.02, 0.3])), p_outlier=1e-3))
+        X = synth.activations(max(B, 1), K, seed=400 + i)[:B]
+        out = torch.full((B, M), float("nan"), device=dev())
+        packs.append(p); Xs.append(X); outs.append(out)
+        xd = to_dev_bits(X).reshape(B, K) if B else torch.empty((0, K), dtype=torch.int16, device=dev())
+        items.append((t12.DeviceTensor12.from_packed(p, dev()), xd, out))
+    moe.gemm_grouped(items, K)
+    torch.cuda.synchronize()
+    for p, X, out in zip(packs, Xs, outs):
+        if X.shape[0]:
+            assert rel_err(out.cpu().numpy(), oracle.gemm(p, X)) < 1e-4
+
+
+def test_grouped_gemm_general_path_and_errors(t12, oracle, synth, moe):
+    """K not a multiple of 64 and a tensor of subnormals (base_exp -1): the groups run one by one through t12_gemm's
+    general kernel; more than 16 groups and a short activation stride are refused."""
+    K = 100
+    ps = [oracle.pack(synth.weights_llm(50, K, seed=1)), oracle.pack(np.full((20, K), 0x0001, np.uint16))]
+    Xs = [synth.activations(5, K, seed=2), synth.activations(70, K, seed=3)]
+    outs = [torch.full((X.shape[0], p.M), float("nan"), device=dev()) for p, X in zip(ps, Xs)]
+    items = [(t12.DeviceTensor12.from_packed(p, dev()), to_dev_bits(X).reshape(-1, K), o) for p, X, o in zip(ps, Xs, outs)]
+    moe.gemm_grouped(items, K)
+    torch.cuda.synchronize()
+    for p, X, o in zip(ps, Xs, outs):
+        ref = oracle.gemm(p, X)
+        assert np.abs(o.cpu().numpy() - ref).max() <= 1e-4 * max(np.abs(ref).max(), 1e-30)
+    with pytest.raises(t12.T12Error, match="groups"):
+        moe.gemm_grouped([items[0]] * 17, K)
+    with pytest.raises(t12.T12Error, match="act_stride"):
+        moe.gemm_grouped([items[0]], K + 8)
+
+
+def test_moe_route_tables_and_refusals(t12, oracle, synth, moe):
+    """Ragged routing incl. an expert nobody chose, int32 ids, a strided activation matrix, k = 3: against the
+    oracle's per-expert products; an id outside the experts is refused."""
+    E, n, n_ff, T, k = 5, 256, 512, 77, 3
+    packs = [[oracle.pack(synth.weights_llm(m, kk, seed=900 + 3 * e + j, p_outlier=1e-3))
+              for j, (m, kk) in enumerate([(n_ff, n), (n_ff, n), (n, n_ff)])] for e in range(E)]
+    layer = moe.MoeLayer([moe.Expert(*[t12.DeviceTensor12.from_packed(p, dev()) for p in ps]) for ps in packs])
+    X = synth.activations(T, n, seed=79)
+    rng = np.random.default_rng(8)
+    ids_h = np.stack([rng.choice([0, 1, 2, 4], size=k, replace=False) for _ in range(T)]).astype(np.int32)   # expert 3 unused
+    w_h = rng.random((T, k)).astype(np.float32)
+    Xd = torch.zeros((T, n + 24), dtype=torch.int16, device=dev())
+    Xd[:, :n] = to_dev_bits(X).reshape(T, n)
+    for _ in range(2):                                      # the second call reuses the workspace
+        got = layer(Xd[:, :n], torch.from_numpy(ids_h).to(dev()), torch.from_numpy(w_h).to(dev())).cpu().numpy()
+    ref = np.zeros((T, n), np.float64)
+    for e in range(E):
+        rows, slots = np.nonzero(ids_h == e)
+        if len(rows) == 0:
+            continue
+        a = oracle.silu_mul_bf16(oracle.gemm(packs[e][0], X[rows]), oracle.gemm(packs[e][1], X[rows]))
+        ref[rows] += w_h[rows, slots][:, None].astype(np.float64) * oracle.gemm(packs[e][2], a)
+    assert rel_err(got, ref) < 1e-4
+    bad = ids_h.copy()
+    bad[5, 1] = E
+    with pytest.raises(t12.T12Error, match="outside"):
+        layer(Xd[:, :n], torch.from_numpy(bad).to(dev()), torch.from_numpy(w_h).to(dev()))

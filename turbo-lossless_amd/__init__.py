@@ -35,6 +35,16 @@ class PatchBatchDesc(C.Structure):
                 ("patch_wrong", C.c_void_p), ("activations", C.c_void_p), ("output", C.c_void_p), ("M", C.c_int)]
 
 
+class Group(C.Structure):
+    """Mirror of T12Group (include/t12_abi.h)."""
+    _fields_ = [("seg", Segment), ("act_bf16", C.c_void_p), ("act_stride", C.c_int), ("B", C.c_int)]
+
+
+class MoeExpert(C.Structure):
+    """Mirror of T12MoeExpert (include/t12_abi.h)."""
+    _fields_ = [("w1", Segment), ("w3", Segment), ("w2", Segment)]
+
+
 class GemmPartials(C.Structure):
     """Mirror of T12GemmPartials (include/t12_abi.h)."""
     _fields_ = [("ws", C.c_void_p), ("nsplit", C.c_int), ("ld", C.c_int), ("split_stride", C.c_size_t)]
@@ -127,6 +137,9 @@ _SIGS = {
     "nv_launch_split12_cublas_batch_async": (_i, [_vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_gemm": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_gemm_noalloc": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
+    "t12_gemm_grouped": (_i, [C.POINTER(Group), _i, _i, _vp]),
+    "t12_moe_workspace_bytes": (C.c_size_t, [_i, _i, _i, _i, _i]),
+    "t12_moe_ffn": (_i, [C.POINTER(MoeExpert), _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, C.c_size_t, _vp, _i, _vp]),
     "t12_gemm_swiglu": (_i, [C.POINTER(Segment), C.POINTER(Segment), _vp, _i, _i, _i, _vp, _i, _vp]),
     "t12_gemm_deferred": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, C.POINTER(GemmPartials), _vp]),
     "launch_sum_add_rms_norm_bf16_batch": (None, [_vp, _vp, _i, C.c_size_t, _i, _vp, _vp, _vp, _i, C.c_float, _i, _vp]),

@@ -1,0 +1,261 @@
+// Mixture-of-experts SwiGLU feed-forward layer over split-12 experts (a Mixtral-shaped layer: 8 experts, top-2):
+//
+//   out[t] = sum_j weights[t, j] * W2_e( silu(W1_e x_t) * (W3_e x_t) ),   e = expert_ids[t, j]
+//
+// The reference engine has no such layer; its decode+GEMM entry point (nv_launch_split12_fused_gemm_async,
+// nvidia_kernels.cu:444) would be called once per expert with that expert's token count as the batch.  Here the
+// layer is five launches plus one copy of the per-expert counts to the host:
+//   1. moe_route_kernel    counting sort of the (token, slot) pairs by expert: counts, slot <-> pair tables
+//   2. moe_gather_kernel   activation rows in slot order (bf16 [P, n_embd], P = T * k)
+//   3. t12_gemm_grouped    gate and up of every expert over its slots (2 E groups)   -> fp32 [P, n_ff] each
+//   4. silu_mul            bf16 [P, n_ff]
+//   5. t12_gemm_grouped    down of every expert over its slots (E groups)           -> fp32 [P, n_embd]
+//   6. moe_combine_kernel  out[t] = sum_j weights[t, j] * Y[slot(t, j)]  (j ascending: a fixed order, no atomics)
+// The host needs the counts to size the grouped launches, so step 1 is followed by a copy of E ints and a wait on
+// the stream.
+
+#include "t12_device.h"
+#include "t12_host.h"
+
+extern "C" void launch_silu_mul_bf16_batch(const float* gate, const float* up, int16_t* out, int n, int batch_size,
+                                           hipStream_t stream);
+
+namespace {
+
+constexpr int ROUTE_THREADS = 256;
+constexpr int MAX_EXPERTS = 32;       // the sort keeps a 256-entry count row per expert in LDS
+
+// One workgroup.  Thread i owns the pairs [i * chunk, (i + 1) * chunk); pairs of one expert keep their order
+// (pair index ascending), so the grouping is the same on every run.
+template <typename IdT>
+__global__ __launch_bounds__(ROUTE_THREADS) void moe_route_kernel(const IdT* __restrict__ ids, int P, int E,
+                                                                  int* __restrict__ counts, int* __restrict__ pair_of_slot,
+                                                                  int* __restrict__ slot_of_pair, int* __restrict__ bad)
+{
+    __shared__ int cnt[MAX_EXPERTS][ROUTE_THREADS + 1];
+    __shared__ int ebase[MAX_EXPERTS + 1];
+    const int tid = threadIdx.x;
+    const int chunk = (P + ROUTE_THREADS - 1) / ROUTE_THREADS;
+    const int lo = min(P, tid * chunk), hi = min(P, lo + chunk);
+    for (int e = 0; e < E; e++) cnt[e][tid] = 0;
+    if (tid == 0) *bad = 0;
+    __syncthreads();
+    for (int q = lo; q < hi; q++) {
+        const long long e = (long long)ids[q];
+        if (e >= 0 && e < E) cnt[(int)e][tid]++;
+        else *bad = 1;                                     // reported by the host; the pair gets no slot
+    }
+    __syncthreads();
+    // per expert: exclusive prefix over the threads (one wave per expert in turn; 256 values = 4 per lane)
+    const int lane = tid & 63, wave = tid >> 6;
+    for (int e = wave; e < E; e += ROUTE_THREADS / 64) {
+        int v[4], run = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[i] = cnt[e][lane * 4 + i];
+            run += v[i];
+        }
+        int incl = run;                                    // inclusive scan of the lanes' sums
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int o = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += o;
+        }
+        int base = incl - run;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            cnt[e][lane * 4 + i] = base;
+            base += v[i];
+        }
+        if (lane == 63) cnt[e][ROUTE_THREADS] = incl;      // the expert's total
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int e = 0; e < E; e++) {
+            ebase[e] = run;
+            run += cnt[e][ROUTE_THREADS];
+            counts[e] = cnt[e][ROUTE_THREADS];
+        }
+        ebase[E] = run;
+    }
+    __syncthreads();
+    for (int q = lo; q < hi; q++) {
+        const long long e = (long long)ids[q];
+        if (e >= 0 && e < E) {
+            const int slot = ebase[(int)e] + cnt[(int)e][tid]++;
+            pair_of_slot[slot] = q;
+            slot_of_pair[q] = slot;
+        } else {
+            slot_of_pair[q] = -1;
+        }
+    }
+}
+
+// Xg[slot, :] = X[pair_of_slot[slot] / k, :]; one workgroup per slot, 16 bytes per thread and step.
+__global__ __launch_bounds__(256) void moe_gather_kernel(const uint16_t* __restrict__ x, int x_stride, const int* __restrict__ pair_of_slot,
+                                                         int k, int n, uint16_t* __restrict__ xg)
+{
+    const int slot = blockIdx.x;
+    const int t = pair_of_slot[slot] / k;
+    const uint16_t* src = x + (size_t)t * x_stride;
+    uint16_t* dst = xg + (size_t)slot * n;
+    if ((n & 7) == 0 && (x_stride & 7) == 0 && ((uintptr_t)x & 15) == 0) {
+        for (int c = threadIdx.x * 8; c < n; c += 256 * 8) *(uint4*)(dst + c) = *(const uint4*)(src + c);
+    } else {
+        for (int c = threadIdx.x; c < n; c += 256) dst[c] = src[c];
+    }
+}
+
+// out[t, c] = sum_j w[t, j] * Y[slot_of_pair[t * k + j], c]
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ slot_of_pair,
+                                                          const float* __restrict__ w, int k, int n, float* __restrict__ out,
+                                                          int out_stride)
+{
+    const int t = blockIdx.x;
+    for (int c = threadIdx.x; c < n; c += 256) {
+        float v = 0.0f;
+        for (int j = 0; j < k; j++) {
+            const int slot = slot_of_pair[t * k + j];
+            if (slot >= 0) v += w[t * k + j] * y[(size_t)slot * n + c];
+        }
+        out[(size_t)t * out_stride + c] = v;
+    }
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct MoeLayout {
+    size_t counts, pair_of_slot, slot_of_pair, bad, xg, gate, up, act, y, total;
+};
+
+MoeLayout moe_layout(int T, int k, int n_embd, int n_ff, int E)
+{
+    const size_t P = (size_t)T * k;
+    MoeLayout l;
+    size_t o = 0;
+    l.counts = o;        o = align256(o + sizeof(int) * (size_t)E);
+    l.bad = o;           o = align256(o + sizeof(int));
+    l.pair_of_slot = o;  o = align256(o + sizeof(int) * P);
+    l.slot_of_pair = o;  o = align256(o + sizeof(int) * P);
+    l.xg = o;            o = align256(o + 2 * P * n_embd);
+    l.gate = o;          o = align256(o + 4 * P * n_ff);
+    l.up = o;            o = align256(o + 4 * P * n_ff);
+    l.act = o;           o = align256(o + 2 * P * n_ff);
+    l.y = o;             o = align256(o + 4 * P * n_embd);
+    l.total = o;
+    return l;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t t12_moe_workspace_bytes(int T, int k, int n_embd, int n_ff, int E)
+{
+    if (T < 1 || k < 1 || n_embd < 1 || n_ff < 1 || E < 1) return 0;
+    return moe_layout(T, k, n_embd, n_ff, E).total;
+}
+
+int t12_moe_ffn(const T12MoeExpert* experts, int E, const void* x_bf16, int x_stride, const void* expert_ids,
+                int id_bytes, const float* weights, int T, int k, int n_embd, int n_ff, void* workspace,
+                size_t workspace_bytes, float* out, int out_stride, void* stream)
+{
+    T12_REQUIRE(experts && x_bf16 && expert_ids && weights && workspace && out, "t12_moe_ffn: null operand");
+    T12_REQUIRE(E >= 1 && E <= MAX_EXPERTS, "t12_moe_ffn: 1..%d experts (got %d)", MAX_EXPERTS, E);
+    T12_REQUIRE(T >= 1 && k >= 1 && k <= E && n_embd >= 1 && n_ff >= 1, "t12_moe_ffn: T %d, k %d, n_embd %d or n_ff %d invalid",
+                T, k, n_embd, n_ff);
+    T12_REQUIRE((long long)T * k < (1ll << 24), "t12_moe_ffn: %lld (token, expert) pairs, at most 2^24", (long long)T * k);
+    T12_REQUIRE(id_bytes == 4 || id_bytes == 8, "t12_moe_ffn: expert ids are int32 or int64 (id_bytes %d)", id_bytes);
+    T12_REQUIRE(x_stride >= n_embd && out_stride >= n_embd, "t12_moe_ffn: x_stride %d or out_stride %d < n_embd %d", x_stride,
+                out_stride, n_embd);
+    T12_REQUIRE((uintptr_t)workspace % 256 == 0, "t12_moe_ffn: workspace must be 256-byte aligned");
+    const MoeLayout l = moe_layout(T, k, n_embd, n_ff, E);
+    T12_REQUIRE(workspace_bytes >= l.total, "t12_moe_ffn: workspace of %zu bytes, t12_moe_workspace_bytes says %zu",
+                workspace_bytes, l.total);
+    for (int e = 0; e < E; e++) {
+        const T12MoeExpert& x = experts[e];
+        T12_REQUIRE(x.w1.M == n_ff && x.w3.M == n_ff && x.w2.M == n_embd, "t12_moe_ffn: expert %d: w1/w3 need %d rows, w2 %d", e,
+                    n_ff, n_embd);
+    }
+    hipStream_t st = (hipStream_t)stream;
+    uint8_t* ws = (uint8_t*)workspace;
+    int* counts = (int*)(ws + l.counts);
+    int* bad = (int*)(ws + l.bad);
+    int* pair_of_slot = (int*)(ws + l.pair_of_slot);
+    int* slot_of_pair = (int*)(ws + l.slot_of_pair);
+    uint16_t* xg = (uint16_t*)(ws + l.xg);
+    float* gate = (float*)(ws + l.gate);
+    float* up = (float*)(ws + l.up);
+    int16_t* act = (int16_t*)(ws + l.act);
+    float* y = (float*)(ws + l.y);
+    const int P = T * k;
+
+    if (id_bytes == 4)
+        hipLaunchKernelGGL(moe_route_kernel<int32_t>, dim3(1), dim3(ROUTE_THREADS), 0, st, (const int32_t*)expert_ids, P, E,
+                           counts, pair_of_slot, slot_of_pair, bad);
+    else
+        hipLaunchKernelGGL(moe_route_kernel<long long>, dim3(1), dim3(ROUTE_THREADS), 0, st, (const long long*)expert_ids, P, E,
+                           counts, pair_of_slot, slot_of_pair, bad);
+    T12_CHECK_LAUNCH("t12_moe_ffn(route)");
+    int host[MAX_EXPERTS + 1];
+    // counts and the flag behind them are 256 bytes apart: two small copies, then one wait
+    if (hipMemcpyAsync(host, counts, sizeof(int) * E, hipMemcpyDeviceToHost, st) != hipSuccess ||
+        hipMemcpyAsync(host + MAX_EXPERTS, bad, sizeof(int), hipMemcpyDeviceToHost, st) != hipSuccess ||
+        hipStreamSynchronize(st) != hipSuccess) {
+        t12_set_error("t12_moe_ffn: reading the per-expert counts failed: %s", hipGetErrorString(hipGetLastError()));
+        return T12_ELAUNCH;
+    }
+    T12_REQUIRE(host[MAX_EXPERTS] == 0, "t12_moe_ffn: an expert id lies outside 0..%d", E - 1);
+
+    int placed = 0;
+    for (int e = 0; e < E; e++) placed += host[e];
+    hipLaunchKernelGGL(moe_gather_kernel, dim3(placed), dim3(256), 0, st, (const uint16_t*)x_bf16, x_stride, pair_of_slot, k,
+                       n_embd, xg);
+    T12_CHECK_LAUNCH("t12_moe_ffn(gather)");
+
+    // gate and up of eight experts per launch (16 groups), then down of sixteen
+    for (int e0 = 0; e0 < E; e0 += 8) {
+        T12Group g[16];
+        int n = 0, slot0 = 0;
+        for (int e = 0; e < e0; e++) slot0 += host[e];
+        for (int e = e0; e < E && e < e0 + 8; e++) {
+            for (int j = 0; j < 2; j++) {
+                T12Group& q = g[n++];
+                q.seg = j == 0 ? experts[e].w1 : experts[e].w3;
+                q.seg.out = (j == 0 ? gate : up) + (size_t)slot0 * n_ff;
+                q.seg.out_stride = n_ff;
+                q.act_bf16 = xg + (size_t)slot0 * n_embd;
+                q.act_stride = n_embd;
+                q.B = host[e];
+            }
+            slot0 += host[e];
+        }
+        const int rc = t12_gemm_grouped(g, n, n_embd, stream);
+        if (rc) return rc;
+    }
+    launch_silu_mul_bf16_batch(gate, up, act, n_ff, placed, st);
+    T12_CHECK_LAUNCH("t12_moe_ffn(silu_mul)");
+    for (int e0 = 0; e0 < E; e0 += 16) {
+        T12Group g[16];
+        int n = 0, slot0 = 0;
+        for (int e = 0; e < e0; e++) slot0 += host[e];
+        for (int e = e0; e < E && e < e0 + 16; e++) {
+            T12Group& q = g[n++];
+            q.seg = experts[e].w2;
+            q.seg.out = y + (size_t)slot0 * n_embd;
+            q.seg.out_stride = n_embd;
+            q.act_bf16 = act + (size_t)slot0 * n_ff;
+            q.act_stride = n_ff;
+            q.B = host[e];
+            slot0 += host[e];
+        }
+        const int rc = t12_gemm_grouped(g, n, n_ff, stream);
+        if (rc) return rc;
+    }
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, st, y, slot_of_pair, weights, k, n_embd, out, out_stride);
+    T12_CHECK_LAUNCH("t12_moe_ffn(combine)");
+    return T12_OK;
+}
+
+}  // extern "C"

@@ -1,12 +1,13 @@
-"""Mixture-of-experts SwiGLU FFN over split-12 experts: tokens grouped per expert, each group
-through the fused decode+GEMM (w1|w3 as one two-segment launch, then w2).
+"""Mixture-of-experts SwiGLU FFN over split-12 experts (a Mixtral-shaped layer).
 
-The reference engine has no MoE layer; this is the host-side grouping that its decode+GEMM
-entry point (`nv_launch_split12_fused_gemm_async`, nvidia_kernels.cu:444) would be driven with
-for a Mixtral-shaped layer: one call per expert with that expert's variable token count as B.
-torch is used for the routing bookkeeping only (top-k, sort, gather, weighted scatter-add).
+The reference engine has no MoE layer; its decode+GEMM entry point (`nv_launch_split12_fused_gemm_async`,
+nvidia_kernels.cu:444) would be called once per expert and projection with that expert's token count as B.  Here
+the layer is the library's `t12_moe_ffn`: the (token, slot) pairs are grouped per expert on the GPU, gate|up and
+down of all experts run as grouped decode+GEMM launches, and the weighted sum is taken in a fixed order.  torch
+holds the buffers; `route_top_k` (top-k and softmax of the router logits) is the only torch arithmetic, and it is
+not part of `moe_ffn`.
 """
-from . import DeviceTensor12, gemm, lib, check, _seg_array, _torch
+from . import DeviceTensor12, Group, MoeExpert, lib, check, current_stream, _torch
 
 
 class Expert:
@@ -24,71 +25,59 @@ def route_top_k(router_logits, k=2):
     return idx, torch.softmax(top, dim=-1)
 
 
-_side_streams = {}
+class MoeLayer:
+    """The experts of one layer as the table t12_moe_ffn takes, with a workspace that grows to the largest call."""
+
+    def __init__(self, experts):
+        self.experts = list(experts)
+        self.n_ff, self.n_embd = self.experts[0].w1.M, self.experts[0].w1.K
+        self.table = (MoeExpert * len(self.experts))()
+        for i, e in enumerate(self.experts):
+            assert (e.w1.M, e.w1.K) == (self.n_ff, self.n_embd)
+            self.table[i].w1, self.table[i].w3, self.table[i].w2 = e.w1.segment(None), e.w3.segment(None), e.w2.segment(None)
+        self.ws = None
+
+    def workspace(self, T, k, device):
+        need = lib.t12_moe_workspace_bytes(T, k, self.n_embd, self.n_ff, len(self.experts))
+        if self.ws is None or self.ws.numel() < need or self.ws.device != device:
+            self.ws = _torch().empty(need, dtype=_torch().uint8, device=device)
+        return self.ws
+
+    def __call__(self, X, expert_ids, weights, out=None, stream=None):
+        """X bf16 bits [T, n_embd] (int16 tensor, rows may be strided); expert_ids [T, k] int32 / int64 and weights
+        [T, k] fp32, contiguous; returns fp32 [T, n_embd] = sum_j w[t,j] * FFN_{e[t,j]}(x_t).  Waits for the stream
+        once (the host sizes the grouped launches by the per-expert counts)."""
+        torch = _torch()
+        T, n = X.shape
+        k = expert_ids.shape[1]
+        assert n == self.n_embd and X.stride(1) == 1 and expert_ids.is_contiguous() and weights.is_contiguous()
+        assert weights.dtype == torch.float32 and expert_ids.dtype in (torch.int32, torch.int64)
+        if out is None:
+            out = torch.empty((T, n), dtype=torch.float32, device=X.device)
+        ws = self.workspace(T, k, X.device)
+        st = current_stream() if stream is None else stream
+        check(lib.t12_moe_ffn(self.table, len(self.experts), X.data_ptr(), X.stride(0), expert_ids.data_ptr(),
+                              expert_ids.element_size(), weights.data_ptr(), T, k, n, self.n_ff, ws.data_ptr(), ws.numel(),
+                              out.data_ptr(), out.stride(0), st), "t12_moe_ffn")
+        return out
 
 
-def _streams_for(device, n):
-    """n side streams of the device (default priority), created once."""
-    torch = _torch()
-    key = (device.index if device.index is not None else torch.cuda.current_device(), n)
-    if key not in _side_streams:
-        _side_streams[key] = [torch.cuda.Stream(device=device) for _ in range(n)]
-    return _side_streams[key]
+def moe_ffn(experts, X, expert_ids, weights, stream=None):
+    """One call of a layer built on the spot (keep a MoeLayer to reuse the table and the workspace).  The workspace
+    is a torch tensor released on return, so the work must be on torch's current stream."""
+    if stream is not None and stream != current_stream():
+        raise ValueError("moe_ffn works on torch's current stream: make the stream current, or keep a MoeLayer")
+    return MoeLayer(experts)(X, expert_ids, weights, stream=stream)
 
 
-def moe_ffn(experts, X, expert_ids, weights, stream=None, concurrency=2):
-    """X bf16 bits [T, n_embd] (int16 tensor); returns fp32 [T, n_embd] = sum_j w[t,j] * FFN_{e[t,j]}(x_t).
-
-    The experts' launch chains (w1|w3, SiLU*mul, w2) are independent of each other: with concurrency > 1 they are
-    issued round-robin on that many side streams, so that one expert's weight stream starts under the tail of
-    another's; the weighted scatter-add of all (token, expert) pairs follows as one operation on the caller's
-    stream.  `stream`, when given, must be torch's current stream: the routing bookkeeping is torch operations."""
-    torch = _torch()
-    T, n = X.shape
-    k = expert_ids.shape[1]
-    n_ff = experts[0].w1.M
-    flat_e = expert_ids.reshape(-1)
-    order = torch.argsort(flat_e, stable=True)                     # (token, slot) pairs grouped per expert
-    counts = torch.bincount(flat_e, minlength=len(experts)).tolist()
-    tok = torch.div(order, k, rounding_mode="floor")
-    Xg = X[tok].contiguous()                                       # [T*k, n] gathered rows
-    wg = weights.reshape(-1)[order]
-    main = torch.cuda.current_stream(X.device)
-    if stream is not None and stream != main.cuda_stream:
-        raise ValueError("moe_ffn works on torch's current stream: make the stream current instead of passing its handle")
-    lanes = max(1, min(int(concurrency), sum(c > 0 for c in counts)))
-    side = _streams_for(X.device, lanes) if lanes > 1 else [None]
-    cap = max(counts)
-    gate = [torch.empty((cap, n_ff), dtype=torch.float32, device=X.device) for _ in side]
-    up = [torch.empty_like(g) for g in gate]
-    act = [torch.empty((cap, n_ff), dtype=torch.int16, device=X.device) for _ in side]
-    Y = torch.empty((T * k, n), dtype=torch.float32, device=X.device)      # every pair's FFN output, grouped like Xg
-    if lanes > 1:
-        ready = torch.cuda.Event()
-        ready.record(main)
-        for s in side:
-            s.wait_event(ready)
-    pos, turn = 0, 0
-    for e, cnt in enumerate(counts):
-        if cnt == 0:
-            continue
-        ex = experts[e]
-        lane = turn % lanes
-        turn += 1
-        st = side[lane].cuda_stream if lanes > 1 else main.cuda_stream
-        xs = Xg[pos:pos + cnt]
-        # SiLU*mul in the GEMM's epilogue where the group is large enough to have such a kernel
-        rc = lib.t12_gemm_swiglu(_seg_array([ex.w1.segment(None)]), _seg_array([ex.w3.segment(None)]), xs.data_ptr(),
-                                 xs.stride(0), n, cnt, act[lane].data_ptr(), n_ff, st)
-        check(min(rc, 0), "t12_gemm_swiglu")
-        if rc == 1:
-            gemm([ex.w1, ex.w3], xs, outs=[gate[lane][:cnt], up[lane][:cnt]], stream=st)
-            lib.launch_silu_mul_bf16_batch(gate[lane].data_ptr(), up[lane].data_ptr(), act[lane].data_ptr(), n_ff, cnt, st)
-        gemm([ex.w2], act[lane][:cnt], outs=[Y[pos:pos + cnt]], stream=st)
-        pos += cnt
-    if lanes > 1:
-        for s in side:
-            main.wait_stream(s)
-    out = torch.zeros((T, n), dtype=torch.float32, device=X.device)
-    out.index_add_(0, tok, Y * wg[:, None])                        # two addends per token: the order cannot matter
-    return out
+def gemm_grouped(items, K, stream=None):
+    """items: (DeviceTensor12, X int16 [B, K] rows strided, out fp32 [B, M]) per group -> one t12_gemm_grouped launch."""
+    g = (Group * len(items))()
+    for i, (w, X, out) in enumerate(items):
+        g[i].seg = w.segment(out)
+        g[i].seg.out_stride = out.stride(0) if out.shape[0] > 1 else w.M
+        g[i].act_bf16 = X.data_ptr()
+        g[i].act_stride = X.stride(0) if X.shape[0] > 0 else K
+        g[i].B = X.shape[0]
+    st = current_stream() if stream is None else stream
+    check(lib.t12_gemm_grouped(g, len(items), K, st), "t12_gemm_grouped")
