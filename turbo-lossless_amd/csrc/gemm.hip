@@ -531,6 +531,40 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmParams p)
     sg.out[(size_t)b * sg.out_stride + m] = v;
 }
 
+// The same sums four rows at a time (16-byte loads and stores): thread = rows 4 c .. 4 c + 3 of one batch row.
+// Used when every segment's row count, first row, output stride and pointers are multiples of four floats.
+__global__ __launch_bounds__(256) void gemm_reduce4_kernel(const GemmParams p)
+{
+    const int col = (blockIdx.x * 256 + threadIdx.x) * 4;
+    const int b = blockIdx.y;
+    if (col >= p.m_total) return;
+    int s = 0;
+#pragma unroll
+    for (int i = 1; i < GMAX; i++)
+        if (i < p.nseg && col >= p.seg_row0[i]) s = i;
+    if (b >= p.seg_B[s]) return;
+    const int m = col - p.seg_row0[s];
+    const float* src = p.ws + p.seg_ws0[s] + (size_t)b * p.seg_ld[s] + m;
+    t12_f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int z = 0; z < p.ksplit; z++) v += *(const t12_f32x4*)(src + (size_t)z * p.split_stride);
+    const T12Segment& sg = p.seg[s];
+    *(t12_f32x4*)(sg.out + (size_t)b * sg.out_stride + m) = v;
+}
+
+// Adds up the partial sums of a K-split launch described by p into the segments' outputs.
+void launch_reduce(const GemmParams& p, int max_b, hipStream_t st)
+{
+    bool vec = p.split_stride % 4 == 0 && (uintptr_t)p.ws % 16 == 0;
+    for (int i = 0; i < p.nseg; i++) {
+        const T12Segment& g = p.seg[i];
+        if (g.M % 4 || p.seg_row0[i] % 4 || p.seg_ws0[i] % 4 || p.seg_ld[i] % 4 || g.out_stride % 4 || (uintptr_t)g.out % 16) vec = false;
+    }
+    if (vec)
+        hipLaunchKernelGGL(gemm_reduce4_kernel, dim3((p.m_total / 4 + 255) / 256, max_b), dim3(256), 0, st, p);
+    else
+        hipLaunchKernelGGL(gemm_reduce_kernel, dim3((p.m_total + 255) / 256, max_b), dim3(256), 0, st, p);
+}
+
 // ---------------------------------------------------------------------------
 // General path: any K, any base_exp, any alignment.  One wave per (row, 8
 // batch rows); scalar decode rule; escapes exact from the CSR list.
@@ -1009,7 +1043,7 @@ int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_st
         part->ld = m_total;
         part->split_stride = (size_t)B * m_total;
     } else if (ks > 1) {
-        hipLaunchKernelGGL(gemm_reduce_kernel, dim3((m_total + 255) / 256, B), dim3(256), 0, st, p);
+        launch_reduce(p, B, st);
         T12_CHECK_LAUNCH("t12_gemm(reduce)");
     }
     return T12_OK;
@@ -1127,7 +1161,7 @@ int t12_gemm_grouped(const T12Group* groups, int ngroups, int K, void* stream)
     else rc = launch_mfma<4, 2, 2, 2>(p, tiles, st);
     if (rc) return rc;
     if (ks > 1) {
-        hipLaunchKernelGGL(gemm_reduce_kernel, dim3((m_total + 255) / 256, max_b), dim3(256), 0, st, p);
+        launch_reduce(p, max_b, st);
         T12_CHECK_LAUNCH("t12_gemm_grouped(reduce)");
     }
     return T12_OK;
