@@ -181,6 +181,12 @@ int t12_moe_ffn(const T12MoeExpert* experts, int E, const void* x_bf16, int x_st
 int t12_gemm_noalloc(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride,
                      int out_stride, int K, int B, void* stream);
 
+/* The library keeps device buffers per (device, stream): K-split partial sums of t12_gemm / _deferred / _grouped, argmax
+ * partials and context-split buffers of the glue launchers.  t12_release_stream waits for the stream and frees those of
+ * (current device, stream); call it before destroying a stream (free_inference_state does).  No counterpart in the
+ * reference, which keeps no such buffers. */
+int t12_release_stream(void* stream);
+
 /* ---- (c) standalone decompress --------------------------------------------
  * out_bf16[m*K + k] = decoded weight bits.  patched != 0: escapes take
  * `correct` (lossless, bit-exact with the tensor that was packed).

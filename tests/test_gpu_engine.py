@@ -366,3 +366,36 @@ def test_errors_come_back_as_codes_not_as_a_dead_process(t12, small_model):
     finally:
         two.close()
         base.close()
+
+
+def test_states_give_their_stream_buffers_back(t12, small_model):
+    """A state's stream carries library buffers (K-split sums, argmax partials, context-split scratch, sampler ids);
+    free_inference_state hands them back (t12_release_stream), so states that come and go leave device memory where it
+    was.  After a release the stream works as before (new buffers on first use)."""
+    path, _ = small_model
+    base = t12.Engine.load(path, batch=1)
+    try:
+        def cycle():
+            for B in (1, 8, 64):
+                e = base.new_state(B)
+                e.set_positions([0] * B)
+                e.forward([5] * B)
+                e.decode_all(3)
+                e.sample()
+                e.close()
+        cycle()
+        torch.cuda.synchronize()
+        free0 = torch.cuda.mem_get_info()[0]
+        for _ in range(6):
+            cycle()
+        torch.cuda.synchronize()
+        assert free0 - torch.cuda.mem_get_info()[0] < (4 << 20)
+        base.set_positions([0])
+        base.forward([9])
+        want = base.decode(4)
+        t12.check(t12.lib.t12_release_stream(t12.lib.t12_engine_stream(base.state)), "release")
+        base.set_positions([0])
+        base.forward([9])
+        assert base.decode(4) == want
+    finally:
+        base.close()

@@ -138,6 +138,7 @@ _SIGS = {
     "t12_gemm": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_gemm_noalloc": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, _vp]),
     "t12_gemm_grouped": (_i, [C.POINTER(Group), _i, _i, _vp]),
+    "t12_release_stream": (_i, [_vp]),
     "t12_moe_workspace_bytes": (C.c_size_t, [_i, _i, _i, _i, _i]),
     "t12_moe_ffn": (_i, [C.POINTER(MoeExpert), _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, C.c_size_t, _vp, _i, _vp]),
     "t12_gemm_swiglu": (_i, [C.POINTER(Segment), C.POINTER(Segment), _vp, _i, _i, _i, _vp, _i, _vp]),

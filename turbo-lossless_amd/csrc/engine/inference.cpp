@@ -254,8 +254,14 @@ void free_inference_state(InferenceState* state)
                     (void*)state->d_positions, (void*)state->d_tokens, (void*)state->bf16_act,
                     (void*)state->bf16_act2, state->patch_descs_gpu})
         if (p) (void)hipFree(p);
-    if (state->stream) (void)hipStreamDestroy(state->stream);
-    if (state->stream2) (void)hipStreamDestroy(state->stream2);
+    if (state->stream) {
+        (void)t12_release_stream(state->stream);          // the library's per-stream buffers go with the stream
+        (void)hipStreamDestroy(state->stream);
+    }
+    if (state->stream2) {
+        (void)t12_release_stream(state->stream2);
+        (void)hipStreamDestroy(state->stream2);
+    }
     if (state->sync_event) (void)hipEventDestroy(state->sync_event);
     Impl* impl = (Impl*)state->impl;
     if (impl) {

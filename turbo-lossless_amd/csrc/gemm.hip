@@ -42,6 +42,9 @@
 #include "t12_device.h"
 #include "t12_host.h"
 
+extern "C" void t12_glue_release_stream(hipStream_t st);      // glue.hip
+extern "C" void t12_sampler_release_stream(hipStream_t st);   // engine/sampler.cpp
+
 namespace {
 
 constexpr int KC = 64;          // K columns staged per pipeline stage
@@ -797,6 +800,18 @@ float* workspace(size_t bytes, hipStream_t st)
     return w.ptr;
 }
 
+// Frees the K-split workspace of (current device, stream).
+void release_workspace(hipStream_t st)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    auto it = g_ws.find({dev, st});
+    if (it == g_ws.end()) return;
+    if (it->second.ptr) (void)hipFree(it->second.ptr);
+    g_ws.erase(it);
+}
+
 // ---- the same workspace for callers that may not allocate: a fixed array in the code object's own device
 //      memory.  Every GPU the library runs on holds its own copy at its own address; the name below is only a
 //      host-side handle for hipGetSymbolAddress, never a pointer a kernel could use.
@@ -1164,6 +1179,22 @@ int t12_gemm_grouped(const T12Group* groups, int ngroups, int K, void* stream)
         launch_reduce(p, max_b, st);
         T12_CHECK_LAUNCH("t12_gemm_grouped(reduce)");
     }
+    return T12_OK;
+}
+
+// The library keeps device buffers per (device, stream): the K-split partial sums of t12_gemm*, the argmax partials and the
+// context-split buffers of the glue kernels, the sampler's result ids.  A caller about to destroy a stream hands them back here (waits for the
+// stream first); a stream that is used again afterwards simply gets new ones.
+int t12_release_stream(void* stream)
+{
+    hipStream_t st = (hipStream_t)stream;
+    if (hipStreamSynchronize(st) != hipSuccess) {
+        t12_set_error("t12_release_stream: hipStreamSynchronize failed: %s", hipGetErrorString(hipGetLastError()));
+        return T12_ELAUNCH;
+    }
+    release_workspace(st);
+    t12_glue_release_stream(st);
+    t12_sampler_release_stream(st);
     return T12_OK;
 }
 

@@ -1376,6 +1376,23 @@ StreamScratch* attn_split_scratch(hipStream_t st)
     return &sc;
 }
 
+}  // namespace
+
+// Frees this file's scratch of (current device, stream): argmax partials, context-split buffers.  The caller has
+// made sure that nothing enqueued on the stream still uses them (t12_release_stream waits for the stream).
+extern "C" void t12_glue_release_stream(hipStream_t st)
+{
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto it = g_scratch.find({current_device(), st});
+    if (it == g_scratch.end()) return;
+    if (it->second.part) (void)hipFree(it->second.part);
+    if (it->second.split_ws) (void)hipFree(it->second.split_ws);
+    if (it->second.split_cnt) (void)hipFree(it->second.split_cnt);
+    g_scratch.erase(it);
+}
+
+namespace {
+
 bool attn_has_fast(int n_head, int n_head_kv, int head_dim)
 {
     const int attn_mode_now = g_attn_mode.load(std::memory_order_relaxed);
