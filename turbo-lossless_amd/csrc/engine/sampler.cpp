@@ -43,7 +43,7 @@ int* result_buffer(int batch, hipStream_t stream)
 }  // namespace
 
 // Called by t12_release_stream: the buffer of (current device, stream) goes with the stream.
-extern "C" void t12_sampler_release_stream(hipStream_t stream)
+extern "C" __attribute__((visibility("hidden"))) void t12_sampler_release_stream(hipStream_t stream)
 {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) dev = 0;

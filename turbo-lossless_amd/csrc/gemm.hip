@@ -42,8 +42,9 @@
 #include "t12_device.h"
 #include "t12_host.h"
 
-extern "C" void t12_glue_release_stream(hipStream_t st);      // glue.hip
-extern "C" void t12_sampler_release_stream(hipStream_t st);   // engine/sampler.cpp
+// library-internal (hidden: not part of the ABI)
+extern "C" __attribute__((visibility("hidden"))) void t12_glue_release_stream(hipStream_t st);      // glue.hip
+extern "C" __attribute__((visibility("hidden"))) void t12_sampler_release_stream(hipStream_t st);   // engine/sampler.cpp
 
 namespace {
 

@@ -1380,7 +1380,7 @@ StreamScratch* attn_split_scratch(hipStream_t st)
 
 // Frees this file's scratch of (current device, stream): argmax partials, context-split buffers.  The caller has
 // made sure that nothing enqueued on the stream still uses them (t12_release_stream waits for the stream).
-extern "C" void t12_glue_release_stream(hipStream_t st)
+extern "C" __attribute__((visibility("hidden"))) void t12_glue_release_stream(hipStream_t st)
 {
     std::lock_guard<std::mutex> lock(g_mu);
     auto it = g_scratch.find({current_device(), st});
