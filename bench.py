@@ -56,9 +56,9 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per gemv launch of the gemv_stack_b1 workload, from two rocprofv3 --pmc runs of this file
 # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from the --calibrate copy kernel; the summary is
 # profiles/gemv_stream_kernel_llama8b_stack_b1.md).  Valid for the full 32-layer stack only.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"gemv_stack_b1": 88.48e6,
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"gemv_stack_b1": 88.50e6,
                                      # gate|up at B = 256 (profiles/gemm_kernels_llama8b_layers.md)
-                                     "gemm_gate_up_b256": 226.8e6}
+                                     "gemm_gate_up_b256": 226.5e6}
 
 
 def synth_weight(torch, M, K, seed, dev, sigma=0.02, p_out=3e-4, sigma_out=8.0):
