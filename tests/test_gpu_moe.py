@@ -173,3 +173,27 @@ def test_moe_route_tables_and_refusals(t12, oracle, synth, moe):
     bad[5, 1] = E
     with pytest.raises(t12.T12Error, match="outside"):
         layer(Xd[:, :n], torch.from_numpy(bad).to(dev()), torch.from_numpy(w_h).to(dev()))
+
+
+def test_moe_twenty_experts_in_several_grouped_launches(t12, oracle, synth, moe):
+    """More experts than one grouped launch holds (16 groups): gate|up go out eight experts at a time, down sixteen."""
+    E, n, n_ff, T, k = 20, 128, 256, 90, 2
+    packs = [[oracle.pack(synth.weights_llm(m, kk, seed=1300 + 3 * e + j, p_outlier=1e-3))
+              for j, (m, kk) in enumerate([(n_ff, n), (n_ff, n), (n, n_ff)])] for e in range(E)]
+    layer = moe.MoeLayer([moe.Expert(*[t12.DeviceTensor12.from_packed(p, dev()) for p in ps]) for ps in packs])
+    X = synth.activations(T, n, seed=80)
+    rng = np.random.default_rng(9)
+    ids_h = np.stack([rng.choice(E, size=k, replace=False) for _ in range(T)]).astype(np.int64)
+    w_h = rng.random((T, k)).astype(np.float32)
+    got = layer(to_dev_bits(X).reshape(T, n), torch.from_numpy(ids_h).to(dev()), torch.from_numpy(w_h).to(dev())).cpu().numpy()
+    ref = np.zeros((T, n), np.float64)
+    for e in range(E):
+        rows, slots = np.nonzero(ids_h == e)
+        if len(rows) == 0:
+            continue
+        a = oracle.silu_mul_bf16(oracle.gemm(packs[e][0], X[rows]), oracle.gemm(packs[e][1], X[rows]))
+        ref[rows] += w_h[rows, slots][:, None].astype(np.float64) * oracle.gemm(packs[e][2], a)
+    assert rel_err(got, ref) < 1e-4
+    with pytest.raises(t12.T12Error, match="experts"):
+        moe.MoeLayer([layer.experts[0]] * 33)(to_dev_bits(X).reshape(T, n), torch.from_numpy(ids_h).to(dev()),
+                                              torch.from_numpy(w_h).to(dev()))
