@@ -1014,16 +1014,12 @@ int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_st
         T12_CHECK_LAUNCH("t12_gemm(dense16)");
         return T12_OK;
     }
-    // K split: fill the chip.  A 256-row batch tile needs a whole CU (LDS, accumulators);
-    // smaller batch tiles fit 2-4 workgroups per CU.  Every split keeps >= 4 stages; with 256-row batch tiles
-    // >= 8: a 4096 x 4096 tensor then runs as 128 workgroups in the time 256 take, and leaves half the partial
-    // sums (4 x 4 MB instead of 8 x 4 MB at B = 256) for the kernel that adds them up.
+    // K split: as many workgroups as the chip has CUs, not more (measured on the four Llama-8B layer shapes at B = 32 ..
+    // 256: 32 row tiles run best as 8 splits, 48 as 4, 224 unsplit -- every doubling past ~one workgroup per CU costs more
+    // in partial sums than it gains), every split at least 8 stages long.
     const int btiles = B > 128 ? (B + 255) / 256 : 1;
-    const int per_cu = B > 64 ? 1 : 2;
-    const int want = 256 * per_cu;
     int ks = 1;
-    const int min_stages = B > 128 ? 16 : 8;
-    while (tiles * btiles * ks * 4 < want * 3 && K / (ks * 2) >= min_stages * KC && ks < T12_MAX_KSPLIT) ks *= 2;
+    while (tiles * btiles * ks * 2 <= 256 + 32 && K / (ks * 2) >= 8 * KC && ks < T12_MAX_KSPLIT) ks *= 2;
     int kslice = (((K + 2 * KC - 1) / (2 * KC) + ks - 1) / ks) * 2 * KC;      // whole windows of two stages
     ks = (K + kslice - 1) / kslice;
     p.ksplit = ks;
@@ -1156,10 +1152,8 @@ int t12_gemm_grouped(const T12Group* groups, int ngroups, int K, void* stream)
         units += (long)t * ((p.seg_B[i] + tb - 1) / tb);
     }
     p.blk_start[n] = tiles;
-    const int want = 256 * (tb <= 64 ? 2 : 1);
     int ks = 1;
-    const int min_stages = tb > 128 ? 16 : 8;
-    while (units * ks * 4 < (long)want * 3 && K / (ks * 2) >= min_stages * KC && ks < T12_MAX_KSPLIT) ks *= 2;
+    while (units * ks * 2 <= 256 + 32 && K / (ks * 2) >= 8 * KC && ks < T12_MAX_KSPLIT) ks *= 2;   // as in t12_gemm
     const int kslice = (((K + 2 * KC - 1) / (2 * KC) + ks - 1) / ks) * 2 * KC;
     ks = (K + kslice - 1) / kslice;
     p.ksplit = ks;
