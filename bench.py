@@ -14,7 +14,7 @@ Workloads (synthetic, seeded, random-init weights of the Llama-3.1-8B shape:
                   `value`; B = 256 is measured in the same run and reported under "b256"; the
                   decode-GEMV launches of a step are also timed alone for `roofline`.
 
-  gemm_layers     the four linear-layer shapes through the fused decode+GEMM at B = 16, 64, 256 on three
+  gemm_layers     the four linear-layer shapes through the fused decode+GEMM at B = 2, 4, 8, 16, 64, 256 on three
                   rotating weight copies; `roofline` prices gate|up at B = 256 against
                   the 2.5 PFLOP/s dense bf16 MFMA peak.
 
@@ -438,7 +438,7 @@ def run_attention(args, t12, torch, dev):
     }
 
 
-def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(4, 8, 16, 64, 256), iters=50):
+def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(2, 4, 8, 16, 64, 256), iters=50):
     """decode+GEMM per layer shape: for each B, each of QKV (3 segments), O, gate|up
     (2 segments), down is timed over `n_rot` distinct weight copies in rotation, so that neither L2 nor
     the 256 MB last-level cache holds a tensor between launches.  weight_of(copy, which) -> (segment, K, P).
@@ -547,7 +547,7 @@ def run_tokenizer(args, t12):
 
 
 def run_gemm_layers(args, t12, torch, dev):
-    """The four Llama-3.1-8B linear-layer shapes through the fused decode+GEMM at B = 16, 64, 256 on three
+    """The four Llama-3.1-8B linear-layer shapes through the fused decode+GEMM at B = 2, 4, 8, 16, 64, 256 on three
     rotating weight copies; one step = the four layer GEMMs of one decoder layer at B = 256."""
     cfg = dict(LLAMA8B)
     n, ff = cfg["n_embd"], cfg["n_ff"]
@@ -577,7 +577,7 @@ def run_gemm_layers(args, t12, torch, dev):
         "ms_per_step": us256 / 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "gemm_layers: QKV 4096->6144 (3 segments), O 4096->4096, gate|up 4096->28672 (2 segments), "
-                               "down 14336->4096; N(0,0.02)+3e-4 outliers; B in {16,64,256}; 3 rotating weight copies"},
+                               "down 14336->4096; N(0,0.02)+3e-4 outliers; B in {2,4,8,16,64,256}; 3 rotating weight copies"},
         "layers": layers,
         "roofline": {"bound": "mfma", "achieved": gu["TFLOPs"], "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": gu["TFLOPs"] / 2500.0, "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get("gemm_gate_up_b256"),

@@ -338,3 +338,24 @@ def test_gemm_small_batch_segments_and_strides(t12, oracle, synth):
     for p in ps:
         assert rel_err(h[:, off:off + p.M], oracle.gemm(p, X)) < TOL
         off += p.M
+
+
+@pytest.mark.parametrize("B", [2, 3, 4])
+@pytest.mark.parametrize("M,K,law", [(4096, 4096, "llm"), (101, 2048, "diffusion"), (8, 1024, "llm"), (300, 8192, "diffusion")])
+def test_gemm_two_to_four_rows_whole_row_kernel(t12, oracle, synth, M, K, law, B):
+    """B = 2 with K a multiple of 1024 (up to 8192) takes the kernel whose waves read whole rows, like the B = 1
+    kernel, with one accumulator per batch row (B = 3, 4 on the same shapes: the 16-row MFMA kernel): ragged row
+    counts, the largest K its LDS holds, escape-heavy rows (more entries than lanes), unpatched mode; and three
+    tensors with three base_exp in one launch."""
+    w = synth.weights_diffusion(M, K, seed=M + K) if law == "diffusion" else synth.weights_llm(M, K, seed=M + K, p_outlier=1e-3)
+    p = oracle.pack(w)
+    X = synth.activations(B, K, seed=B)
+    (got,) = run_gemm(t12, [p], X)
+    assert rel_err(got, oracle.gemm(p, X)) < TOL
+    (un,) = run_gemm(t12, [p], X, patched=False)
+    assert rel_err(un, oracle.gemm(p, X, patched=False)) < TOL
+    if M == 101:
+        ps = [p, oracle.pack(synth.weights_llm(9, K, seed=2, sigma=0.3)), oracle.pack(synth.weights_llm(64, K, seed=3, sigma=0.002))]
+        outs = run_gemm(t12, ps, X)
+        for q, o in zip(ps, outs):
+            assert rel_err(o, oracle.gemm(q, X)) < TOL

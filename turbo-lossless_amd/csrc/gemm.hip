@@ -776,6 +776,127 @@ __global__ __launch_bounds__(NW * 64) void gemm_dense16_kernel(const GemmParams 
     }
 }
 
+// ---------------------------------------------------------------------------
+// Two batch rows: the B = 1 kernel's shape with NB accumulators.  A workgroup = 8 waves = 8 consecutive rows;
+// a wave reads its whole row front to back in 1024-column tiles (16 bytes of sign/mantissa + 8 bytes of nibbles per
+// lane and tile, nontemporal, ring of two tiles) -- the access pattern that streams fastest on this chip -- rebuilds
+// 16 weights per tile and multiplies them with the NB activation rows (v_dot2_f32_bf16), which the workgroup staged
+// in LDS, paired the way t12_decode8 orders its outputs, laid out per row and 1024-column chunk as [half][lane] x 16 B.
+// The decode is shared by the batch rows; per weight the kernel spends 2.25 + NB x 0.5 VALU operations and NB x 2
+// bytes of LDS reads: measured with NB = 4 it is level with the MFMA kernel below, which therefore takes over from
+// three rows on.  Escapes: (correct - wrong) * x[b, col] after the stream, x from LDS.  Wave sums by DPP.
+// Requires K % 1024 == 0, NB * K * 2 bytes of LDS (K <= 8192), 0 <= base_exp <= 240, aligned activation rows.
+// blk_start counts 8-row groups per segment.
+// ---------------------------------------------------------------------------
+template <int NB, int D>
+__global__ __launch_bounds__(512) void gemm_rows_kernel(const GemmParams p)
+{
+    extern __shared__ uint4 lds_x[];                   // [NB][T * 128]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = p.K, B = p.B;
+    const int T = K >> 10;
+    const int blk = blockIdx.x;
+    const int s = find_segment(p, blk);
+    const T12Segment& sg = p.seg[s];
+    const int M = sg.M;
+    const int row = (blk - p.blk_start[s]) * 8 + wave;
+    const bool live = row < M;                         // wave-uniform
+    const uint32_t be2 = t12_opaque(((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23));
+
+    // activations first (they come out of L2 and must not queue behind the weight tiles): piece = 8 columns,
+    // NB * K / 8 pieces over 512 threads
+    constexpr int XU = NB * 2;                         // pieces per thread at K = 8192
+    const int kp = K >> 3;                             // pieces per batch row
+    uint4 xpre[XU];
+#pragma unroll
+    for (int u = 0; u < XU; u++) {
+        const int idx = tid + 512 * u;
+        xpre[u] = make_uint4(0, 0, 0, 0);
+        if (idx < NB * kp) {
+            const int nb = idx / kp, q = idx - nb * kp;
+            xpre[u] = *(const uint4*)(p.act + (size_t)min(nb, B - 1) * p.act_stride + q * 8);   // rows past the batch: clamped, never stored
+        }
+    }
+    int e_beg = 0, e_end = 0;
+    if (live && sg.row_off) {
+        e_beg = sg.row_off[row];
+        e_end = sg.row_off[row + 1];
+    }
+    const size_t e0 = (size_t)min(row, M - 1) * K;     // rows past the end: clamped, never stored
+    const uint8_t* smp = sg.sm + e0 + lane * 16;
+    const uint8_t* grp = sg.gr + (e0 >> 1) + lane * 8;
+    uint4 rS[D];
+    uint2 rG[D];
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+        const int t = min(d, T - 1);
+        rS[d] = t12_ldg_stream16(smp + (size_t)t * 1024);
+        rG[d] = t12_ldg_stream8(grp + (size_t)t * 512);
+    }
+#pragma unroll
+    for (int u = 0; u < XU; u++) {
+        const int idx = tid + 512 * u;
+        if (idx < NB * kp) {
+            const int nb = idx / kp, q = idx - nb * kp;
+            lds_x[nb * (T * 128) + (q >> 7) * 128 + (q & 1) * 64 + ((q & 127) >> 1)] = t12_pair_acts(xpre[u]);
+        }
+    }
+    __syncthreads();
+
+    float acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) acc[nb] = 0.0f;
+    auto consume = [&](int slot, int t) {
+        uint32_t w0[4], w1[4];
+        t12_decode8(rS[slot].x, rS[slot].y, rG[slot].x, be2, w0);
+        t12_decode8(rS[slot].z, rS[slot].w, rG[slot].y, be2, w1);
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            const uint4 a0 = lds_x[nb * (T * 128) + t * 128 + lane];
+            const uint4 a1 = lds_x[nb * (T * 128) + t * 128 + 64 + lane];
+            float v = acc[nb];
+            v = t12_dot2(w0[0], a0.x, v);
+            v = t12_dot2(w0[1], a0.y, v);
+            v = t12_dot2(w0[2], a0.z, v);
+            v = t12_dot2(w0[3], a0.w, v);
+            v = t12_dot2(w1[0], a1.x, v);
+            v = t12_dot2(w1[1], a1.y, v);
+            v = t12_dot2(w1[2], a1.z, v);
+            v = t12_dot2(w1[3], a1.w, v);
+            acc[nb] = v;
+        }
+    };
+    for (int t = 0; t < T; t += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            if (t + d < T) {
+                consume(d, t + d);
+                if (t + d + D < T) {
+                    rS[d] = t12_ldg_stream16(smp + (size_t)(t + d + D) * 1024);
+                    rG[d] = t12_ldg_stream8(grp + (size_t)(t + d + D) * 512);
+                }
+            }
+        }
+    }
+    // escapes: the streamed value of an escaped weight is its "wrong" value
+    for (int e = e_beg + lane; e < e_end; e += 64) {
+        const int col = sg.cols[e];
+        const float delta = t12_bf16_to_f32((uint16_t)sg.correct[e]) - t12_bf16_to_f32((uint16_t)sg.wrong[e]);
+        const int q = col >> 3, i = col & 7;
+        const int slot = (q >> 7) * 128 + (q & 1) * 64 + ((q & 127) >> 1);
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            const uint16_t* h = (const uint16_t*)(lds_x + nb * (T * 128) + slot);
+            acc[nb] += delta * t12_bf16_to_f32(h[(i & 3) * 2 + (i >> 2)]);
+        }
+    }
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+        const float v = t12_wave_sum_lane63(acc[nb]);
+        if (lane == 63 && live && nb < B) sg.out[(size_t)nb * sg.out_stride + row] = v;
+    }
+}
+
 // ---- workspace for the K-split partial sums: one per (device, stream), grown on demand.  Launches on different
 //      streams may overlap, so they must not share partial sums; launches on one stream are ordered.
 struct Workspace {
@@ -992,6 +1113,21 @@ int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_st
         tiles += (segs[i].M + TM - 1) / TM;
     }
     p.blk_start[nseg] = tiles;
+    if (B == 2 && K % 1024 == 0 && K <= 8192) {
+        // two batch rows: whole-row waves with two accumulators (gate|up 32 us against 42 for the kernel below; with
+        // four accumulators the same kernel is no faster than the kernel below, 43-48 us, so it stops at two)
+        int groups = 0;
+        for (int i = 0; i < nseg; i++) {
+            p.blk_start[i] = groups;
+            groups += (segs[i].M + 7) / 8;
+        }
+        p.blk_start[nseg] = groups;
+        p.ksplit = 1;
+        p.kslice = K;
+        hipLaunchKernelGGL((gemm_rows_kernel<2, 2>), dim3(groups), dim3(512), (size_t)2 * K * 2, st, p);
+        T12_CHECK_LAUNCH("t12_gemm(rows)");
+        return T12_OK;
+    }
     if (B <= 16 && K % 128 == 0) {
         // row groups that share an activation load: as many as leave the launch >= 448 workgroups
         int groups16 = 0;
