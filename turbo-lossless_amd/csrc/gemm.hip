@@ -913,11 +913,18 @@ float* workspace(size_t bytes, hipStream_t st)
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     Workspace& w = g_ws[{dev, st}];
     if (w.bytes < bytes) {
+        // grows geometrically, in whole MiB: a caller whose shapes grow step by step pays the allocation (a device-wide
+        // wait) a few times, not once per shape
+        size_t want = bytes > 2 * w.bytes ? bytes : 2 * w.bytes;
+        want = (want + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
         if (w.ptr) (void)hipFree(w.ptr);          // waits for the device: nothing still reads the old buffer
         w.ptr = nullptr;
         w.bytes = 0;
-        if (hipMalloc((void**)&w.ptr, bytes) != hipSuccess) return nullptr;
-        w.bytes = bytes;
+        if (hipMalloc((void**)&w.ptr, want) != hipSuccess) {
+            want = bytes;
+            if (hipMalloc((void**)&w.ptr, want) != hipSuccess) return nullptr;
+        }
+        w.bytes = want;
     }
     return w.ptr;
 }
