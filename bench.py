@@ -482,6 +482,38 @@ def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(2, 4
             out["%s_b%d" % (name, B)] = {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
                                          "mfma_frac": round(flops / us / 1e6 / 2500.0, 4),
                                          "weight_GBps": round(wbytes / us / 1e3, 1), "flops": flops}
+        if B > 64:
+            # gate|up the way the engine's layer runs it: SiLU*mul in the GEMM's epilogue, bf16 [B, n_ff] out
+            # (t12_gemm_swiglu); same flops, 14.7 MB written at B = 256 instead of 58.7 MB
+            abuf = torch.empty((B, cfg["n_ff"]), dtype=torch.int16, device=dev)
+            pairs = []
+            for copy in range(n_rot):
+                sg, K, _ = weight_of(copy, 4)
+                su, _, _ = weight_of(copy, 5)
+                pairs.append((t12._seg_array([sg]), t12._seg_array([su]), K))
+            flops = 2.0 * 2 * cfg["n_ff"] * cfg["n_embd"] * B
+
+            def swiglu_pass():
+                for sg, su, K in pairs:
+                    rc = t12.lib.t12_gemm_swiglu(sg, su, xs[K].data_ptr(), K, K, B, abuf.data_ptr(), cfg["n_ff"], cur.cuda_stream)
+                    if rc:
+                        t12.check(min(rc, 0), "t12_gemm_swiglu")
+                        raise RuntimeError("t12_gemm_swiglu has no kernel for B = %d" % B)
+            for _ in range(5):
+                swiglu_pass()
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+            torch.cuda.synchronize()
+            for e0, e1 in evs:
+                e0.record(cur)
+                swiglu_pass()
+                e1.record(cur)
+            torch.cuda.synchronize()
+            rounds = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+            us = rounds[len(rounds) // 2] * 1e3 / n_rot
+            out["gate_up_swiglu_b%d" % B] = {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
+                                             "mfma_frac": round(flops / us / 1e6 / 2500.0, 4),
+                                             "weight_GBps": round(1.5 * 2 * cfg["n_ff"] * cfg["n_embd"] / us / 1e3, 1),
+                                             "flops": flops}
     return out
 
 
@@ -491,7 +523,10 @@ def gemm_b256_roofline(layers):
     fl = sum(layers["%s_b256" % k]["flops"] for k in names)
     return {"bound": "mfma", "achieved": fl / us / 1e6, "peak": 2500.0, "unit": "TFLOP/s", "frac": fl / us / 1e6 / 2500.0,
             "traffic": None, "kernel": "gemm_mfma_kernel, QKV + O + gate|up + down at B=256", "flops_per_step": fl,
-            "us_per_step": us, "gate_up_frac": layers["gate_up_b256"]["mfma_frac"]}
+            "us_per_step": us, "gate_up_frac": layers["gate_up_b256"]["mfma_frac"],
+            # the same four products as the engine's layer issues them: gate|up with SiLU*mul in its epilogue
+            "gate_up_swiglu_frac": layers["gate_up_swiglu_b256"]["mfma_frac"],
+            "frac_with_swiglu_epilogue": fl / (us - layers["gate_up_b256"]["us"] + layers["gate_up_swiglu_b256"]["us"]) / 1e6 / 2500.0}
 
 
 def run_tokenizer(args, t12):
