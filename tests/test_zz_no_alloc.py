@@ -19,6 +19,51 @@ def _call(t12, fn, dts, X, outs):
     return rc
 
 
+def _free_device_bytes():
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(), C.c_size_t()
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
+def test_noalloc_allocates_nothing_on_a_fresh_stream(t12, oracle):
+    """The property the entry point exists for: a K-split launch on a stream the library has never seen changes the
+    free device memory by nothing (t12_gemm on the same fresh stream grows a workspace with hipMalloc: the control
+    that shows the measurement sees such a thing)."""
+    synth = importlib.import_module("turbo_lossless_amd.synth")
+    lib = t12.lib
+    M, K, B = 1024, 4096, 200                                     # 8 row tiles: K is split, partial sums are needed
+    p = oracle.pack(synth.weights_llm(M, K, seed=61, p_outlier=2e-3))
+    dt = t12.DeviceTensor12.from_packed(p, dev())
+    X = synth.activations(B, K, seed=62)
+    Xd = to_dev_bits(X).reshape(X.shape)
+    o = torch.full((B, M), float("nan"), device=dev())
+    o2 = torch.full((B, M), float("nan"), device=dev())
+    segs = t12._seg_array([dt.segment(o)])
+    segs2 = t12._seg_array([dt.segment(o2)])
+    fresh = torch.cuda.Stream()                                   # default priority
+    fresh.wait_stream(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    # on the caller's own stream first: the library takes the array's device address once per device
+    assert lib.t12_gemm_noalloc(segs, 1, Xd.data_ptr(), K, M, K, B, t12.current_stream()) == 0
+    torch.cuda.synchronize()
+    o.fill_(float("nan"))
+    torch.cuda.synchronize()
+    before = _free_device_bytes()
+    assert lib.t12_gemm_noalloc(segs, 1, Xd.data_ptr(), K, M, K, B, fresh.cuda_stream) == 0, lib.t12_last_error()
+    torch.cuda.synchronize()
+    assert _free_device_bytes() == before
+    assert rel_err(o.cpu().numpy(), oracle.gemm(p, X)) < 1e-4
+    # control: the allocating entry point on the same fresh stream takes memory for its partial sums
+    assert lib.t12_gemm(segs2, 1, Xd.data_ptr(), K, M, K, B, fresh.cuda_stream) == 0
+    torch.cuda.synchronize()
+    taken = before - _free_device_bytes()
+    assert taken >= 8 * B * M * 4 // 2                            # at least the partial sums of a few splits
+    assert torch.equal(o, o2)
+    assert lib.t12_release_stream(fresh.cuda_stream) == 0
+
+
 def test_noalloc_equals_gemm_two_calls_in_a_row(t12, oracle):
     synth = importlib.import_module("turbo_lossless_amd.synth")
     lib = t12.lib
