@@ -141,8 +141,9 @@ int t12_gemm_swiglu(const T12Segment* gate, const T12Segment* up, const void* ac
 /* Several decode+GEMM products in one launch, group i multiplying its own activations:
  *   seg.out[b*seg.out_stride + m] = sum_k dec(W_i[m,k]) * X_i[b*act_stride + k],  b < B   (B == 0: group skipped)
  * for the experts of a mixture-of-experts layer (each expert over the rows routed to it; gate and up of one expert
- * are two groups with the same activations).  Same kernels and per-element results as one t12_gemm per group.  Up
- * to 16 groups.  No counterpart in the reference, whose entry point (nv_launch_split12_fused_gemm_async,
+ * are two groups with the same activations).  Every group runs on the tile kernel (also groups of 16 rows or
+ * fewer, which t12_gemm would give to its weight-stream kernels): the values are those of one t12_gemm per group
+ * up to the order of the fp32 sums.  Up to 16 groups.  No counterpart in the reference, whose entry point (nv_launch_split12_fused_gemm_async,
  * nvidia_kernels.cu:444) takes one tensor and would be called once per expert. */
 typedef struct T12Group {
     T12Segment  seg;          /* the tensor and its output (out, out_stride must be set) */
@@ -155,14 +156,18 @@ int t12_gemm_grouped(const T12Group* groups, int ngroups, int K, void* stream);
 /* A mixture-of-experts SwiGLU feed-forward layer over split-12 experts (a Mixtral-shaped layer):
  *   out[t, :] = sum_j weights[t*k + j] * W2_e( silu(W1_e x_t) * (W3_e x_t) ),  e = expert_ids[t*k + j],  j ascending
  * x bf16 [T, x_stride]; expert_ids [T, k] int32 or int64 (id_bytes 4 / 8) and weights [T, k] fp32 on the device;
- * out fp32 [T, out_stride].  The (token, slot) pairs are grouped per expert on the GPU, gate|up and down of all
- * experts run as t12_gemm_grouped launches (the SwiGLU activation rounded to bf16 in between, as the engine does,
- * inference.cpp:327), and the weighted sum is taken in a fixed order.  The call copies the per-expert counts to
- * the host and waits for the stream once.  workspace: device memory of t12_moe_workspace_bytes(...) bytes,
- * 256-byte aligned, owned by the caller (used from the first launch to the last).  Up to 32 experts; w1, w3 are
- * [n_ff, n_embd], w2 is [n_embd, n_ff]; their out fields are ignored.  No counterpart in the reference (no
- * MoE layer there); what it replaces is one nv_launch_split12_fused_gemm_async (nvidia_kernels.cu:444) per expert
- * and projection. */
+ * out fp32 [T, out_stride].  The (token, slot) pairs are grouped per expert on the GPU, gate|up and down of all experts
+ * run as grouped decode+GEMM launches (the SwiGLU activation rounded to bf16 in between, as the engine does,
+ * inference.cpp:327; in the gate|up epilogue when the experts receive more than 128 rows each), and the weighted sum
+ * is taken in a fixed order.  The call never waits for the stream: the grouped launches read the rows per expert from
+ * the routing kernel's tables on the device (one workgroup per row tile, which walks the expert's batch tiles).  An id
+ * outside 0..E-1 leaves its pair out of the sum and raises a flag that t12_moe_status reads (it waits for the stream).
+ * Shapes the tile kernel does not take (n_embd or n_ff not a multiple of 64, base_exp outside 0..240) copy the counts
+ * to the host and wait once per call.
+ * workspace: device memory of t12_moe_workspace_bytes(...) bytes, 256-byte aligned, owned by the caller (used from the
+ * first launch to the last).  Up to 128 experts; w1, w3 are [n_ff, n_embd], w2 is [n_embd, n_ff]; their out fields are
+ * ignored.  No counterpart in the reference (no MoE layer there); what it replaces is one
+ * nv_launch_split12_fused_gemm_async (nvidia_kernels.cu:444) per expert and projection. */
 typedef struct T12MoeExpert {
     T12Segment w1, w3, w2;
 } T12MoeExpert;
@@ -170,6 +175,7 @@ size_t t12_moe_workspace_bytes(int T, int k, int n_embd, int n_ff, int E);
 int t12_moe_ffn(const T12MoeExpert* experts, int E, const void* x_bf16, int x_stride, const void* expert_ids,
                 int id_bytes, const float* weights, int T, int k, int n_embd, int n_ff, void* workspace,
                 size_t workspace_bytes, float* out, int out_stride, void* stream);
+int t12_moe_status(const void* workspace, void* stream);
 
 /* t12_gemm for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  No counterpart in the reference (its GEMM never splits K and so has no

@@ -148,7 +148,7 @@ def test_grouped_gemm_general_path_and_errors(t12, oracle, synth, moe):
 
 def test_moe_route_tables_and_refusals(t12, oracle, synth, moe):
     """Ragged routing incl. an expert nobody chose, int32 ids, a strided activation matrix, k = 3: against the
-    oracle's per-expert products; an id outside the experts is refused."""
+    oracle's per-expert products; an id outside the experts is left out and reported by status()."""
     E, n, n_ff, T, k = 5, 256, 512, 77, 3
     packs = [[oracle.pack(synth.weights_llm(m, kk, seed=900 + 3 * e + j, p_outlier=1e-3))
               for j, (m, kk) in enumerate([(n_ff, n), (n_ff, n), (n, n_ff)])] for e in range(E)]
@@ -169,10 +169,35 @@ def test_moe_route_tables_and_refusals(t12, oracle, synth, moe):
         a = oracle.silu_mul_bf16(oracle.gemm(packs[e][0], X[rows]), oracle.gemm(packs[e][1], X[rows]))
         ref[rows] += w_h[rows, slots][:, None].astype(np.float64) * oracle.gemm(packs[e][2], a)
     assert rel_err(got, ref) < 1e-4
+    layer.status()                                          # nothing to report
+    # an id outside the experts: its pair is left out of the sum, and status() says so
     bad = ids_h.copy()
     bad[5, 1] = E
+    got_bad = layer(Xd[:, :n], torch.from_numpy(bad).to(dev()), torch.from_numpy(w_h).to(dev())).cpu().numpy()
     with pytest.raises(t12.T12Error, match="outside"):
-        layer(Xd[:, :n], torch.from_numpy(bad).to(dev()), torch.from_numpy(w_h).to(dev()))
+        layer.status()
+    e5 = int(ids_h[5, 1])
+    a = oracle.silu_mul_bf16(oracle.gemm(packs[e5][0], X[5:6]), oracle.gemm(packs[e5][1], X[5:6]))
+    ref_bad = ref.copy()
+    ref_bad[5] -= float(w_h[5, 1]) * oracle.gemm(packs[e5][2], a)[0].astype(np.float64)
+    assert rel_err(got_bad, ref_bad) < 1e-4
+    # tokens that name one expert twice: an expert then receives more rows than there are tokens (and more than one
+    # batch tile); both slots count
+    twice = ids_h.copy()
+    twice[:, 1] = twice[:, 0]
+    twice[:, 2] = twice[:, 0]
+    twice[:, 0] = 0                                          # expert 0 receives every token at least once
+    got2 = layer(Xd[:, :n], torch.from_numpy(twice).to(dev()), torch.from_numpy(w_h).to(dev())).cpu().numpy()
+    layer.status()
+    ref2 = np.zeros((T, n), np.float64)
+    for e in range(E):
+        rows, slots = np.nonzero(twice == e)
+        if len(rows) == 0:
+            continue
+        a = oracle.silu_mul_bf16(oracle.gemm(packs[e][0], X[rows]), oracle.gemm(packs[e][1], X[rows]))
+        np.add.at(ref2, rows, w_h[rows, slots][:, None].astype(np.float64) * oracle.gemm(packs[e][2], a))
+    assert np.bincount(twice.ravel(), minlength=E).max() > T
+    assert rel_err(got2, ref2) < 1e-4
 
 
 def test_moe_twenty_experts_in_several_grouped_launches(t12, oracle, synth, moe):
@@ -195,5 +220,28 @@ def test_moe_twenty_experts_in_several_grouped_launches(t12, oracle, synth, moe)
         ref[rows] += w_h[rows, slots][:, None].astype(np.float64) * oracle.gemm(packs[e][2], a)
     assert rel_err(got, ref) < 1e-4
     with pytest.raises(t12.T12Error, match="experts"):
-        moe.MoeLayer([layer.experts[0]] * 33)(to_dev_bits(X).reshape(T, n), torch.from_numpy(ids_h).to(dev()),
-                                              torch.from_numpy(w_h).to(dev()))
+        moe.MoeLayer([layer.experts[0]] * 129)(to_dev_bits(X).reshape(T, n), torch.from_numpy(ids_h).to(dev()),
+                                               torch.from_numpy(w_h).to(dev()))
+
+
+def test_moe_sixty_four_experts_and_a_shape_sized_on_the_host(t12, oracle, synth, moe):
+    """64 experts (the routing sort's count rows take more than 48 KB of LDS), top-4; and a layer whose widths are not
+    multiples of 64, which the tile kernel does not take: its launches are sized from a host copy of the counts."""
+    for E, n, n_ff, T, k, seed in [(64, 128, 128, 150, 4, 1500), (3, 96, 160, 40, 2, 1700)]:
+        packs = [[oracle.pack(synth.weights_llm(m, kk, seed=seed + 3 * e + j, p_outlier=1e-3))
+                  for j, (m, kk) in enumerate([(n_ff, n), (n_ff, n), (n, n_ff)])] for e in range(E)]
+        layer = moe.MoeLayer([moe.Expert(*[t12.DeviceTensor12.from_packed(p, dev()) for p in ps]) for ps in packs])
+        X = synth.activations(T, n, seed=seed + 1)
+        rng = np.random.default_rng(seed)
+        ids_h = np.stack([rng.choice(E, size=k, replace=False) for _ in range(T)]).astype(np.int32)
+        w_h = rng.random((T, k)).astype(np.float32)
+        got = layer(to_dev_bits(X).reshape(T, n), torch.from_numpy(ids_h).to(dev()), torch.from_numpy(w_h).to(dev())).cpu().numpy()
+        layer.status()
+        ref = np.zeros((T, n), np.float64)
+        for e in range(E):
+            rows, slots = np.nonzero(ids_h == e)
+            if len(rows) == 0:
+                continue
+            a = oracle.silu_mul_bf16(oracle.gemm(packs[e][0], X[rows]), oracle.gemm(packs[e][1], X[rows]))
+            ref[rows] += w_h[rows, slots][:, None].astype(np.float64) * oracle.gemm(packs[e][2], a)
+        assert rel_err(got, ref) < 1e-4, (E, n)

@@ -82,8 +82,16 @@ struct GemmParams {
     int m_total;                           // sum of M over segments
     const uint16_t* act;
     float* ws;                             // partial sums when ksplit > 1
-    uint16_t* out_bf16;                    // SwiGLU mode: bf16 [B, out_bf16_ld], silu(seg 0) * seg 1
+    uint16_t* out_bf16;                    // SwiGLU mode: bf16 [B, out_bf16_ld], silu(seg 2i) * seg 2i+1 of pair i
     int out_bf16_ld;
+    int npair = 1;                         // SwiGLU mode: (gate, up) pairs of the launch; blk_start[i] = first tile of pair i
+    // Rows per group known on the device only (the experts of a mixture-of-experts layer, counted by the routing
+    // kernel): group_of_seg[s] picks an entry of dev_counts / dev_base, the segment's batch is dev_counts[.] and its
+    // activations, outputs (fp32 and bf16) start dev_base[.] rows into the pointers given.  The grid then has one
+    // workgroup per row tile, which walks the group's batch tiles.  nullptr: seg_B as given.
+    const int* dev_counts = nullptr;
+    const int* dev_base = nullptr;
+    int group_of_seg[GMAX];
 };
 
 // LDS slot of (unit, row) in a [units][rows] array of 16-byte units.  Rows are rotated
@@ -109,6 +117,14 @@ __device__ __forceinline__ int find_segment(const GemmParams& p, int tile)
 #pragma unroll
     for (int i = 1; i < GMAX; i++)
         if (i < p.nseg && tile >= p.blk_start[i]) s = i;
+    return s;
+}
+__device__ __forceinline__ int find_pair(const GemmParams& p, int tile)
+{
+    int s = 0;
+#pragma unroll
+    for (int i = 1; i < GMAX / 2; i++)
+        if (i < p.npair && tile >= p.blk_start[i]) s = i;
     return s;
 }
 
@@ -138,8 +154,9 @@ __device__ __forceinline__ int find_segment(const GemmParams& p, int tile)
 // 32..63 -- so that the two accumulator tiles of a wave are gate and up of the SAME 32 rows and the epilogue
 // writes bf16( silu(gate) * up ) straight from registers: the reference's silu_mul_bf16 kernel
 // (engine/kernels.hip:447-459) and the fp32 round trip of both projections folded away.
+// bt: batch tile.  Returns false when the tile lies past the segment's rows (nothing was done).
 template <int WB, int WM, int FB, int FM, bool SWI = false>
-__device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
+__device__ __forceinline__ bool gemm_mfma_body(const GemmParams& p, const int bt)
 {
     static_assert(!SWI || FM == 2, "the SwiGLU epilogue pairs the two row tiles of a wave");
     constexpr int TB = WB * FB * 32;                  // batch rows per workgroup
@@ -158,24 +175,27 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
     const int ln = lane & 31, lh = lane >> 5;
 
     const int tile = blockIdx.x;
-    const int s = SWI ? 0 : find_segment(p, tile);
+    const int pair = SWI ? find_pair(p, tile) : 0;
+    const int s = SWI ? 2 * pair : find_segment(p, tile);          // SWI: the gate segment of the tile's pair
     const T12Segment& sg = p.seg[s];
-    const int M = sg.M, K = p.K, B = p.seg_B[s];
-    const uint16_t* const act = p.seg_act[s];
+    const int M = sg.M, K = p.K;
+    const int B = p.dev_counts ? p.dev_counts[p.group_of_seg[s]] : p.seg_B[s];
+    const int row_base = p.dev_base ? p.dev_base[p.group_of_seg[s]] : 0;     // first row of this group in act / out
     const int act_stride = p.seg_act_stride[s];
-    if ((int)blockIdx.y * (WB * FB * 32) >= B) return;     // grouped launch: this segment has fewer batch tiles than the grid
-    const int m0 = SWI ? tile * (TM / 2) : (tile - p.blk_start[s]) * TM;
+    const uint16_t* const act = p.seg_act[s] + (size_t)row_base * act_stride;
+    if (bt * (WB * FB * 32) >= B) return false;            // grouped launch: this segment has fewer batch tiles than the grid
+    const int m0 = SWI ? (tile - p.blk_start[pair]) * (TM / 2) : (tile - p.blk_start[s]) * TM;
     // local row r of the tile -> segment and matrix row
-    auto row_seg = [&](int r) { return SWI ? (r >> 5) & 1 : s; };
+    auto row_seg = [&](int r) { return SWI ? s + ((r >> 5) & 1) : s; };
     auto row_mat = [&](int r) { return SWI ? m0 + ((r >> 6) << 5) + (r & 31) : m0 + r; };
-    const int b0 = blockIdx.y * TB;
+    const int b0 = bt * TB;
     const int k_begin = blockIdx.z * p.kslice;
     const int k_end = min(K, k_begin + p.kslice);
     const int nstage = (k_end - k_begin) / KC;
     uint32_t be2s[2];
 #pragma unroll
     for (int j = 0; j < 2; j++) {
-        const int be = p.seg[SWI ? j : s].base_exp;
+        const int be = p.seg[SWI ? s + j : s].base_exp;
         be2s[j] = t12_opaque(((uint32_t)be << 7) | ((uint32_t)be << 23));
     }
 
@@ -266,8 +286,8 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
     int esc_mode = 0;
     if (SWI) {
         // two slices: the 64 gate rows, then the 64 up rows
-        const T12Segment& g0 = p.seg[0];
-        const T12Segment& g1 = p.seg[1];
+        const T12Segment& g0 = p.seg[s];
+        const T12Segment& g1 = p.seg[s + 1];
         const int r_lo = min(m0, M), r_hi = min(m0 + TM / 2, M);
         const int e00 = g0.row_off ? g0.row_off[r_lo] : 0, e10 = g1.row_off ? g1.row_off[r_lo] : 0;
         const int n0 = g0.row_off ? g0.row_off[r_hi] - e00 : 0, n1 = g1.row_off ? g1.row_off[r_hi] - e10 : 0;
@@ -448,7 +468,7 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
     if (blockIdx.z == 0 && esc_mode == 2) {
 #pragma unroll
         for (int j = 0; j < FM; j++) {
-            const T12Segment& g = p.seg[SWI ? j : s];
+            const T12Segment& g = p.seg[SWI ? s + j : s];
             const int m = SWI ? m0 + wm * 32 + ln : m0 + (wm * FM + j) * 32 + ln;
             if (m < M && g.row_off) {
                 const int beg = g.row_off[m], end = g.row_off[m + 1];
@@ -472,6 +492,7 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
     //      D[row = 8*(r/4) + 4*lh + r%4][col = ln]   (row = batch, col = m)
     if (SWI) {
         const int m = m0 + wm * 32 + ln;
+        uint16_t* const ob = p.out_bf16 + (size_t)row_base * p.out_bf16_ld;
 #pragma unroll
         for (int i = 0; i < FB; i++)
 #pragma unroll
@@ -479,9 +500,9 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
                 const int b = b0 + (wb * FB + i) * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
                 const float g = acc[i][0][r];
                 if (m < M && b < B)
-                    p.out_bf16[(size_t)b * p.out_bf16_ld + m] = t12_f32_to_bf16(g / (1.0f + expf(-g)) * acc[i][FM - 1][r]);
+                    ob[(size_t)b * p.out_bf16_ld + m] = t12_f32_to_bf16(g / (1.0f + expf(-g)) * acc[i][FM - 1][r]);
             }
-        return;
+        return true;
     }
     float* dst;
     size_t ld;
@@ -489,7 +510,7 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
         dst = p.ws + (size_t)blockIdx.z * p.split_stride + p.seg_ws0[s];
         ld = p.seg_ld[s];
     } else {
-        dst = sg.out;
+        dst = sg.out + (size_t)row_base * sg.out_stride;
         ld = sg.out_stride;
     }
 #pragma unroll
@@ -503,13 +524,20 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams& p)
                 if (m < M && b < B) dst[(size_t)b * ld + m] = acc[i][j][r];
             }
         }
+    return true;
 }
 
 // Eight waves per workgroup, two per SIMD: one wave's decode / LDS traffic runs under the other's MFMAs.
+// Batch tiles: one per workgroup (blockIdx.y), except when the rows per group are known on the device only: such
+// a launch has one workgroup per row tile, which takes the group's batch tiles one after the other (a group within
+// the tile -- the usual case -- is streamed once, a larger one once per tile; no group's rows can fall outside the grid).
 template <int WB, int WM, int FB, int FM, bool SWI = false>
 __global__ __launch_bounds__(WB * WM * 64) void gemm_mfma_kernel(const GemmParams p)
 {
-    gemm_mfma_body<WB, WM, FB, FM, SWI>(p);
+    for (int bt = blockIdx.y;; bt++) {
+        if (!gemm_mfma_body<WB, WM, FB, FM, SWI>(p, bt) || !p.dev_counts) break;
+        __syncthreads();                                   // the next tile reuses the staging buffers
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -971,17 +999,21 @@ int launch_mfma(GemmParams& p, int tiles, hipStream_t st)
     const dim3 grid(tiles, (p.B + TB - 1) / TB, p.ksplit);   // batch tiles of one row tile are neighbours in time
     auto kfn = gemm_mfma_kernel<WB, WM, FB, FM, SWI>;
     static bool attr_done[16] = {};                    // the attribute is per device
+    static std::mutex attr_mutex;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) dev = 0;
-    bool& attr_set = attr_done[dev];
-    if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                2 * STAGE_BYTES + PATCH_BYTES) !=
-            hipSuccess) {
-            t12_set_error("t12_gemm: cannot reserve %d bytes of LDS", 2 * STAGE_BYTES);
-            return T12_ELAUNCH;
+    {
+        std::lock_guard<std::mutex> attr_lock(attr_mutex);
+        bool& attr_set = attr_done[dev];
+        if (!attr_set) {
+            if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    2 * STAGE_BYTES + PATCH_BYTES) !=
+                hipSuccess) {
+                t12_set_error("t12_gemm: cannot reserve %d bytes of LDS", 2 * STAGE_BYTES);
+                return T12_ELAUNCH;
+            }
+            attr_set = true;
         }
-        attr_set = true;
     }
     hipLaunchKernelGGL(kfn, grid, dim3(WB * WM * 64), 2 * STAGE_BYTES + PATCH_BYTES, st, p);
     T12_CHECK_LAUNCH("t12_gemm");
@@ -1318,6 +1350,69 @@ int t12_gemm_grouped(const T12Group* groups, int ngroups, int K, void* stream)
         T12_CHECK_LAUNCH("t12_gemm_grouped(reduce)");
     }
     return T12_OK;
+}
+
+// Library-internal (t12_moe_ffn): the experts of a mixture-of-experts layer in one launch, with the rows per expert
+// known on the device only.  pairs = 0: segment i belongs to group first_group + i; 1 or 2: the segments are (gate, up)
+// pairs, segment i belongs to group first_group + i / 2.  Group g has dev_counts[g] rows, which start dev_base[g] rows
+// into act_bf16 and into the outputs: seg.out (fp32), or for pairs = 1 out_bf16 = bf16( silu(gate) * up ), row stride
+// out_bf16_ld.  hint_b is a count few groups exceed: it
+// picks the batch tile (a group above it is streamed once per tile it needs).  K is never split.  Returns 1 when the shape has no such kernel (the caller then sizes launches on the host).
+__attribute__((visibility("hidden"))) int t12_gemm_experts(const T12Segment* segs, int nseg, int K, const void* act_bf16,
+                                                           int act_stride, const int* dev_counts, const int* dev_base,
+                                                           int first_group, int hint_b, int pairs,
+                                                           void* out_bf16, int out_bf16_ld, void* stream)
+{
+    const bool swiglu = pairs == 1;
+    if (nseg < 1 || nseg > GMAX || (pairs && nseg % 2)) return 1;
+    if (K % KC || act_stride % 8 || (uintptr_t)act_bf16 % 16) return 1;
+    for (int i = 0; i < nseg; i++)
+        if (segs[i].base_exp < 0 || segs[i].base_exp > 240 || !segs[i].sm || !segs[i].gr) return 1;
+    GemmParams p;
+    p.K = K;
+    p.act = (const uint16_t*)act_bf16;
+    p.act_stride = act_stride;
+    p.ws = nullptr;
+    p.ksplit = 1;
+    p.kslice = ((K + 2 * KC - 1) / (2 * KC)) * 2 * KC;
+    p.out_bf16 = (uint16_t*)out_bf16;
+    p.out_bf16_ld = out_bf16_ld;
+    p.dev_counts = dev_counts;
+    p.dev_base = dev_base;
+    p.nseg = nseg;
+    p.B = 1;                               // one workgroup per row tile (it walks the group's batch tiles itself)
+    p.split_stride = 0;
+    int tiles = 0, m_total = 0;
+    for (int i = 0; i < nseg; i++) {
+        p.seg[i] = segs[i];
+        p.seg_row0[i] = m_total;
+        p.seg_act[i] = p.act;
+        p.seg_B[i] = 0;
+        p.seg_act_stride[i] = act_stride;
+        p.seg_ws0[i] = 0;
+        p.seg_ld[i] = segs[i].M;
+        p.group_of_seg[i] = first_group + (pairs ? i / 2 : i);
+        m_total += segs[i].M;
+        if (!swiglu) {
+            p.blk_start[i] = tiles;
+            tiles += (segs[i].M + TM - 1) / TM;
+        } else if (i % 2 == 0) {
+            if (segs[i].M != segs[i + 1].M) return 1;
+            p.blk_start[i / 2] = tiles;
+            tiles += (segs[i].M + TM / 2 - 1) / (TM / 2);
+        }
+    }
+    p.m_total = m_total;
+    p.npair = swiglu ? nseg / 2 : 1;
+    if (!swiglu) p.blk_start[nseg] = tiles;
+    hipStream_t st = (hipStream_t)stream;
+    if (swiglu) {
+        if (hint_b <= 128) return launch_mfma<4, 2, 1, 2, true>(p, tiles, st);
+        return launch_mfma<4, 2, 2, 2, true>(p, tiles, st);
+    }
+    if (hint_b <= 64) return launch_mfma<2, 4, 1, 1>(p, tiles, st);
+    if (hint_b <= 128) return launch_mfma<2, 4, 2, 1>(p, tiles, st);
+    return launch_mfma<4, 2, 2, 2>(p, tiles, st);
 }
 
 // The library keeps device buffers per (device, stream): the K-split partial sums of t12_gemm*, the argmax partials and the

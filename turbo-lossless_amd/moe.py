@@ -2,8 +2,9 @@
 
 The reference engine has no MoE layer; its decode+GEMM entry point (`nv_launch_split12_fused_gemm_async`,
 nvidia_kernels.cu:444) would be called once per expert and projection with that expert's token count as B.  Here
-the layer is the library's `t12_moe_ffn`: the (token, slot) pairs are grouped per expert on the GPU, gate|up and
-down of all experts run as grouped decode+GEMM launches, and the weighted sum is taken in a fixed order.  torch
+the layer is the library's `t12_moe_ffn`: the (token, slot) pairs are grouped per expert on the GPU, gate|up (SwiGLU
+in the epilogue) and down of all experts run as grouped decode+GEMM launches that read the rows per expert from the
+device, and the weighted sum is taken in a fixed order; the host never waits.  torch
 holds the buffers; `route_top_k` (top-k and softmax of the router logits) is the only torch arithmetic, and it is
 not part of `moe_ffn`.
 """
@@ -45,8 +46,9 @@ class MoeLayer:
 
     def __call__(self, X, expert_ids, weights, out=None, stream=None):
         """X bf16 bits [T, n_embd] (int16 tensor, rows may be strided); expert_ids [T, k] int32 / int64 and weights
-        [T, k] fp32, contiguous; returns fp32 [T, n_embd] = sum_j w[t,j] * FFN_{e[t,j]}(x_t).  Waits for the stream
-        once (the host sizes the grouped launches by the per-expert counts)."""
+        [T, k] fp32, contiguous; returns fp32 [T, n_embd] = sum_j w[t,j] * FFN_{e[t,j]}(x_t).  Nothing waits for the
+        stream; the k ids of a token must be distinct.  An id outside the experts leaves its pair out of the sum:
+        status() tells (it waits for the stream)."""
         torch = _torch()
         T, n = X.shape
         k = expert_ids.shape[1]
@@ -59,7 +61,14 @@ class MoeLayer:
         check(lib.t12_moe_ffn(self.table, len(self.experts), X.data_ptr(), X.stride(0), expert_ids.data_ptr(),
                               expert_ids.element_size(), weights.data_ptr(), T, k, n, self.n_ff, ws.data_ptr(), ws.numel(),
                               out.data_ptr(), out.stride(0), st), "t12_moe_ffn")
+        self._last_stream = st
         return out
+
+    def status(self):
+        """Waits for the stream of the last call and raises T12Error if its routing met an id outside the experts (or
+        a token that named one expert twice)."""
+        if self.ws is not None:
+            check(lib.t12_moe_status(self.ws.data_ptr(), getattr(self, "_last_stream", current_stream())), "t12_moe_status")
 
 
 def moe_ffn(experts, X, expert_ids, weights, stream=None):
