@@ -53,12 +53,28 @@ sys.path.insert(0, ROOT)
 
 LLAMA8B = dict(n_layer=32, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=8, n_vocab=128256)
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per gemv launch of the gemv_stack_b1 workload, from two rocprofv3 --pmc runs of this file
-# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from the --calibrate copy kernel; the summary is
-# profiles/gemv_stream_kernel_llama8b_stack_b1.md).  Valid for the full 32-layer stack only.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"gemv_stack_b1": 88.50e6,
-                                     # gate|up at B = 256 (profiles/gemm_kernels_llama8b_layers.md)
-                                     "gemm_gate_up_b256": 226.5e6}
+
+
+def measured_traffic(key):
+    """HBM bytes per launch of the named kernel, from profiles/measured_traffic.txt: the figure two rocprofv3 --pmc
+    runs of this file gave (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from the --calibrate copy kernel), written
+    down with the first 16 hex digits of the SHA-256 of the kernel's source file at the time.  A figure whose source
+    file has changed since is reported as None: counters are not read by this run."""
+    import hashlib
+    path = os.path.join(ROOT, "profiles", "measured_traffic.txt")
+    try:
+        lines = open(path).read().splitlines()
+    except OSError:
+        return None
+    for line in lines:
+        f = line.split()
+        if len(f) >= 4 and not line.startswith("#") and f[0] == key:
+            try:
+                now = hashlib.sha256(open(os.path.join(ROOT, f[2]), "rb").read()).hexdigest()[:16]
+            except OSError:
+                return None
+            return float(f[1]) if now == f[3] else None
+    return None
 
 
 def synth_weight(torch, M, K, seed, dev, sigma=0.02, p_out=3e-4, sigma_out=8.0):
@@ -248,7 +264,8 @@ def run_decode(args, t12, torch, dev):
     achieved = alg_bytes / (ms_gemv * 1e-3) / 1e9
 
     gemm_layers = gemm_layer_leg(t12, torch, dev, cfg, lambda layer, which: eng.weight(layer, which), min(3, n_l),
-                                 cur, g)
+                                 cur, g, batches=(2, 4, 8, 16, 32, 64, 128, 256), yardstick=True)
+    probe = clock_probe(t12)
 
     # ---- B = 256
     b256 = None
@@ -298,12 +315,16 @@ def run_decode(args, t12, torch, dev):
         "gemm_layers": gemm_layers,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["gemv_stack_b1"] if n_l == LLAMA8B["n_layer"] else None,
+                     "traffic": measured_traffic("gemv_stack_b1") if n_l == LLAMA8B["n_layer"] else None,
                      "kernel": "gemv_stream_kernel", "bytes_per_launch": alg_bytes / len(tabs),
                      "us_per_launch": ms_gemv * 1e3 / len(tabs),
                      # the other target of the path: decode+GEMM at B = 256 over the four linear layers of a decoder
                      # layer, against the dense bf16 MFMA peak (median launch times of gemm_layers above)
-                     "gemm_b256": gemm_b256_roofline(gemm_layers)},
+                     "gemm_b256": {**gemm_b256_roofline(gemm_layers),
+                                   "clock_ghz_mfma_only_256wg": probe["mfma_only_256wg"]["ghz"],
+                                   "clock_ghz_mfma_decode_lds_256wg": probe["mfma_decode_lds_256wg"]["ghz"],
+                                   "mfma_only_probe_TFLOPs": probe["mfma_only_256wg"]["TFLOPs"]}},
+        "clock_probe": probe,
         "setup_s": t_build,
     }
     if not args.no_cpu_baseline:
@@ -438,7 +459,8 @@ def run_attention(args, t12, torch, dev):
     }
 
 
-def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(2, 4, 8, 16, 64, 256), iters=50):
+def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(2, 4, 8, 16, 32, 64, 128, 256), iters=50,
+                   yardstick=True):
     """decode+GEMM per layer shape: for each B, each of QKV (3 segments), O, gate|up
     (2 segments), down is timed over `n_rot` distinct weight copies in rotation, so that neither L2 nor
     the 256 MB last-level cache holds a tensor between launches.  weight_of(copy, which) -> (segment, K, P).
@@ -448,6 +470,37 @@ def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(2, 4
     out = {}
     groups = [(0, 1, 2), (3,), (4, 5), (6,)]
     names = ["qkv", "o", "gate_up", "down"]
+
+    def median_us(fn, launches):
+        for _ in range(5):
+            fn()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+        torch.cuda.synchronize()
+        for e0, e1 in evs:
+            e0.record(cur)
+            fn()
+            e1.record(cur)
+        torch.cuda.synchronize()
+        rounds = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+        return rounds[len(rounds) // 2] * 1e3 / launches
+
+    if yardstick:
+        # A yardstick off the product path: the vendor library's plain bf16 GEMM (torch.nn.functional.linear ->
+        # hipBLASLt) on the same shapes with UNCOMPRESSED bf16 weights (2 bytes per weight from HBM, no decode), three
+        # rotating copies, same timing.  It shows what a tuned dense kernel reaches on these skinny problems on this chip.
+        for name, grp in zip(names, groups):
+            M = sum(weight_of(0, w)[0].M for w in grp)
+            K = weight_of(0, grp[0])[1]
+            ws = [(torch.randn((M, K), generator=g, device=dev) * 0.02).to(torch.bfloat16) for _ in range(n_rot)]
+            for B in batches:
+                if B < 16:
+                    continue
+                x = torch.randn((B, K), generator=g, device=dev).to(torch.bfloat16)
+                us = median_us(lambda: [torch.nn.functional.linear(x, w) for w in ws], n_rot)
+                out["vendor_bf16_%s_b%d" % (name, B)] = {"us": round(us, 2), "mfma_frac": round(2.0 * M * K * B / us / 1e6 / 2500.0, 4),
+                                                          "weight_GBps": round(2.0 * M * K / us / 1e3, 1)}
+            del ws
+        torch.cuda.empty_cache()
     for B in batches:
         xs = {K: torch.randn((B, K), generator=g, device=dev).to(torch.bfloat16) for K in (cfg["n_embd"], cfg["n_ff"])}
         obuf = torch.empty((B, 2 * cfg["n_ff"]), dtype=torch.float32, device=dev)
@@ -517,11 +570,32 @@ def gemm_layer_leg(t12, torch, dev, cfg, weight_of, n_rot, cur, g, batches=(2, 4
     return out
 
 
+def clock_probe(t12):
+    """Shader clock and MFMA rate under load (t12_probe_clock): MFMA only, and MFMA with the decode / LDS work of a
+    decode+GEMM stage beside it, on 64 / 128 / 256 workgroups of eight waves.  The published 2.5 PFLOP/s is priced at
+    2.4 GHz; the chip lowers its clock with the activity of the launch."""
+    import ctypes as C
+    out = {}
+    for mix, name in ((0, "mfma_only"), (1, "mfma_decode_lds")):
+        for wgs in (64, 128, 256):
+            ghz, tf = C.c_double(), C.c_double()
+            rc = t12.lib.t12_probe_clock(wgs, 20000, mix, C.byref(ghz), C.byref(tf), t12.current_stream())
+            if rc:
+                t12.check(rc, "t12_probe_clock")
+            out["%s_%dwg" % (name, wgs)] = {"ghz": round(ghz.value, 3), "TFLOPs": round(tf.value, 1)}
+    return out
+
+
 def gemm_b256_roofline(layers):
     names = ("qkv", "o", "gate_up", "down")
     us = sum(layers["%s_b256" % k]["us"] for k in names)
     fl = sum(layers["%s_b256" % k]["flops"] for k in names)
-    return {"bound": "mfma", "achieved": fl / us / 1e6, "peak": 2500.0, "unit": "TFLOP/s", "frac": fl / us / 1e6 / 2500.0,
+    extra = {}
+    if "vendor_bf16_gate_up_b256" in layers:
+        vus = sum(layers["vendor_bf16_%s_b256" % k]["us"] for k in names)
+        extra = {"vendor_bf16_frac": fl / vus / 1e6 / 2500.0, "vendor_bf16_us_per_step": vus,
+                 "vendor_bf16_gate_up_frac": layers["vendor_bf16_gate_up_b256"]["mfma_frac"]}
+    return {**extra, "bound": "mfma", "achieved": fl / us / 1e6, "peak": 2500.0, "unit": "TFLOP/s", "frac": fl / us / 1e6 / 2500.0,
             "traffic": None, "kernel": "gemm_mfma_kernel, QKV + O + gate|up + down at B=256", "flops_per_step": fl,
             "us_per_step": us, "gate_up_frac": layers["gate_up_b256"]["mfma_frac"],
             # the same four products as the engine's layer issues them: gate|up with SiLU*mul in its epilogue
@@ -582,8 +656,10 @@ def run_tokenizer(args, t12):
 
 
 def run_gemm_layers(args, t12, torch, dev):
-    """The four Llama-3.1-8B linear-layer shapes through the fused decode+GEMM at B = 2, 4, 8, 16, 64, 256 on three
-    rotating weight copies; one step = the four layer GEMMs of one decoder layer at B = 256."""
+    """The four Llama-3.1-8B linear-layer shapes through the fused decode+GEMM at B = 2 .. 256 on three rotating weight
+    copies, the vendor library's plain bf16 GEMM on the same shapes as a yardstick, the same launch on half and a
+    quarter of its row tiles, and the shader clock under load; one step = the four layer GEMMs of one decoder layer at
+    B = 256."""
     cfg = dict(LLAMA8B)
     n, ff = cfg["n_embd"], cfg["n_ff"]
     kv = cfg["n_head_kv"] * (n // cfg["n_head"])
@@ -603,6 +679,36 @@ def run_gemm_layers(args, t12, torch, dev):
     if args.calibrate:
         calibration_copy(torch, dev)
     layers = gemm_layer_leg(t12, torch, dev, cfg, weight_of, 3, cur, g, iters=max(args.steps, 50))
+    # gate|up at B = 256 on the first half and the first quarter of the rows (112 / 56 row tiles instead of 224: half and
+    # a quarter of the work on half and a quarter of the CUs).  Were the launch bound by what one workgroup does, the time
+    # would not change; it drops, because the chip clocks higher with fewer CUs busy.
+    occupancy = {}
+    xs = torch.randn((256, n), generator=g, device=dev).to(torch.bfloat16)
+    obuf = torch.empty((256, 2 * ff), dtype=torch.float32, device=dev)
+    for frac in (1, 2, 4):
+        calls = []
+        for copy in range(3):
+            segs = []
+            for j, which in enumerate((4, 5)):
+                seg, K, P = weight_of(copy, which)
+                seg.M = seg.M // frac
+                seg.out = obuf.data_ptr() + 4 * j * seg.M
+                segs.append(seg)
+            calls.append(t12._seg_array(segs))
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(50)]
+        for it in range(55):
+            if it >= 5:
+                evs[it - 5][0].record(cur)
+            for sa in calls:
+                rc = t12.lib.t12_gemm(sa, 2, xs.data_ptr(), n, 2 * ff, n, 256, cur.cuda_stream)
+                if rc:
+                    t12.check(rc, "t12_gemm")
+            if it >= 5:
+                evs[it - 5][1].record(cur)
+        torch.cuda.synchronize()
+        rounds = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+        occupancy["gate_up_b256_rows_1_%d" % frac] = {"row_tiles": 2 * (ff // frac) // 128, "us": round(rounds[25] * 1e3 / 3, 2)}
+    probe = clock_probe(t12)
     us256 = sum(layers["%s_b256" % k]["us"] for k in ("qkv", "o", "gate_up", "down"))
     fl256 = sum(layers["%s_b256" % k]["flops"] for k in ("qkv", "o", "gate_up", "down"))
     gu = layers["gate_up_b256"]
@@ -612,12 +718,17 @@ def run_gemm_layers(args, t12, torch, dev):
         "ms_per_step": us256 / 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "gemm_layers: QKV 4096->6144 (3 segments), O 4096->4096, gate|up 4096->28672 (2 segments), "
-                               "down 14336->4096; N(0,0.02)+3e-4 outliers; B in {2,4,8,16,64,256}; 3 rotating weight copies"},
+                               "down 14336->4096; N(0,0.02)+3e-4 outliers; B in {2,4,8,16,32,64,128,256}; 3 rotating weight copies"},
         "layers": layers,
+        "occupancy_probe": occupancy,
+        "clock_probe": probe,
         "roofline": {"bound": "mfma", "achieved": gu["TFLOPs"], "peak": 2500.0, "unit": "TFLOP/s",
-                     "frac": gu["TFLOPs"] / 2500.0, "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get("gemm_gate_up_b256"),
+                     "frac": gu["TFLOPs"] / 2500.0, "traffic": measured_traffic("gemm_gate_up_b256"),
                      "kernel": "gemm_mfma_kernel<4,2,2,2> on gate|up at B=256", "flops_per_launch": gu["flops"],
-                     "us_per_launch": gu["us"]},
+                     "us_per_launch": gu["us"],
+                     "vendor_bf16_gemm_frac": layers.get("vendor_bf16_gate_up_b256", {}).get("mfma_frac"),
+                     "clock_ghz_mfma_decode_lds_256wg": probe["mfma_decode_lds_256wg"]["ghz"],
+                     "clock_ghz_mfma_only_256wg": probe["mfma_only_256wg"]["ghz"]},
         "setup_s": t_build,
     }
 
@@ -712,6 +823,46 @@ def main():
     ms = e0.elapsed_time(e1) / args.steps          # HIP events on the launch stream
     ms_step = max(ms, wall_ms)
 
+    # ---- what could fill the time between two launches (about 3 us per launch, a fifth of the stack)?
+    #   same_tensor: one launch repeated on ONE weight copy -- were the last-level cache to serve it, the repeat would beat
+    #                the rotating stack's rate for that shape;
+    #   two_streams: two independent passes of the stack interleaved on two streams -- the rate when a second, independent
+    #                launch is there to run in the gaps (a decode step has none: each launch reads the previous one's output)
+    def rate(fn, nbytes, reps):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return nbytes * reps / (a.elapsed_time(b) * 1e-3) / 1e9
+
+    probes = {}
+    for idx, name in ((0, "qkv"), (1, "o"), (2, "gate_up"), (3, "down")):
+        segs, n, act, K = seg_tabs[idx]
+        nb = sum(1.5 * t.M * t.K for t in launches[idx][0])
+
+        def same():
+            for _ in range(20):
+                t12.lib.t12_gemv(segs, n, act, K, stream)
+        probes["same_tensor_%s_GBps" % name] = round(rate(same, 20 * nb, 5), 1)
+    side = torch.cuda.Stream()
+    outs2 = [[torch.empty(t.M, dtype=torch.float32, device=dev) for t in tensors] for tensors, _ in launches]
+    seg_tabs2 = [(t12._seg_array([t.segment(o) for t, o in zip(tensors, out)]), len(tensors), acts[key].data_ptr(),
+                  tensors[0].K) for (tensors, key), out in zip(launches, outs2)]
+    plane_all = sum(1.5 * t.M * t.K for tensors, _ in launches for t in tensors)
+
+    def two():
+        for a_, b_ in zip(seg_tabs, seg_tabs2):
+            t12.lib.t12_gemv(a_[0], a_[1], a_[2], a_[3], stream)
+            t12.lib.t12_gemv(b_[0], b_[1], b_[2], b_[3], side.cuda_stream)
+        torch.cuda.current_stream().wait_stream(side)
+    side.wait_stream(torch.cuda.current_stream())
+    probes["two_streams_two_passes_GBps"] = round(rate(two, 2 * plane_all, 3), 1)
+
     n_launch = len(launches)
     alg_bytes = sum(algorithmic_bytes(t) for tensors, _ in launches for t in tensors)
     plane_bytes = sum(1.5 * t.M * t.K for tensors, _ in launches for t in tensors)
@@ -727,10 +878,10 @@ def main():
                    "compressed_GB_per_step": plane_bytes / 1e9, "escape_fraction":
                        sum(t.P for tensors, _ in launches for t in tensors) / n_weights},
         "gemv_compressed_GBps": plane_bytes / (ms * 1e-3) / 1e9,
+        "gap_probes": probes,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload)
-                     if cfg["n_layer"] == LLAMA8B["n_layer"] else None,
+                     "traffic": measured_traffic(args.workload) if cfg["n_layer"] == LLAMA8B["n_layer"] else None,
                      "kernel": "gemv_stream_kernel", "bytes_per_launch": alg_bytes / n_launch,
                      "us_per_launch": ms * 1e3 / n_launch},
         "setup_s": t_build,

@@ -66,6 +66,15 @@ const char* t12_last_error(void);      /* text of the last failure on this threa
  * host this way, without a DMA-engine hand-over in the middle of the stream).  No counterpart in the reference. */
 int t12_util_copy_i32(void* dst, const void* src, int n, void* stream);
 
+/* Measurement aid, no counterpart in the reference: the shader clock under load.  Runs `workgroups` workgroups of
+ * eight waves, each wave `iters` rounds of four independent v_mfma_f32_32x32x16_bf16 on pseudo-random operands
+ * (mix = 0), or the same with what a decode+GEMM stage adds per round (mix = 1: two packed 8-weight decodes, two
+ * 16-byte LDS writes, four 16-byte LDS reads), and reports the clock the waves saw (shader-clock counter against
+ * the constant 100 MHz counter, mean over the workgroups, GHz) and the dense bf16 MFMA rate of the launch (TFLOP/s).
+ * Synchronous.  The published 2.5 PFLOP/s is 256 CUs x 4 SIMDs x 1024 flop/clk at 2.4 GHz; bench.py prints the
+ * measured clock beside the MFMA roofline. */
+int t12_probe_clock(int workgroups, int iters, int mix, double* ghz, double* tflops, void* stream);
+
 /* ---- (a) decode-GEMV, one activation vector ------------------------------
  * out_s[m] = sum_k dec(W_s[m,k]) * x[k] for every segment s, escapes exact.
  * Replaces launch_split12_v2_async (decompress_v2.hip:530) +
