@@ -199,7 +199,11 @@ int t12_gemm_noalloc(const T12Segment* segs, int nseg, const void* act_bf16, int
 
 /* The library keeps device buffers per (device, stream): K-split partial sums of t12_gemm / _deferred / _grouped, argmax
  * partials and context-split buffers of the glue launchers.  t12_release_stream waits for the stream and frees those of
- * (current device, stream); call it before destroying a stream (free_inference_state does).  No counterpart in the
+ * (current device, stream); call it before destroying a stream (free_inference_state does).  A launch that needs a
+ * larger buffer than any before it on its stream calls hipMalloc once (sizes double, so this happens a few times per
+ * stream) and keeps the outgrown buffer until t12_release_stream rather than freeing it, so no launch call waits for
+ * the device; only when that hipMalloc fails are the outgrown buffers freed inside the call (a device-wide wait)
+ * before one more attempt.  Callers that cannot allocate at all use t12_gemm_noalloc.  No counterpart in the
  * reference, which keeps no such buffers. */
 int t12_release_stream(void* stream);
 

@@ -207,6 +207,9 @@ InferenceState* create_inference_state(Model* model, int batch_size, int max_seq
     const char* nofuse = getenv("TURBO_NO_FUSE");     // debugging aid: one kernel per reference kernel
     impl->fused_b1 = !(nofuse && nofuse[0] == '1');   // confirmed against the tensors at the first forward
     impl->no_pipeline = getenv("TURBO_NO_PIPELINE") != nullptr;   // the reference's order: sample, wait, forward
+    // the pipelined decode loop keeps the logits of the previous step while the next forward overwrites
+    // state->logits: its second buffer belongs to the state's memory budget, not to the first decode call
+    if (!impl->no_pipeline) impl->logits_alt = fbuf(bs * n_vocab);
     s->impl = impl;
     init_sampler(batch_size);
     return s;
@@ -668,8 +671,6 @@ std::vector<int> decode_loop(InferenceState* state, int max_tokens, int stop_a, 
         }
         return output;
     }
-    if (!impl->logits_alt)
-        check_gpu(hipMalloc((void**)&impl->logits_alt, (size_t)bs * n_vocab * sizeof(float)), "hipMalloc");
     for (int i = 0; i < 2; i++) {
         if (!impl->h_tokens[i]) check_gpu(hipHostMalloc((void**)&impl->h_tokens[i], bs * sizeof(int)), "hipHostMalloc");
         if (!impl->sampled[i]) check_gpu(hipEventCreateWithFlags(&impl->sampled[i], hipEventDisableTiming), "hipEventCreate");

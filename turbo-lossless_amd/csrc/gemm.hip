@@ -38,6 +38,7 @@
 #include <map>
 #include <mutex>
 #include <utility>
+#include <vector>
 
 #include "t12_device.h"
 #include "t12_host.h"
@@ -928,8 +929,9 @@ __global__ __launch_bounds__(512) void gemm_rows_kernel(const GemmParams p)
 // ---- workspace for the K-split partial sums: one per (device, stream), grown on demand.  Launches on different
 //      streams may overlap, so they must not share partial sums; launches on one stream are ordered.
 struct Workspace {
-    float* ptr;
-    size_t bytes;
+    float* ptr = nullptr;
+    size_t bytes = 0;
+    std::vector<float*> retired;      // outgrown buffers: kernels already in the stream may still write them
 };
 std::mutex g_ws_mutex;
 std::map<std::pair<int, hipStream_t>, Workspace> g_ws;
@@ -941,23 +943,34 @@ float* workspace(size_t bytes, hipStream_t st)
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     Workspace& w = g_ws[{dev, st}];
     if (w.bytes < bytes) {
-        // grows geometrically, in whole MiB: a caller whose shapes grow step by step pays the allocation (a device-wide
-        // wait) a few times, not once per shape
+        // Grows geometrically, in whole MiB, so a caller whose shapes grow step by step allocates a few times and the
+        // outgrown buffers together stay below the live one.  They are kept until release_workspace: hipFree waits
+        // for the whole device, which a launch call must not do.
         size_t want = bytes > 2 * w.bytes ? bytes : 2 * w.bytes;
         want = (want + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
-        if (w.ptr) (void)hipFree(w.ptr);          // waits for the device: nothing still reads the old buffer
-        w.ptr = nullptr;
-        w.bytes = 0;
-        if (hipMalloc((void**)&w.ptr, want) != hipSuccess) {
+        float* fresh = nullptr;
+        if (hipMalloc((void**)&fresh, want) != hipSuccess) {
+            (void)hipGetLastError();
+            // short of memory: give the outgrown buffers back (this waits for the device) and ask for the exact size
+            for (float* r : w.retired) (void)hipFree(r);
+            w.retired.clear();
+            if (w.ptr) (void)hipFree(w.ptr);
+            w.ptr = nullptr;
+            w.bytes = 0;
             want = bytes;
-            if (hipMalloc((void**)&w.ptr, want) != hipSuccess) return nullptr;
+            if (hipMalloc((void**)&fresh, want) != hipSuccess) {
+                (void)hipGetLastError();
+                return nullptr;
+            }
         }
+        if (w.ptr) w.retired.push_back(w.ptr);
+        w.ptr = fresh;
         w.bytes = want;
     }
     return w.ptr;
 }
 
-// Frees the K-split workspace of (current device, stream).
+// Frees the K-split workspace of (current device, stream), outgrown buffers included.
 void release_workspace(hipStream_t st)
 {
     int dev = 0;
@@ -965,6 +978,7 @@ void release_workspace(hipStream_t st)
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     auto it = g_ws.find({dev, st});
     if (it == g_ws.end()) return;
+    for (float* r : it->second.retired) (void)hipFree(r);
     if (it->second.ptr) (void)hipFree(it->second.ptr);
     g_ws.erase(it);
 }
@@ -1092,10 +1106,11 @@ int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_st
         part->ld = 0;
         part->split_stride = 0;
     }
-    T12_REQUIRE(segs && nseg >= 1 && nseg <= T12_MAX_SEGMENTS, "t12_gemm: nseg must be 1..%d (got %d)",
+    const char* who = static_ws ? "t12_gemm_noalloc" : "t12_gemm";
+    T12_REQUIRE(segs && nseg >= 1 && nseg <= T12_MAX_SEGMENTS, "%s: nseg must be 1..%d (got %d)", who,
                 T12_MAX_SEGMENTS, nseg);
-    T12_REQUIRE(act_bf16 && K >= 1 && B >= 1, "t12_gemm: activations null or K/B < 1 (K=%d B=%d)", K, B);
-    T12_REQUIRE(act_stride >= K, "t12_gemm: act_stride %d < K %d", act_stride, K);
+    T12_REQUIRE(act_bf16 && K >= 1 && B >= 1, "%s: activations null or K/B < 1 (K=%d B=%d)", who, K, B);
+    T12_REQUIRE(act_stride >= K, "%s: act_stride %d < K %d", who, act_stride, K);
     hipStream_t st = (hipStream_t)stream;
     GemmParams p;
     p.nseg = nseg;
@@ -1110,14 +1125,14 @@ int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_st
     int m_total = 0;
     for (int i = 0; i < nseg; i++) {
         const T12Segment& g = segs[i];
-        T12_REQUIRE(g.M >= 1 && g.sm && g.gr && g.out, "t12_gemm: segment %d has M < 1 or a null pointer", i);
-        T12_REQUIRE(!g.row_off || (g.cols && g.correct && g.wrong), "t12_gemm: segment %d: row_off without lists", i);
-        T12_REQUIRE(g.base_exp >= -1 && g.base_exp <= 254, "t12_gemm: segment %d: base_exp %d out of range", i,
+        T12_REQUIRE(g.M >= 1 && g.sm && g.gr && g.out, "%s: segment %d has M < 1 or a null pointer", who, i);
+        T12_REQUIRE(!g.row_off || (g.cols && g.correct && g.wrong), "%s: segment %d: row_off without lists", who, i);
+        T12_REQUIRE(g.base_exp >= -1 && g.base_exp <= 254, "%s: segment %d: base_exp %d out of range", who, i,
                     g.base_exp);
         if (g.base_exp < 0 || g.base_exp > 240) fast = false;
         p.seg[i] = g;
         if (p.seg[i].out_stride == 0) p.seg[i].out_stride = out_stride;
-        T12_REQUIRE(p.seg[i].out_stride >= g.M, "t12_gemm: out_stride %d < M %d of segment %d", p.seg[i].out_stride,
+        T12_REQUIRE(p.seg[i].out_stride >= g.M, "%s: out_stride %d < M %d of segment %d", who, p.seg[i].out_stride,
                     g.M, i);
         p.seg_row0[i] = m_total;
         p.seg_act[i] = p.act;
@@ -1213,7 +1228,7 @@ int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_st
     } else if (ks > 1) {
         p.ws = workspace((size_t)ks * B * m_total * sizeof(float), st);
         if (!p.ws) {
-            t12_set_error("t12_gemm: cannot allocate %zu bytes of K-split workspace",
+            t12_set_error("%s: cannot allocate %zu bytes of K-split workspace", who,
                           (size_t)ks * B * m_total * sizeof(float));
             return T12_ELAUNCH;
         }
