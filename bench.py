@@ -679,35 +679,6 @@ def run_gemm_layers(args, t12, torch, dev):
     if args.calibrate:
         calibration_copy(torch, dev)
     layers = gemm_layer_leg(t12, torch, dev, cfg, weight_of, 3, cur, g, iters=max(args.steps, 50))
-    # gate|up at B = 256 on the first half and the first quarter of the rows (112 / 56 row tiles instead of 224: half and
-    # a quarter of the work on half and a quarter of the CUs).  Were the launch bound by what one workgroup does, the time
-    # would not change; it drops, because the chip clocks higher with fewer CUs busy.
-    occupancy = {}
-    xs = torch.randn((256, n), generator=g, device=dev).to(torch.bfloat16)
-    obuf = torch.empty((256, 2 * ff), dtype=torch.float32, device=dev)
-    for frac in (1, 2, 4):
-        calls = []
-        for copy in range(3):
-            segs = []
-            for j, which in enumerate((4, 5)):
-                seg, K, P = weight_of(copy, which)
-                seg.M = seg.M // frac
-                seg.out = obuf.data_ptr() + 4 * j * seg.M
-                segs.append(seg)
-            calls.append(t12._seg_array(segs))
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(50)]
-        for it in range(55):
-            if it >= 5:
-                evs[it - 5][0].record(cur)
-            for sa in calls:
-                rc = t12.lib.t12_gemm(sa, 2, xs.data_ptr(), n, 2 * ff, n, 256, cur.cuda_stream)
-                if rc:
-                    t12.check(rc, "t12_gemm")
-            if it >= 5:
-                evs[it - 5][1].record(cur)
-        torch.cuda.synchronize()
-        rounds = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
-        occupancy["gate_up_b256_rows_1_%d" % frac] = {"row_tiles": 2 * (ff // frac) // 128, "us": round(rounds[25] * 1e3 / 3, 2)}
     probe = clock_probe(t12)
     us256 = sum(layers["%s_b256" % k]["us"] for k in ("qkv", "o", "gate_up", "down"))
     fl256 = sum(layers["%s_b256" % k]["flops"] for k in ("qkv", "o", "gate_up", "down"))
@@ -720,7 +691,6 @@ def run_gemm_layers(args, t12, torch, dev):
         "config": {"workload": "gemm_layers: QKV 4096->6144 (3 segments), O 4096->4096, gate|up 4096->28672 (2 segments), "
                                "down 14336->4096; N(0,0.02)+3e-4 outliers; B in {2,4,8,16,32,64,128,256}; 3 rotating weight copies"},
         "layers": layers,
-        "occupancy_probe": occupancy,
         "clock_probe": probe,
         "roofline": {"bound": "mfma", "achieved": gu["TFLOPs"], "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": gu["TFLOPs"] / 2500.0, "traffic": measured_traffic("gemm_gate_up_b256"),
@@ -752,6 +722,10 @@ def main():
     ap.add_argument("--no-batch256", dest="batch256", action="store_false")
     ap.add_argument("--layers", type=int, default=LLAMA8B["n_layer"], help="debug: fewer layers (invalid as a result)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--probes", action="store_true",
+                    help="gemv_stack_b1: after the timed steps also measure what could fill the time between launches (one "
+                         "tensor launched repeatedly, two independent passes on two streams, a chain of idle kernels); "
+                         "off by default so that a kernel trace of the workload holds the stack's launches only")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one plain 1 GiB copy kernel (a torch tensor copy) before the steps: the known-size "
                          "yardstick for the profiler's FETCH_SIZE / WRITE_SIZE counters")
@@ -823,45 +797,56 @@ def main():
     ms = e0.elapsed_time(e1) / args.steps          # HIP events on the launch stream
     ms_step = max(ms, wall_ms)
 
-    # ---- what could fill the time between two launches (about 3 us per launch, a fifth of the stack)?
-    #   same_tensor: one launch repeated on ONE weight copy -- were the last-level cache to serve it, the repeat would beat
-    #                the rotating stack's rate for that shape;
-    #   two_streams: two independent passes of the stack interleaved on two streams -- the rate when a second, independent
-    #                launch is there to run in the gaps (a decode step has none: each launch reads the previous one's output)
-    def rate(fn, nbytes, reps):
-        for _ in range(2):
-            fn()
-        torch.cuda.synchronize()
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        for _ in range(reps):
-            fn()
-        b.record()
-        torch.cuda.synchronize()
-        return nbytes * reps / (a.elapsed_time(b) * 1e-3) / 1e9
+    probes = None
+    if args.probes:
+        # ---- what could fill the time between two launches (about 3 us per launch, a fifth of the stack)?
+        #   same_tensor: one launch repeated on ONE weight copy -- were the last-level cache to serve it, the repeat would beat
+        #                the rotating stack's rate for that shape;
+        #   two_streams: two independent passes of the stack interleaved on two streams -- the rate when a second, independent
+        #                launch is there to run in the gaps (a decode step has none: each launch reads the previous one's output)
+        def rate(fn, nbytes, reps):
+            for _ in range(2):
+                fn()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(reps):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            return nbytes * reps / (a.elapsed_time(b) * 1e-3) / 1e9
 
-    probes = {}
-    for idx, name in ((0, "qkv"), (1, "o"), (2, "gate_up"), (3, "down")):
-        segs, n, act, K = seg_tabs[idx]
-        nb = sum(1.5 * t.M * t.K for t in launches[idx][0])
+        probes = {}
+        for idx, name in ((0, "qkv"), (1, "o"), (2, "gate_up"), (3, "down")):
+            segs, n, act, K = seg_tabs[idx]
+            nb = sum(1.5 * t.M * t.K for t in launches[idx][0])
 
-        def same():
-            for _ in range(20):
-                t12.lib.t12_gemv(segs, n, act, K, stream)
-        probes["same_tensor_%s_GBps" % name] = round(rate(same, 20 * nb, 5), 1)
-    side = torch.cuda.Stream()
-    outs2 = [[torch.empty(t.M, dtype=torch.float32, device=dev) for t in tensors] for tensors, _ in launches]
-    seg_tabs2 = [(t12._seg_array([t.segment(o) for t, o in zip(tensors, out)]), len(tensors), acts[key].data_ptr(),
-                  tensors[0].K) for (tensors, key), out in zip(launches, outs2)]
-    plane_all = sum(1.5 * t.M * t.K for tensors, _ in launches for t in tensors)
+            def same():
+                for _ in range(20):
+                    t12.lib.t12_gemv(segs, n, act, K, stream)
+            probes["same_tensor_%s_GBps" % name] = round(rate(same, 20 * nb, 5), 1)
+        side = torch.cuda.Stream()
+        outs2 = [[torch.empty(t.M, dtype=torch.float32, device=dev) for t in tensors] for tensors, _ in launches]
+        seg_tabs2 = [(t12._seg_array([t.segment(o) for t, o in zip(tensors, out)]), len(tensors), acts[key].data_ptr(),
+                      tensors[0].K) for (tensors, key), out in zip(launches, outs2)]
+        plane_all = sum(1.5 * t.M * t.K for tensors, _ in launches for t in tensors)
 
-    def two():
-        for a_, b_ in zip(seg_tabs, seg_tabs2):
-            t12.lib.t12_gemv(a_[0], a_[1], a_[2], a_[3], stream)
-            t12.lib.t12_gemv(b_[0], b_[1], b_[2], b_[3], side.cuda_stream)
-        torch.cuda.current_stream().wait_stream(side)
-    side.wait_stream(torch.cuda.current_stream())
-    probes["two_streams_two_passes_GBps"] = round(rate(two, 2 * plane_all, 3), 1)
+        def two():
+            for a_, b_ in zip(seg_tabs, seg_tabs2):
+                t12.lib.t12_gemv(a_[0], a_[1], a_[2], a_[3], stream)
+                t12.lib.t12_gemv(b_[0], b_[1], b_[2], b_[3], side.cuda_stream)
+            torch.cuda.current_stream().wait_stream(side)
+        side.wait_stream(torch.cuda.current_stream())
+        probes["two_streams_two_passes_GBps"] = round(rate(two, 2 * plane_all, 3), 1)
+        #   launch interval: a chain of kernels that do nothing, in stream order (what every dependent launch of a decode step
+        #   pays at least) and with the ordering between them lifted (hipExtAnyOrderLaunch: no option for dependent launches)
+        import ctypes as C
+        for key, any_order in (("idle_kernel_chain_us_per_launch", 0), ("idle_kernel_chain_any_order_us_per_launch", 1)):
+            us = C.c_double()
+            rc = t12.lib.t12_probe_launch_gap(2000, any_order, C.byref(us), stream)
+            if rc:
+                t12.check(rc, "t12_probe_launch_gap")
+            probes[key] = round(us.value, 2)
 
     n_launch = len(launches)
     alg_bytes = sum(algorithmic_bytes(t) for tensors, _ in launches for t in tensors)

@@ -75,6 +75,15 @@ int t12_util_copy_i32(void* dst, const void* src, int n, void* stream);
  * measured clock beside the MFMA roofline. */
 int t12_probe_clock(int workgroups, int iters, int mix, double* ghz, double* tflops, void* stream);
 
+/* Measurement aid, no counterpart in the reference: the time per launch (us) of a chain of `launches` one-wave
+ * kernels that do nothing, on `stream`, as the GPU paces them (a first kernel holds the stream for 4 us per launch
+ * while the host enqueues the chain; the clock runs from its end).  any_order = 0: ordinary stream order (each kernel waits for the one
+ * before it), the floor under a chain of dependent launches such as the B = 1 decode step.  any_order = 1: the
+ * launches carry hipExtAnyOrderLaunch, which lifts the ordering between them -- such kernels overlap, so it is
+ * no option for launches that read what their predecessor wrote; the difference is what the ordering costs.
+ * Synchronous. */
+int t12_probe_launch_gap(int launches, int any_order, double* us_per_launch, void* stream);
+
 /* ---- (a) decode-GEMV, one activation vector ------------------------------
  * out_s[m] = sum_k dec(W_s[m,k]) * x[k] for every segment s, escapes exact.
  * Replaces launch_split12_v2_async (decompress_v2.hip:530) +

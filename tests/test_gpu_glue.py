@@ -444,3 +444,19 @@ def test_context_split_equals_single_pass(t12, oracle, nh, nkv, hd, B, pos):
         assert np.abs(want[0] - wantr).max() <= 2e-2 * np.abs(wantr).max()
     finally:
         t12.lib.t12_tune_attention(1)
+
+
+def test_measurement_aids_return_plausible_figures(t12):
+    """t12_probe_clock and t12_probe_launch_gap (no counterpart in the reference): they run, return T12_OK and figures
+    a gfx950 can have; bad operands are refused on the host."""
+    import ctypes as C
+    ghz, tf, us = C.c_double(), C.c_double(), C.c_double()
+    assert t12.lib.t12_probe_clock(64, 200, 0, C.byref(ghz), C.byref(tf), st(t12)) == 0
+    assert 0.5 < ghz.value < 3.0 and 10.0 < tf.value < 2500.0, (ghz.value, tf.value)
+    assert t12.lib.t12_probe_clock(64, 200, 1, C.byref(ghz), C.byref(tf), st(t12)) == 0
+    assert 0.5 < ghz.value < 3.0 and 1.0 < tf.value < 2500.0, (ghz.value, tf.value)
+    for any_order in (0, 1):
+        assert t12.lib.t12_probe_launch_gap(200, any_order, C.byref(us), st(t12)) == 0
+        assert 0.2 < us.value < 50.0, us.value
+    assert t12.lib.t12_probe_launch_gap(0, 0, C.byref(us), st(t12)) < 0
+    assert t12.lib.t12_probe_clock(0, 1, 0, C.byref(ghz), C.byref(tf), st(t12)) < 0

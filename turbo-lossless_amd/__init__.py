@@ -143,6 +143,7 @@ _SIGS = {
     "t12_moe_ffn": (_i, [C.POINTER(MoeExpert), _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, C.c_size_t, _vp, _i, _vp]),
     "t12_moe_status": (_i, [_vp, _vp]),
     "t12_probe_clock": (_i, [_i, _i, _i, C.POINTER(C.c_double), C.POINTER(C.c_double), _vp]),
+    "t12_probe_launch_gap": (_i, [_i, _i, C.POINTER(C.c_double), _vp]),
     "t12_gemm_swiglu": (_i, [C.POINTER(Segment), C.POINTER(Segment), _vp, _i, _i, _i, _vp, _i, _vp]),
     "t12_gemm_deferred": (_i, [C.POINTER(Segment), _i, _vp, _i, _i, _i, _i, C.POINTER(GemmPartials), _vp]),
     "launch_sum_add_rms_norm_bf16_batch": (None, [_vp, _vp, _i, C.c_size_t, _i, _vp, _vp, _vp, _i, C.c_float, _i, _vp]),

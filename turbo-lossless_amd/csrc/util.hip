@@ -1,5 +1,7 @@
 // Small utility kernels of the engine.
 
+#include <hip/hip_ext.h>
+
 #include <vector>
 
 #include "t12_device.h"
@@ -11,6 +13,18 @@ __global__ void copy_i32_kernel(int* __restrict__ dst, const int* __restrict__ s
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) dst[i] = src[i];
+}
+
+// A kernel that does nothing (hold_ticks == 0): the launch-interval probe below times a chain of them.  With
+// hold_ticks > 0 its one wave waits that many ticks of the constant 100 MHz counter first (bounded by an iteration
+// count as well): it holds the stream while the host enqueues the chain behind it.
+__global__ void idle_kernel(int hold_ticks, int* __restrict__ sink)
+{
+    if (hold_ticks > 0) {
+        const long long t0 = wall_clock64();
+        for (int guard = 0; guard < (1 << 24) && wall_clock64() - t0 < hold_ticks; guard++) __builtin_amdgcn_s_sleep(16);
+    }
+    if (sink && threadIdx.x == 0xFFFF) *sink = 0;      // never true
 }
 
 // Shader-clock probe: what the chip clocks at under a given instruction mix.  Every workgroup (eight waves) runs
@@ -127,6 +141,49 @@ int t12_probe_clock(int workgroups, int iters, int mix, double* ghz, double* tfl
     }
     *ghz = sum_ghz / workgroups;
     *tflops = max_ns > 0.0 ? 2.0 * 32 * 32 * 16 * 4.0 * 8 * (double)iters * workgroups / max_ns / 1e3 : 0.0;
+    return T12_OK;
+}
+
+// Measurement aid (no counterpart in the reference): the interval between consecutive kernels of one stream, as
+// the GPU's command processor paces them (the host's enqueue cost is kept out: a first kernel holds the stream
+// for 4 us per launch while the host enqueues the whole chain behind it, and the clock runs from its end).
+// Reports the time per launch of `launches` one-wave kernels that do nothing (us).  any_order = 0: the ordinary
+// stream order, every kernel waits for the one before it -- the floor under any chain of dependent launches such
+// as the B = 1 decode step.  any_order = 1: the launches carry hipExtAnyOrderLaunch, which lifts that ordering
+// (such kernels overlap and may start before their predecessor has ended, so no launch whose input another launch
+// of the chain writes may carry it): what the ordering itself costs.  Synchronous; allocates two events.
+int t12_probe_launch_gap(int launches, int any_order, double* us_per_launch, void* stream)
+{
+    T12_REQUIRE(launches >= 1 && launches <= 20000 && us_per_launch, "t12_probe_launch_gap: launches must be 1..20000");
+    hipStream_t st = (hipStream_t)stream;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+        if (e0) (void)hipEventDestroy(e0);
+        t12_set_error("t12_probe_launch_gap: hipEventCreate failed");
+        return T12_ELAUNCH;
+    }
+    const int flags = any_order ? hipExtAnyOrderLaunch : 0;
+    hipError_t e = hipSuccess;
+    for (int rep = 0; rep < 2 && e == hipSuccess; rep++) {            // the first chain warms the queue up
+        hipLaunchKernelGGL(idle_kernel, dim3(1), dim3(64), 0, st, launches * 400, (int*)nullptr);
+        e = hipGetLastError();
+        if (e == hipSuccess) e = hipEventRecord(e0, st);
+        for (int i = 0; i < launches && e == hipSuccess; i++) {
+            hipExtLaunchKernelGGL(idle_kernel, dim3(1), dim3(64), 0, st, nullptr, nullptr, flags, 0, (int*)nullptr);
+            e = hipGetLastError();
+        }
+        if (e == hipSuccess) e = hipEventRecord(e1, st);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+    }
+    float ms = 0.0f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (e != hipSuccess) {
+        t12_set_error("t12_probe_launch_gap: %s", hipGetErrorString(e));
+        return T12_ELAUNCH;
+    }
+    *us_per_launch = (double)ms * 1e3 / launches;
     return T12_OK;
 }
 
