@@ -385,6 +385,21 @@ def run_moe(args, t12, torch, dev):
     ms_step, ms = timed(torch, cur, step, args.steps)
     flops = 2.0 * (T * 2) * 3 * n * ff
     wbytes = 1.5 * E * 3 * n * ff
+    # the same layer on the first 1 / 4 / 16 tokens (a decode step of a MoE model): only the experts those tokens name are
+    # streamed; the rate is over their planes
+    small = {}
+    for Ts in (1, 4, 16):
+        Xs, ids_s, w_s = X[:Ts].contiguous(), ids[:Ts].contiguous(), w[:Ts].contiguous()
+        outs = torch.empty((Ts, n), dtype=torch.float32, device=dev)
+
+        def step_s():
+            layer(Xs, ids_s, w_s, out=outs, stream=cur.cuda_stream)
+        for _ in range(args.warmup):
+            step_s()
+        _, ms_s = timed(torch, cur, step_s, args.steps)
+        active = int(torch.unique(ids_s).numel())
+        small["tokens_%d" % Ts] = {"ms": round(ms_s, 4), "experts_named": active,
+                                   "weight_GBps": round(1.5 * active * 3 * n * ff / ms_s / 1e6, 1)}
     return {
         "metric": "tokens/s through one Mixtral-8x7B-shaped split-12 MoE FFN layer (8 experts, top-2), 256 tokens",
         "value": T * 1e3 / ms_step, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -393,6 +408,7 @@ def run_moe(args, t12, torch, dev):
         "config": {"workload": "moe_mixtral_b256", "experts": E, "top_k": 2, "tokens": T,
                    "tokens_per_expert": torch.bincount(ids.reshape(-1), minlength=E).tolist()},
         "TFLOPs": flops / ms / 1e9, "weight_GBps": wbytes / ms / 1e6,
+        "small_batches": small,
         "roofline": {"bound": "hbm", "achieved": wbytes / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": wbytes / ms / 1e6 / HBM_PEAK_GBS, "traffic": None, "kernel": "gemm_mfma_kernel"},
         "setup_s": t_build,

@@ -178,7 +178,9 @@ int t12_gemm_grouped(const T12Group* groups, int ngroups, int K, void* stream);
  * run as grouped decode+GEMM launches (the SwiGLU activation rounded to bf16 in between, as the engine does,
  * inference.cpp:327; in the gate|up epilogue when the experts receive more than 128 rows each), and the weighted sum
  * is taken in a fixed order.  The call never waits for the stream: the grouped launches read the rows per expert from
- * the routing kernel's tables on the device (one workgroup per row tile, which walks the expert's batch tiles).  An id
+ * the routing kernel's tables on the device (one workgroup per row tile, which walks the expert's batch tiles; with
+ * few rows per expert -- a decode step -- the small-batch kernel that sweeps 16 whole weight rows per workgroup, and
+ * an expert nobody names costs a workgroup's exit).  An id
  * outside 0..E-1 leaves its pair out of the sum and raises a flag that t12_moe_status reads (it waits for the stream).
  * Shapes the tile kernel does not take (n_embd or n_ff not a multiple of 64, base_exp outside 0..240) copy the counts
  * to the host and wait once per call.

@@ -225,9 +225,10 @@ def test_moe_twenty_experts_in_several_grouped_launches(t12, oracle, synth, moe)
 
 
 def test_moe_sixty_four_experts_and_a_shape_sized_on_the_host(t12, oracle, synth, moe):
-    """64 experts (the routing sort's count rows take more than 48 KB of LDS), top-4; and a layer whose widths are not
+    """64 experts (the routing sort's count rows take more than 48 KB of LDS), top-4; 128 experts, the most the call takes
+    (131 KB of count rows), top-3; and a layer whose widths are not
     multiples of 64, which the tile kernel does not take: its launches are sized from a host copy of the counts."""
-    for E, n, n_ff, T, k, seed in [(64, 128, 128, 150, 4, 1500), (3, 96, 160, 40, 2, 1700)]:
+    for E, n, n_ff, T, k, seed in [(64, 128, 128, 150, 4, 1500), (128, 64, 64, 90, 3, 1600), (3, 96, 160, 40, 2, 1700)]:
         packs = [[oracle.pack(synth.weights_llm(m, kk, seed=seed + 3 * e + j, p_outlier=1e-3))
                   for j, (m, kk) in enumerate([(n_ff, n), (n_ff, n), (n, n_ff)])] for e in range(E)]
         layer = moe.MoeLayer([moe.Expert(*[t12.DeviceTensor12.from_packed(p, dev()) for p in ps]) for ps in packs])
@@ -245,3 +246,35 @@ def test_moe_sixty_four_experts_and_a_shape_sized_on_the_host(t12, oracle, synth
             a = oracle.silu_mul_bf16(oracle.gemm(packs[e][0], X[rows]), oracle.gemm(packs[e][1], X[rows]))
             ref[rows] += w_h[rows, slots][:, None].astype(np.float64) * oracle.gemm(packs[e][2], a)
         assert rel_err(got, ref) < 1e-4, (E, n)
+
+
+def test_moe_few_rows_per_expert_and_one_expert_above_sixteen(t12, oracle, synth, moe):
+    """Few (token, expert) pairs per expert on average: the layer takes the kernel that sweeps whole rows and reads each
+    expert's row count on the device; experts nobody names cost nothing, and an expert that, against the odds, gets
+    more than 16 rows (every token names expert 3 here) is swept once per 16 rows."""
+    E, n, n_ff, seed = 16, 128, 256, 2300
+    packs = [[oracle.pack(synth.weights_llm(m, kk, seed=seed + 3 * e + j, p_outlier=1e-3))
+              for j, (m, kk) in enumerate([(n_ff, n), (n_ff, n), (n, n_ff)])] for e in range(E)]
+    layer = moe.MoeLayer([moe.Expert(*[t12.DeviceTensor12.from_packed(p, dev()) for p in ps]) for ps in packs])
+    rng = np.random.default_rng(seed)
+    cases = []
+    T = 24
+    cases.append((T, np.full((T, 1), 3, np.int32)))                                   # one expert, 24 rows
+    ids = np.stack([np.array([3, 1 + rng.integers(0, 2) * 8]) for _ in range(17)]).astype(np.int32)
+    cases.append((17, ids))                                                            # 17 rows on expert 3, the rest on 1 / 9
+    cases.append((1, np.array([[5, 11]], np.int32)))                                   # a single token, top-2
+    cases.append((3, np.stack([rng.choice(E, size=2, replace=False) for _ in range(3)]).astype(np.int32)))
+    for T, ids_h in cases:
+        k = ids_h.shape[1]
+        X = synth.activations(T, n, seed=seed + T)
+        w_h = rng.random((T, k)).astype(np.float32)
+        got = layer(to_dev_bits(X).reshape(T, n), torch.from_numpy(ids_h).to(dev()), torch.from_numpy(w_h).to(dev())).cpu().numpy()
+        layer.status()
+        ref = np.zeros((T, n), np.float64)
+        for e in range(E):
+            rows, slots = np.nonzero(ids_h == e)
+            if len(rows) == 0:
+                continue
+            a = oracle.silu_mul_bf16(oracle.gemm(packs[e][0], X[rows]), oracle.gemm(packs[e][1], X[rows]))
+            ref[rows] += w_h[rows, slots][:, None].astype(np.float64) * oracle.gemm(packs[e][2], a)
+        assert rel_err(got, ref) < 1e-4, (T, k)
