@@ -612,7 +612,8 @@ def gemm_b256_roofline(layers):
         extra = {"vendor_bf16_frac": fl / vus / 1e6 / 2500.0, "vendor_bf16_us_per_step": vus,
                  "vendor_bf16_gate_up_frac": layers["vendor_bf16_gate_up_b256"]["mfma_frac"]}
     return {**extra, "bound": "mfma", "achieved": fl / us / 1e6, "peak": 2500.0, "unit": "TFLOP/s", "frac": fl / us / 1e6 / 2500.0,
-            "traffic": None, "kernel": "gemm_mfma_kernel, QKV + O + gate|up + down at B=256", "flops_per_step": fl,
+            "traffic": None, "gate_up_traffic": measured_traffic("gemm_gate_up_b256"),
+            "kernel": "gemm_mfma_kernel, QKV + O + gate|up + down at B=256", "flops_per_step": fl,
             "us_per_step": us, "gate_up_frac": layers["gate_up_b256"]["mfma_frac"],
             # the same four products as the engine's layer issues them: gate|up with SiLU*mul in its epilogue
             "gate_up_swiglu_frac": layers["gate_up_swiglu_b256"]["mfma_frac"],
