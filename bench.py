@@ -25,6 +25,9 @@ Workloads (synthetic, seeded, random-init weights of the Llama-3.1-8B shape:
                   INT8 cache) with every sequence on its own cache region, at several (batch, context) points;
                   `roofline` prices the cache bytes of B = 256 at 2000 positions against the HBM peak.
 
+  codec           the standalone codec kernels on three Llama-3.1-8B tensors: t12_decompress (planes -> bf16, patched and
+                  unpatched) and the GPU packer's passes (histogram, planes, escapes), in GB/s of the bytes each must move.
+
   tokenizer       host only: one step = encoding ~1 MB of text (150 000 words of a 4000-word list) with the engine's
                   byte-level BPE tokenizer over the ~20 000 merges that build those words; `cpu_baseline` is the reference's rule restated literally (one pass over the
                   text per merge) on a 4 KB sample of the same text.
@@ -415,6 +418,73 @@ def run_moe(args, t12, torch, dev):
     }
 
 
+def run_codec(args, t12, torch, dev):
+    """The standalone codec kernels on Llama-3.1-8B tensors (three rotating copies each, so nothing is served from a
+    cache): t12_decompress (split-12 planes -> bf16, patched = lossless and unpatched) and the GPU packer's three passes
+    (histogram, planes, escapes).  `value` is the patched decode of gate 14336 x 4096 in GB/s of HBM traffic."""
+    import ctypes as C
+    cur = torch.cuda.current_stream()
+    st = cur.cuda_stream
+    shapes = {"gate_14336x4096": (14336, 4096), "down_4096x14336": (4096, 14336), "o_4096x4096": (4096, 4096)}
+    out = {}
+    t0 = time.time()
+    for name, (M, K) in shapes.items():
+        ws = [synth_weight(torch, M, K, 7000 + i, dev) for i in range(3)]
+        ts = [t12.pack_device(w) for w in ws]
+        dst = torch.empty((M, K), dtype=torch.int16, device=dev)
+        n = float(M) * K
+        P = sum(t.P for t in ts) / 3.0
+        res = {"weights": int(n), "escapes": P / n}
+
+        def med(fn, reps=max(args.steps, 20)):
+            for _ in range(3):
+                fn()
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+            for a, b in evs:
+                a.record(cur)
+                fn()
+                b.record(cur)
+            torch.cuda.synchronize()
+            return sorted(a.elapsed_time(b) for a, b in evs)[reps // 2] / 3.0        # ms per tensor
+
+        for patched in (1, 0):
+            ms = med(lambda: [t12.decompress(t, patched=bool(patched), out=dst, stream=st) for t in ts])
+            nbytes = 1.5 * n + 2.0 * n + (8.0 * P + 4.0 * (M + 1) if patched else 0.0)
+            res["decompress_patched" if patched else "decompress_unpatched"] = {"us": ms * 1e3, "GBps": nbytes / ms / 1e6}
+        hist = torch.empty(256, dtype=torch.int64, device=dev)
+        ms = med(lambda: [t12.check(t12.lib.t12_pack_histogram(w.data_ptr(), w.numel(), hist.data_ptr(), st), "hist") for w in ws])
+        res["pack_histogram"] = {"us": ms * 1e3, "GBps": 2.0 * n / ms / 1e6}
+        sm = torch.empty(int(n), dtype=torch.uint8, device=dev)
+        gr = torch.empty((int(n) + 1) // 2, dtype=torch.uint8, device=dev)
+        cnt = torch.empty(M, dtype=torch.int32, device=dev)
+        ms = med(lambda: [t12.check(t12.lib.t12_pack_planes(w.data_ptr(), M, K, t.base_exp, sm.data_ptr(), gr.data_ptr(),
+                                                            cnt.data_ptr(), st), "planes") for w, t in zip(ws, ts)])
+        res["pack_planes"] = {"us": ms * 1e3, "GBps": 3.5 * n / ms / 1e6}
+        ms = med(lambda: [t12.check(t12.lib.t12_pack_escapes(w.data_ptr(), M, K, t.base_exp, t.row_off.data_ptr(), t.cols.data_ptr(),
+                                                             t.correct.data_ptr(), t.wrong.data_ptr(), st), "escapes")
+                          for w, t in zip(ws, ts) if t.P])
+        res["pack_escapes"] = {"us": ms * 1e3, "GBps": (2.0 * n + 8.0 * P) / ms / 1e6}
+        tot_us = res["pack_histogram"]["us"] + res["pack_planes"]["us"] + res["pack_escapes"]["us"]
+        res["pack_total"] = {"us": tot_us, "Gweights_per_s": n / tot_us / 1e3}
+        out[name] = res
+        del ws, ts, dst, sm, gr
+    head = out["gate_14336x4096"]["decompress_patched"]
+    return {
+        "metric": "GB/s of HBM traffic of the standalone split-12 decode (1.5 B read + 2 B written per weight, escapes exact), "
+                  "gate 14336x4096 of Llama-3.1-8B",
+        "value": head["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": max(args.steps, 20), "warmup": 3,
+        "ms_per_step": head["us"] / 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "codec: t12_decompress and the GPU packer (histogram, planes, escapes) on gate 14336x4096, down "
+                               "4096x14336, O 4096x4096; N(0,0.02)+3e-4 outliers; 3 rotating copies"},
+        "tensors": out,
+        "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": head["GBps"] / HBM_PEAK_GBS, "traffic": None, "kernel": "decompress_vec_kernel",
+                     "bytes_per_launch": 3.5 * 14336 * 4096, "us_per_launch": head["us"]},
+        "setup_s": time.time() - t0,
+    }
+
+
 def run_attention(args, t12, torch, dev):
     """The attention step of one Llama-3.1-8B decoder layer (RoPE of q and k, INT8 store of the new K / V
     row, GQA attention over the INT8 cache: launch_rope_store_attention), every sequence on its own cache
@@ -734,7 +804,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="decode", choices=["decode", "gemv_stack_b1", "moe", "gemm_layers", "attention", "tokenizer"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "gemv_stack_b1", "moe", "gemm_layers", "attention", "codec", "tokenizer"])
     ap.add_argument("--prompt", type=int, default=128)
     ap.add_argument("--no-batch256", dest="batch256", action="store_false")
     ap.add_argument("--layers", type=int, default=LLAMA8B["n_layer"], help="debug: fewer layers (invalid as a result)")
@@ -773,6 +843,9 @@ def main():
         return
     if args.workload == "attention":
         emit(run_attention(args, t12, torch, dev), json_fd)
+        return
+    if args.workload == "codec":
+        emit(run_codec(args, t12, torch, dev), json_fd)
         return
     cfg = dict(LLAMA8B, n_layer=args.layers)
 
