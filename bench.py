@@ -28,6 +28,9 @@ Workloads (synthetic, seeded, random-init weights of the Llama-3.1-8B shape:
   codec           the standalone codec kernels on three Llama-3.1-8B tensors: t12_decompress (planes -> bf16, patched and
                   unpatched) and the GPU packer's passes (histogram, planes, escapes), in GB/s of the bytes each must move.
 
+  convert         checkpoint ingestion end to end: a 1.4 GB bf16 safetensors checkpoint (two Llama-3.1-8B layers, embedding,
+                  head) through convert() -- mmap read, packing on the GPU, model directory written -- in GB/s of checkpoint.
+
   tokenizer       host only: one step = encoding ~1 MB of text (150 000 words of a 4000-word list) with the engine's
                   byte-level BPE tokenizer over the ~20 000 merges that build those words; `cpu_baseline` is the reference's rule restated literally (one pass over the
                   text per merge) on a 4 KB sample of the same text.
@@ -485,6 +488,63 @@ def run_codec(args, t12, torch, dev):
     }
 
 
+def run_convert(args, t12, torch, dev):
+    """Checkpoint ingestion end to end: a bf16 safetensors checkpoint of Llama-3.1-8B's layer shapes (2 layers, vocabulary
+    32000, untied head: 1.4 GB) is written to a temporary directory, then convert() reads it (mmap), packs every matrix
+    on the GPU and writes the engine's model directory.  `value` = GB of checkpoint per second of convert(); host file
+    I/O and the PCIe copies are inside the timed region (this is the path's real boundary), the GPU packer's own rate is
+    under --workload codec."""
+    import importlib
+    import shutil
+    import tempfile
+    conv = importlib.import_module(t12.__name__ + ".convert")
+    st = importlib.import_module("safetensors.torch")
+    n, ff, kv, V, nl = 4096, 14336, 1024, 32000, 2
+    cfg = dict(hidden_size=n, num_attention_heads=32, num_key_value_heads=8, num_hidden_layers=nl, intermediate_size=ff,
+               vocab_size=V, max_position_embeddings=8192, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+    src, dst = tempfile.mkdtemp(prefix="t12_ckpt_"), tempfile.mkdtemp(prefix="t12_model_")
+    try:
+        t0 = time.time()
+        tensors = {"model.embed_tokens.weight": synth_weight(torch, V, n, 8000, dev, sigma=1.0, p_out=0.0).cpu(),
+                   "model.norm.weight": torch.ones(n, dtype=torch.bfloat16),
+                   "lm_head.weight": synth_weight(torch, V, n, 8001, dev).cpu()}
+        for i in range(nl):
+            pfx = "model.layers.%d." % i
+            tensors[pfx + "input_layernorm.weight"] = torch.ones(n, dtype=torch.bfloat16)
+            tensors[pfx + "post_attention_layernorm.weight"] = torch.ones(n, dtype=torch.bfloat16)
+            for j, (name, (M, K)) in enumerate((("self_attn.q_proj", (n, n)), ("self_attn.k_proj", (kv, n)),
+                                                ("self_attn.v_proj", (kv, n)), ("self_attn.o_proj", (n, n)),
+                                                ("mlp.gate_proj", (ff, n)), ("mlp.up_proj", (ff, n)), ("mlp.down_proj", (n, ff)))):
+                tensors[pfx + name + ".weight"] = synth_weight(torch, M, K, 8100 + 10 * i + j, dev).cpu()
+        nbytes = sum(t.numel() * t.element_size() for t in tensors.values())
+        st.save_file(tensors, os.path.join(src, "model.safetensors"))
+        with open(os.path.join(src, "config.json"), "w") as f:
+            json.dump(cfg, f)
+        del tensors
+        t_setup = time.time() - t0
+        secs = []
+        for _ in range(2):                                  # the second pass reads the checkpoint from the page cache
+            shutil.rmtree(dst, ignore_errors=True)
+            t1 = time.time()
+            stats = conv.convert(src, dst, device=str(dev))
+            torch.cuda.synchronize()
+            secs.append(time.time() - t1)
+        out_bytes = sum(os.path.getsize(os.path.join(dst, f)) for f in os.listdir(dst))
+    finally:
+        shutil.rmtree(src, ignore_errors=True)
+        shutil.rmtree(dst, ignore_errors=True)
+    best = min(secs)
+    return {
+        "metric": "GB/s of bf16 checkpoint through convert(): safetensors -> GPU packer -> split-12 model directory",
+        "value": nbytes / best / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": 2, "warmup": 0, "ms_per_step": best * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "convert: 2 Llama-3.1-8B layers + 32000 x 4096 embedding and head, bf16 safetensors, one shard",
+                   "checkpoint_GB": nbytes / 1e9, "model_dir_GB": out_bytes / 1e9, "tensors": len(stats)},
+        "seconds_per_pass": secs, "compression_ratio": out_bytes / nbytes,
+        "roofline": None, "setup_s": t_setup,
+    }
+
+
 def run_attention(args, t12, torch, dev):
     """The attention step of one Llama-3.1-8B decoder layer (RoPE of q and k, INT8 store of the new K / V
     row, GQA attention over the INT8 cache: launch_rope_store_attention), every sequence on its own cache
@@ -804,7 +864,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="decode", choices=["decode", "gemv_stack_b1", "moe", "gemm_layers", "attention", "codec", "tokenizer"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "gemv_stack_b1", "moe", "gemm_layers", "attention", "codec", "convert", "tokenizer"])
     ap.add_argument("--prompt", type=int, default=128)
     ap.add_argument("--no-batch256", dest="batch256", action="store_false")
     ap.add_argument("--layers", type=int, default=LLAMA8B["n_layer"], help="debug: fewer layers (invalid as a result)")
@@ -846,6 +906,9 @@ def main():
         return
     if args.workload == "codec":
         emit(run_codec(args, t12, torch, dev), json_fd)
+        return
+    if args.workload == "convert":
+        emit(run_convert(args, t12, torch, dev), json_fd)
         return
     cfg = dict(LLAMA8B, n_layer=args.layers)
 
