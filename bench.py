@@ -530,6 +530,16 @@ def run_convert(args, t12, torch, dev):
             torch.cuda.synchronize()
             secs.append(time.time() - t1)
         out_bytes = sum(os.path.getsize(os.path.join(dst, f)) for f in os.listdir(dst))
+        # and the way back in: load_model on the directory just written (files in the page cache), derived escape
+        # tables and the upload included
+        os.environ["TURBO_CTX"] = "256"
+        load_s = []
+        for _ in range(2):
+            t1 = time.time()
+            eng = t12.Engine.load(dst, batch=1)
+            torch.cuda.synchronize()
+            load_s.append(time.time() - t1)
+            eng.close()
     finally:
         shutil.rmtree(src, ignore_errors=True)
         shutil.rmtree(dst, ignore_errors=True)
@@ -541,6 +551,7 @@ def run_convert(args, t12, torch, dev):
         "config": {"workload": "convert: 2 Llama-3.1-8B layers + 32000 x 4096 embedding and head, bf16 safetensors, one shard",
                    "checkpoint_GB": nbytes / 1e9, "model_dir_GB": out_bytes / 1e9, "tensors": len(stats)},
         "seconds_per_pass": secs, "compression_ratio": out_bytes / nbytes,
+        "load_model": {"seconds_per_pass": load_s, "GBps": out_bytes / min(load_s) / 1e9},
         "roofline": None, "setup_s": t_setup,
     }
 
