@@ -1219,9 +1219,18 @@ int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_st
     // K split: as many workgroups as the chip has CUs, not more (measured on the four Llama-8B layer shapes at B = 32 ..
     // 256: 32 row tiles run best as 8 splits, 48 as 4, 224 unsplit -- every doubling past ~one workgroup per CU costs more
     // in partial sums than it gains), every split at least 8 stages long.
-    const int btiles = B > 128 ? (B + 255) / 256 : 1;
-    int ks = 1;
-    while (tiles * btiles * ks * 2 <= 256 + 32 && K / (ks * 2) >= 8 * KC && ks < T12_MAX_KSPLIT) ks *= 2;
+    auto splits_for = [&](int btiles) {
+        int ks = 1;
+        while (tiles * btiles * ks * 2 <= 256 + 32 && K / (ks * 2) >= 8 * KC && ks < T12_MAX_KSPLIT) ks *= 2;
+        return ks;
+    };
+    int ks = splits_for(B > 128 ? (B + 255) / 256 : 1);
+    // A 256-row batch tile whose K slice is under 16 stages (O of the Llama layer: 32 row tiles, 8 splits of 512
+    // columns) spends its time filling and draining, and leaves twice the partial sums: such a launch takes 128-row
+    // batch tiles and half the splits (O at B = 256 32 -> 27.5 us with the reduction; down, whose slices are long,
+    // 55 -> 58 us and QKV 34 -> 37 us the same way, so they keep the 256-row tile).
+    const bool tb128 = B > 128 && ks > 1 && K / ks < 16 * KC;
+    if (tb128) ks = splits_for((B + 127) / 128);
     int kslice = (((K + 2 * KC - 1) / (2 * KC) + ks - 1) / ks) * 2 * KC;      // whole windows of two stages
     ks = (K + kslice - 1) / kslice;
     p.ksplit = ks;
@@ -1247,7 +1256,7 @@ int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_st
     }
     int rc;
     if (B <= 64) rc = launch_mfma<2, 4, 1, 1>(p, tiles, st);
-    else if (B <= 128) rc = launch_mfma<2, 4, 2, 1>(p, tiles, st);
+    else if (B <= 128 || tb128) rc = launch_mfma<2, 4, 2, 1>(p, tiles, st);
     else rc = launch_mfma<4, 2, 2, 2>(p, tiles, st);
     if (rc) return rc;
 
