@@ -813,6 +813,42 @@ def run_tokenizer(args, t12):
             "roofline": None, "cpu_baseline": cpu}
 
 
+def reference_named_leg(t12, torch, dev, copies_gate, cur, g, iters):
+    """launch_split12_batch4/8_async (the reference's own small-batch entry points, escapes as the derived tables of its
+    loader) on the gate tensor, three rotating copies, next to t12_gemm on the same tensors and batch."""
+    import numpy as np
+    M, K = copies_gate[0].M, copies_gate[0].K
+
+    def tables(t):
+        ro, cols, cor = t.row_off.cpu().numpy(), t.cols.cpu().numpy(), t.correct.cpu().numpy()
+        rows = np.repeat(np.arange(M), np.diff(ro))
+        order = np.lexsort((cols, cols % 256, rows))            # (row, col % 256, ascending col): engine/model.cpp:92-125
+        return [torch.from_numpy(a).to(dev) for a in (ro[:-1].astype(np.int32).copy(), cor[order].copy())]
+    tabs = [tables(t) for t in copies_gate]
+    out = {}
+    for NB in (4, 8):
+        X = torch.randn((NB, K), device=dev, generator=g).to(torch.bfloat16).view(torch.int16)
+        outs = [torch.zeros(M, device=dev) for _ in range(NB)]
+        fn = t12.lib.launch_split12_batch4_async if NB == 4 else t12.lib.launch_split12_batch8_async
+
+        def named():
+            for t, (rb, vl) in zip(copies_gate, tabs):
+                t12.check(fn(*([t.sm.data_ptr(), t.gr.data_ptr(), t.base_exp] + [X[j].data_ptr() for j in range(NB)] +
+                               [rb.data_ptr(), None, vl.data_ptr()] + [o.data_ptr() for o in outs] + [M, K, cur.cuda_stream])))
+        dense = torch.zeros((NB, M), device=dev)
+
+        def own():
+            for t in copies_gate:
+                t12.gemm([t], X, outs=[dense])
+        for name, fn_ in (("launch_split12_batch%d_async" % NB, named), ("t12_gemm_b%d" % NB, own)):
+            for _ in range(3):
+                fn_()
+            _, ms = timed(torch, cur, fn_, iters)
+            us = ms * 1e3 / len(copies_gate)
+            out[name] = {"us": round(us, 2), "weight_GBps": round(1.5 * M * K / us / 1e3, 1)}
+    return out
+
+
 def run_gemm_layers(args, t12, torch, dev):
     """The four Llama-3.1-8B linear-layer shapes through the fused decode+GEMM at B = 2 .. 256 on three rotating weight
     copies, the vendor library's plain bf16 GEMM on the same shapes as a yardstick, the same launch on half and a
@@ -838,6 +874,7 @@ def run_gemm_layers(args, t12, torch, dev):
         calibration_copy(torch, dev)
     layers = gemm_layer_leg(t12, torch, dev, cfg, weight_of, 3, cur, g, iters=max(args.steps, 50))
     probe = clock_probe(t12)
+    named = reference_named_leg(t12, torch, dev, [copies[c][4] for c in range(3)], cur, g, 20)
     us256 = sum(layers["%s_b256" % k]["us"] for k in ("qkv", "o", "gate_up", "down"))
     fl256 = sum(layers["%s_b256" % k]["flops"] for k in ("qkv", "o", "gate_up", "down"))
     gu = layers["gate_up_b256"]
@@ -850,6 +887,7 @@ def run_gemm_layers(args, t12, torch, dev):
                                "down 14336->4096; N(0,0.02)+3e-4 outliers; B in {2,4,8,16,32,64,128,256}; 3 rotating weight copies"},
         "layers": layers,
         "clock_probe": probe,
+        "reference_named_launchers_gate_14336x4096": named,
         "roofline": {"bound": "mfma", "achieved": gu["TFLOPs"], "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": gu["TFLOPs"] / 2500.0, "traffic": measured_traffic("gemm_gate_up_b256"),
                      "kernel": "gemm_mfma_kernel<4,2,2,2> on gate|up at B=256", "flops_per_launch": gu["flops"],

@@ -274,6 +274,11 @@ typedef struct PatchBatchDesc {
 } PatchBatchDesc;
 int launch_patches_b1_batched_async(void* descs_gpu, const void* descs_cpu, int num_descs,
                                     int max_M, void* stream);
+/* Batches of 4 / 8 with the escapes as the derived tables of the reference's loader (engine/model.cpp:86-160):
+ * esc_vals ordered (row, col % 256, ascending col), esc_row_base[row] = first slot of the row, esc_counts optional and
+ * unused when K % 128 == 0 (both table pointers NULL: the unpatched product).  K % 128 == 0, K <= 65536, base_exp in
+ * 0..240 and 16-byte aligned planes and activations stream the planes like t12_gemm at B <= 16 and place every escape by
+ * its rank within its row; other shapes keep the reference's column ownership (one column per lane and step). */
 int launch_split12_batch4_async(const void* sm, const void* gr, int base_exp,
                                 const void* a0, const void* a1, const void* a2, const void* a3,
                                 const void* esc_row_base, const void* esc_counts, const void* esc_vals,

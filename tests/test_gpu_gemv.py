@@ -195,28 +195,70 @@ def test_full_size_linearity(t12, oracle, synth):
     assert rel_err(o.cpu().numpy(), ref) < TOL
 
 
+def _run_batch_launcher(t12, NB, d, acts, tables, M, K):
+    """launch_split12_batch{NB}_async on device tensor d; tables = (row_base, counts or None, vals) or None."""
+    fn = t12.lib.launch_split12_batch4_async if NB == 4 else t12.lib.launch_split12_batch8_async
+    outs = [torch.zeros(M, device=dev()) for _ in range(NB)]
+    tb = [None, None, None] if tables is None else [None if a is None else a.data_ptr() for a in tables]
+    args = [d.sm.data_ptr(), d.gr.data_ptr(), d.base_exp] + [a.data_ptr() for a in acts] + tb + \
+           [o.data_ptr() for o in outs] + [M, K, t12.current_stream()]
+    t12.check(fn(*args))
+    torch.cuda.synchronize()
+    return np.stack([o.cpu().numpy() for o in outs])
+
+
+# (M, K, p_outlier): K % 128 == 0 runs the streaming form, the others the reference's column ownership;
+# 77 and 5 rows: a last group of 16 that is part empty; 4096 columns: every col % 256 class 16 columns deep
 @pytest.mark.parametrize("NB", [4, 8])
-def test_reference_named_batch_launchers(t12, oracle, synth, NB):
+@pytest.mark.parametrize("M,K,p_out", [(96, 2304, 5e-3), (77, 4096, 2e-3), (5, 128, 2e-2), (64, 2320, 5e-3),
+                                       (33, 1000, 5e-3), (300, 8192, 3e-4)])
+def test_reference_named_batch_launchers(t12, oracle, synth, NB, M, K, p_out):
     """launch_split12_batch4/8_async take the derived escape tables of the reference's loader
-    (esc_row_base / esc_counts / esc_vals, engine/model.cpp:86-160); esc_counts may be NULL here."""
-    M, K = 96, 2304
-    p = oracle.pack(synth.weights_llm(M, K, seed=50 + NB, p_outlier=5e-3))
+    (esc_row_base / esc_counts / esc_vals, engine/model.cpp:86-160); esc_counts may be NULL here, and without
+    tables the product is the unpatched one (decompress_v2.hip:573-701 with esc_vals == NULL)."""
+    p = oracle.pack(synth.weights_llm(M, K, seed=50 + NB + M, p_outlier=p_out))
+    assert p.P > 0
     row_base, counts, vals, _ = oracle.escape_tables(p)
     X = synth.activations(NB, K, seed=60)
     ref = oracle.gemm(p, X)
     d = t12.DeviceTensor12.from_packed(p, dev())
     acts = [to_dev_bits(X[j]) for j in range(NB)]
     rb, cn, vl = (torch.from_numpy(a).to(dev()) for a in (row_base, counts, vals))
-    fn = t12.lib.launch_split12_batch4_async if NB == 4 else t12.lib.launch_split12_batch8_async
-    for use_counts in (True, False):
-        outs = [torch.zeros(M, device=dev()) for _ in range(NB)]
-        args = [d.sm.data_ptr(), d.gr.data_ptr(), d.base_exp] + [a.data_ptr() for a in acts] + \
-               [rb.data_ptr(), cn.data_ptr() if use_counts else None, vl.data_ptr()] + \
-               [o.data_ptr() for o in outs] + [M, K, t12.current_stream()]
-        t12.check(fn(*args))
-        torch.cuda.synchronize()
+    for tables in ((rb, cn, vl), (rb, None, vl)):
+        got = _run_batch_launcher(t12, NB, d, acts, tables, M, K)
         for j in range(NB):
-            assert rel_err(outs[j].cpu().numpy(), ref[j]) < TOL, (use_counts, j)
+            assert rel_err(got[j], ref[j]) < TOL, (tables[1] is None, j)
+    got = _run_batch_launcher(t12, NB, d, acts, None, M, K)
+    assert rel_err(got, oracle.gemm(p, X, patched=False)) < TOL
+
+
+def test_reference_named_batch_launchers_escape_order_and_overflow(t12, oracle, synth):
+    """The slot of an escape in esc_vals is its rank by (col % 256, col) within its row: rows whose escapes share
+    col % 256 classes in both orders, distinct values everywhere (a wrong rank picks a wrong value), and one row
+    with more escapes than the streaming form keeps per row (it then recomputes its 16 rows the reference's way)."""
+    M, K, NB = 40, 4096, 8
+    w = synth.weights_llm(M, K, seed=91, p_outlier=0.0).copy()
+    rng = np.random.default_rng(92)
+    big = lambda n: oracle.f32_to_bf16_bits((rng.uniform(3.0, 60.0, n) * rng.choice([-1.0, 1.0], n)).astype(np.float32))
+    w[3, [5, 261, 517, 4, 260, 1029, 2, 4095, 3839]] = big(9)          # classes 5, 4, 2, 255 in mixed column order
+    w[17, np.arange(0, 4096, 256)] = big(16)                           # one class, sixteen deep
+    w[18, np.arange(255, 0, -5)] = big(51)                             # one per class
+    heavy = rng.choice(K, 300, replace=False)
+    w[37, heavy] = big(300)                                            # above the per-row list of the streaming form
+    p = oracle.pack(w)
+    row_base, counts, vals, _ = oracle.escape_tables(p)
+    slot3 = vals[row_base[3]:row_base[4]].tolist()
+    assert len(slot3) >= 9 and len(set(slot3)) == len(slot3)
+    X = synth.activations(NB, K, seed=93)
+    ref = oracle.gemm(p, X)
+    d = t12.DeviceTensor12.from_packed(p, dev())
+    acts = [to_dev_bits(X[j]) for j in range(NB)]
+    rb, cn, vl = (torch.from_numpy(a).to(dev()) for a in (row_base, counts, vals))
+    for tables in ((rb, cn, vl), (rb, None, vl)):
+        got = _run_batch_launcher(t12, NB, d, acts, tables, M, K)
+        # per row: an escape taken from the wrong slot moves its row by the size of an outlier
+        for r in range(M):
+            assert np.abs(got[:, r] - ref[:, r]).max() <= 1e-4 * max(np.abs(ref[:, r]).max(), 1.0), r
 
 
 def test_gemv_batch_entry_point(t12, oracle, synth):
