@@ -243,6 +243,47 @@ def test_c4_full_width_logits_and_greedy_stream(t12, oracle, full_width_model):
     assert got_stream == want_stream
 
 
+@pytest.mark.parametrize("batch", [1, 8])
+def test_c4_full_width_reference_host_engine_on_this_builds_launchers(t12, full_width_model, batch, capsys):
+    """The reference's host engine (engine/model.cpp + inference.cpp + sampler.cpp compiled unchanged by oracle/Makefile,
+    target ref_engine) linked with libturbo12.so, on the full-width model directory: its loader reads what this build's
+    save_model wrote, its forward_b1 / forward_b8 issue this build's launchers, and its greedy stream of 48 tokens is
+    this engine's (which the test above ties to the CPU decode step).  Prints both decode rates."""
+    import subprocess
+    import time
+    driver = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "_ref",
+                          "reference_engine_driver")
+    if not os.path.exists(driver):
+        pytest.skip("oracle/_ref/reference_engine_driver not built (needs the reference tree at build time)")
+    path, _ = full_width_model
+    rng = np.random.default_rng(4102)
+    prompt = [int(t) for t in rng.integers(3, FULL["n_vocab"], size=6)]
+    n_new = 48
+    env = dict(os.environ, TURBO_CTX="256", REF_DRIVER_TIMED="1")
+    env.pop("TURBO_FAST", None)
+    r = subprocess.run([driver, path, str(batch), str(n_new)] + [str(t) for t in prompt], capture_output=True,
+                       timeout=170, env=env)
+    assert r.returncode == 0, (r.returncode, r.stdout[-1500:], r.stderr[-1500:])
+    lines = r.stdout.split(b"\n")
+    got = [int(t) for t in [l for l in lines if l.startswith(b"tokens:")][0].split()[1:]]
+    sec, calls = [l for l in lines if l.startswith(b"timed:")][0].split()[1:]
+    eng = t12.Engine.load(path, batch=batch)
+    try:
+        want = eng.generate(prompt, n_new)
+        t0 = time.perf_counter()
+        again = eng.generate(prompt, n_new)
+        own_sec = time.perf_counter() - t0
+    finally:
+        eng.close()
+    assert again == want and len(want) >= 16
+    assert got == want
+    with capsys.disabled():
+        print("\n[2 layers at Llama-3.1-8B widths, B=%d] reference host code over this build's launchers: %.2f ms per "
+              "forward; this build's engine: %.2f ms per forward" % (batch, float(sec) / int(calls) * 1e3,
+                                                                    own_sec / (len(prompt) + len(want)) * 1e3), flush=True)
+
+
+
 def test_c4_full_width_b256_rows_equal_b1(t12, full_width_model):
     """256 lock-step copies through the decode+GEMM kernels give 256 identical rows that agree with the B = 1
     decode-GEMV logits up to the summation order."""
