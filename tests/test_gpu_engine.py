@@ -166,6 +166,8 @@ def test_synthetic_model_save_load_roundtrip(t12, tmp_path):
     cfg = dict(SMALL, n_layer=1)
     a = t12.Engine.synthetic(cfg, seed=77, max_seq=128, p_outlier=2e-3)
     try:
+        with pytest.raises(t12.T12Error, match="directory must exist"):
+            a.save(str(tmp_path / "not" / "there"))
         a.save(str(tmp_path))
         toks = [4, 8, 15]
         la = []

@@ -169,6 +169,41 @@ def test_reference_named_launchers(t12, oracle, synth):
     assert rel_err(ob.cpu().numpy(), oracle.gemv(pb, x)) < TOL
 
 
+def test_patch_launchers_ragged_rows_and_heavy_rows(t12, oracle, synth):
+    """The patch launchers alone, on a zeroed output: a row count that is no multiple of the rows a workgroup takes,
+    rows with 0, 1, 9, 70 and 300 entries, two descriptors of different M in one call; the sum of a row's entries
+    against float64."""
+    K = 4096
+    shapes = [(77, 51), (1000, 52)]
+    rng = np.random.default_rng(53)
+    x = synth.activations(1, K, seed=54)[0]
+    xd = to_dev_bits(x)
+    xf = oracle.bf16_bits_to_f32(x).astype(np.float64)
+    packs, devs, outs = [], [], []
+    for M, seed in shapes:
+        w = synth.weights_llm(M, K, seed=seed, p_outlier=3e-4).copy()
+        for r, n in ((0, 1), (M // 2, 9), (M - 2, 70), (M - 1, 300)):
+            w[r, rng.choice(K, n, replace=False)] = oracle.f32_to_bf16_bits(rng.uniform(3.0, 60.0, n).astype(np.float32))
+        p = oracle.pack(w)
+        packs.append(p)
+        devs.append(t12.DeviceTensor12.from_packed(p, dev()))
+        outs.append(torch.zeros(M, device=dev()))
+    descs = (t12.PatchBatchDesc * 2)(*[
+        t12.PatchBatchDesc(d.row_off.data_ptr(), d.cols.data_ptr(), d.correct.data_ptr(), d.wrong.data_ptr(),
+                           xd.data_ptr(), o.data_ptr(), d.M) for d, o in zip(devs, outs)])
+    scratch = torch.zeros(8 * 56, dtype=torch.uint8, device=dev())
+    t12.check(t12.lib.launch_patches_b1_batched_async(scratch.data_ptr(), descs, 2, 1000, t12.current_stream()))
+    torch.cuda.synchronize()
+    for p, o in zip(packs, outs):
+        delta = oracle.bf16_bits_to_f32(p.correct.view(np.uint16)).astype(np.float64) - \
+                oracle.bf16_bits_to_f32(p.wrong.view(np.uint16)).astype(np.float64)
+        want = np.zeros(p.M)
+        np.add.at(want, np.repeat(np.arange(p.M), np.diff(p.row_off)), delta * xf[p.cols])
+        got = o.cpu().numpy()
+        assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+        assert (got[np.diff(p.row_off) == 0] == 0).all()
+
+
 def test_gemv_rejects_bad_operands(t12):
     segs = (t12.Segment * 1)(t12.Segment(None, None, None, None, None, None, None, 4, 100, 0, 0))
     x = torch.zeros(16, dtype=torch.int16, device=dev())

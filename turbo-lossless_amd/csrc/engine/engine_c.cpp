@@ -65,7 +65,12 @@ void* t12_engine_create_synthetic(int n_vocab, int n_embd, int n_head, int n_hea
 
 int t12_engine_save(void* model, const char* dir)
 {
-    return guarded([&] { return save_model((Model*)model, dir) ? 0 : -1; });
+    return guarded([&] {
+        if (save_model((Model*)model, dir)) return 0;
+        t12_set_error("save_model: could not write the model files under %s (the directory must exist; the file is named on "
+                      "standard error)", dir);
+        return -1;
+    });
 }
 void t12_engine_free_model(void* model) { free_model((Model*)model); }
 

@@ -453,8 +453,8 @@ bool dump(const std::string& path, const T* dev, size_t count)
     std::vector<T> h(count);
     if (count && !gpu_ok(hipMemcpy(h.data(), dev, count * sizeof(T), hipMemcpyDeviceToHost), "download")) return false;
     std::ofstream f(path, std::ios::binary);
-    if (!f) return false;
-    if (count) f.write((const char*)h.data(), (std::streamsize)(count * sizeof(T)));
+    if (f && count) f.write((const char*)h.data(), (std::streamsize)(count * sizeof(T)));
+    if (!f) fprintf(stderr, "Cannot write: %s\n", path.c_str());
     return (bool)f;
 }
 
@@ -537,7 +537,10 @@ bool save_model(const Model* m, const std::string& dir)
                                                        c.n_ctx}, c.rope_theta, c.rms_norm_eps};
     {
         std::ofstream f(dir + "/config.bin", std::ios::binary);
-        if (!f) return false;
+        if (!f) {
+            fprintf(stderr, "Cannot write: %s/config.bin (the directory must exist)\n", dir.c_str());
+            return false;
+        }
         f.write((const char*)&raw, sizeof raw);
     }
     if (c.rope_scaling[0] > 0.0f) {

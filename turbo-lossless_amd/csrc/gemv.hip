@@ -371,17 +371,31 @@ __global__ __launch_bounds__(256) void gemv_general_kernel(const GemvParams p)
     if (lane == 0) sg.out[row] = p.add ? acc + p.add[row] : acc;
 }
 
-// Only the escape corrections (the reference's separate patch kernels).
+// Only the escape corrections (the reference's separate patch kernels): out[row] += sum over the row's entries of
+// (correct - wrong) * x[col].  Eight lanes per row (a row of an LLM tensor holds a handful of entries: one step), 32
+// rows per workgroup; the eight partial sums are folded with three xor exchanges, in an order that does not depend on
+// timing.  A row without entries is not written.
+constexpr int PATCH_LANES = 8;
+constexpr int PATCH_ROWS = 256 / PATCH_LANES;          // rows per workgroup; blk_start counts such groups
 __global__ __launch_bounds__(256) void patches_kernel(const GemvParams p)
 {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = threadIdx.x & (PATCH_LANES - 1), rloc = threadIdx.x / PATCH_LANES;
     const int blk = blockIdx.x;
     const int s = find_segment(p, blk);
     const T12Segment& sg = p.seg[s];
-    const int row = (blk - p.blk_start[s]) * 4 + wave;
-    if (row >= sg.M) return;
-    float c = t12_wave_sum(patch_partial<true>(sg, row, lane, p.act));
-    if (lane == 0 && c != 0.0f) sg.out[row] += c;
+    const int row = (blk - p.blk_start[s]) * PATCH_ROWS + rloc;
+    float c = 0.0f;
+    bool any = false;
+    if (row < sg.M) {
+        const int beg = sg.row_off[row], end = sg.row_off[row + 1];
+        any = end > beg;
+        for (int q = beg + sub; q < end; q += PATCH_LANES)
+            c += (t12_bf16_to_f32((uint16_t)sg.correct[q]) - t12_bf16_to_f32((uint16_t)sg.wrong[q])) *
+                 t12_bf16_to_f32(p.act[sg.cols[q]]);
+    }
+#pragma unroll
+    for (int off = PATCH_LANES / 2; off > 0; off >>= 1) c += __shfl_xor(c, off, T12_WAVE);
+    if (sub == 0 && any && c != 0.0f) sg.out[row] += c;
 }
 
 template <int NW, int R, int D, int MINB = 1>
@@ -646,7 +660,7 @@ static int launch_patch_descs(const PatchBatchDesc* d, int n, hipStream_t st)
             g.base_exp = 0;
             g.out_stride = g.reserved = 0;
             p.blk_start[cnt] = total;
-            total += (d[i].M + 3) / 4;
+            total += (d[i].M + PATCH_ROWS - 1) / PATCH_ROWS;
             cnt++;
             i++;
         }
