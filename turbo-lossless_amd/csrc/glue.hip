@@ -1541,10 +1541,14 @@ static bool norm_vec_ok(int n, const void* x, const void* res, const void* w, co
     return n >= 4 && n % 4 == 0 && n <= 8192 && al(x, 16) && al(res, 16) && al(w, 16) && al(y, 8) && al(part, 16) &&
            split_stride % 4 == 0 && ld % 4 == 0;
 }
-static int norm_vec_threads(int n)
+// Threads per row of the vectorised norm: one 16-byte piece per thread; with many rows in flight two pieces per thread
+// (half the waves at the block sum, two independent sets of loads per thread: 7.4 -> 7.05 us at 256 rows of 4096 with
+// four partial rows).
+static int norm_vec_threads(int n, int batch_size)
 {
-    const int t = (n / 4 + 63) / 64 * 64;
-    return t > 1024 ? 1024 : t;
+    const int per = batch_size >= 64 ? 8 : 4;
+    const int t = (n / per + 63) / 64 * 64;
+    return t < 64 ? 64 : (t > 1024 ? 1024 : t);
 }
 
 static int norm_threads(int n)
@@ -1558,7 +1562,7 @@ void launch_rms_norm_bf16_batch(const float* x, const float* weight, int16_t* y,
                                 hipStream_t stream)
 {
     if (norm_vec_ok(n, x, nullptr, weight, y, nullptr, 0, 0))
-        hipLaunchKernelGGL((rms_norm_vec_kernel<false, false, 1>), dim3(batch_size), dim3(norm_vec_threads(n)), 0, stream,
+        hipLaunchKernelGGL((rms_norm_vec_kernel<false, false, 1>), dim3(batch_size), dim3(norm_vec_threads(n, batch_size)), 0, stream,
                            (float*)x, (const float*)nullptr, weight, (uint16_t*)y, n, eps, (const float*)nullptr, 0,
                            (size_t)0, 0);
     else
@@ -1571,7 +1575,7 @@ void launch_add_rms_norm_bf16_batch(float* x, const float* residual, const float
                                     int batch_size, hipStream_t stream)
 {
     if (norm_vec_ok(n, x, residual, weight, y, nullptr, 0, 0))
-        hipLaunchKernelGGL((rms_norm_vec_kernel<true, false, 1>), dim3(batch_size), dim3(norm_vec_threads(n)), 0, stream, x,
+        hipLaunchKernelGGL((rms_norm_vec_kernel<true, false, 1>), dim3(batch_size), dim3(norm_vec_threads(n, batch_size)), 0, stream, x,
                            residual, weight, (uint16_t*)y, n, eps, (const float*)nullptr, 0, (size_t)0, 0);
     else
         hipLaunchKernelGGL(rms_norm_kernel<true>, dim3(batch_size), dim3(norm_threads(n)), 0, stream, x, residual, weight,
@@ -1591,7 +1595,7 @@ void launch_sum_add_rms_norm_bf16_batch(float* x, const float* partials, int nsp
         return;
     }
     if (norm_vec_ok(n, x, residual, weight, y, partials, split_stride, ld)) {
-        const dim3 g(batch_size), b(norm_vec_threads(n));
+        const dim3 g(batch_size), b(norm_vec_threads(n, batch_size));
         if (nsplit <= 4)
             hipLaunchKernelGGL((rms_norm_vec_kernel<true, true, 4>), g, b, 0, stream, x, residual, weight, (uint16_t*)y, n,
                                eps, partials, nsplit, split_stride, ld);
