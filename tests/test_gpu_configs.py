@@ -243,18 +243,21 @@ def test_c4_full_width_logits_and_greedy_stream(t12, oracle, full_width_model):
     assert got_stream == want_stream
 
 
-@pytest.mark.parametrize("batch", [1, 8])
-def test_c4_full_width_reference_host_engine_on_this_builds_launchers(t12, full_width_model, batch, capsys):
+@pytest.mark.parametrize("batch,variant", [(1, ""), (8, ""), (64, "_nv")])
+def test_c4_full_width_reference_host_engine_on_this_builds_launchers(t12, full_width_model, batch, variant, capsys):
     """The reference's host engine (engine/model.cpp + inference.cpp + sampler.cpp compiled unchanged by oracle/Makefile,
     target ref_engine) linked with libturbo12.so, on the full-width model directory: its loader reads what this build's
     save_model wrote, its forward_b1 / forward_b8 issue this build's launchers, and its greedy stream of 48 tokens is
-    this engine's (which the test above ties to the CPU decode step).  Prints both decode rates."""
+    this engine's (which the test above ties to the CPU decode step).  Prints both decode rates.
+    variant "_nv": the build of the same files with their other branch selected (oracle/Makefile); at 64 rows its
+    forward_batch_tiled calls nv_launch_split12_fused_gemm_async for the tensors of 4096 rows and more,
+    nv_launch_split12_cublas_batch_async for wk / wv, and the corrections as nv_launch_patches_batch_async."""
     import subprocess
     import time
     driver = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "_ref",
-                          "reference_engine_driver")
+                          "reference_engine_driver" + variant)
     if not os.path.exists(driver):
-        pytest.skip("oracle/_ref/reference_engine_driver not built (needs the reference tree at build time)")
+        pytest.skip("oracle/_ref/reference_engine_driver%s not built (needs the reference tree at build time)" % variant)
     path, _ = full_width_model
     rng = np.random.default_rng(4102)
     prompt = [int(t) for t in rng.integers(3, FULL["n_vocab"], size=6)]
@@ -278,8 +281,8 @@ def test_c4_full_width_reference_host_engine_on_this_builds_launchers(t12, full_
     assert again == want and len(want) >= 16
     assert got == want
     with capsys.disabled():
-        print("\n[2 layers at Llama-3.1-8B widths, B=%d] reference host code over this build's launchers: %.2f ms per "
-              "forward; this build's engine: %.2f ms per forward" % (batch, float(sec) / int(calls) * 1e3,
+        print("\n[2 layers at Llama-3.1-8B widths, B=%d%s] reference host code over this build's launchers: %.2f ms per "
+              "forward; this build's engine: %.2f ms per forward" % (batch, variant, float(sec) / int(calls) * 1e3,
                                                                     own_sec / (len(prompt) + len(want)) * 1e3), flush=True)
 
 

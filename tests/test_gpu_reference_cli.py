@@ -143,3 +143,33 @@ def test_reference_host_engine_runs_on_this_builds_launchers(oracle, model_dir, 
     want = oracle.RefModel(SMALL, *parts, max_seq=CTX).generate(prompt, max_tokens, eos=EOS)
     assert len(want) >= 8
     assert got == want
+
+
+DRIVER_NV = os.path.join(ROOT, "oracle", "_ref", "reference_engine_driver_nv")
+
+
+@pytest.mark.parametrize("batch", [1, 8, 12, 64, 256])
+def test_reference_host_engine_other_branch_runs_on_this_builds_launchers(oracle, model_dir, batch):
+    """The same three reference files compiled with the macro that selects their other branch (inference.cpp:32-41,
+    227-330, 537-677): batch 1 goes through nv_launch_split12_v2(_dual)_async and the batched patch launcher, batch 8
+    through launch_split12_batch8_async, larger batches through forward_batch_tiled -- nv_launch_split12_cublas_batch_async
+    for this model's tensors (all under 4096 rows), the corrections as nv_launch_patches_batch_async on the state's second
+    stream, the batch forms of the RoPE / store / attention launchers.  Greedy stream = the CPU decode step's."""
+    if not os.path.exists(DRIVER_NV):
+        pytest.skip("oracle/_ref/reference_engine_driver_nv not built (needs the reference tree at build time)")
+    path, parts = model_dir
+    rng = np.random.default_rng(8)
+    prompt = [BOS] + [int(t) for t in rng.integers(3, SMALL["n_vocab"], 7)]
+    max_tokens = 20
+    env = dict(os.environ, TURBO_CTX=str(CTX))
+    env.pop("TURBO_FAST", None)
+    env.pop("TURBO_CUBLAS", None)
+    r = subprocess.run([DRIVER_NV, path, str(batch), str(max_tokens)] + [str(t) for t in prompt], capture_output=True,
+                       timeout=120, env=env)
+    assert r.returncode == 0, (r.returncode, r.stdout[-1500:], r.stderr[-1500:])
+    line = [l for l in r.stdout.split(b"\n") if l.startswith(b"tokens:")]
+    assert len(line) == 1, r.stdout[-1500:]
+    got = [int(t) for t in line[0].split()[1:]]
+    want = oracle.RefModel(SMALL, *parts, max_seq=CTX).generate(prompt, max_tokens, eos=EOS)
+    assert len(want) >= 8
+    assert got == want

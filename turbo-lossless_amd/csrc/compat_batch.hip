@@ -323,6 +323,9 @@ int launch(const void* sm, const void* gr, int base_exp, const void* const* a, c
 
 // nv_apply_patches_batch (nvidia_kernels.cu:295-319): one thread per (listed row, batch row) pair walks the row's
 // escape slice: out[b, row] += sum over entries of (correct - wrong) * x[b, col]; nothing is written when the sum is 0.
+// Neighbouring threads take neighbouring listed rows of ONE batch row: the read-modify-write of out[b, row] then covers
+// whole cache lines (with neighbouring batch rows per wave every lane touched a line of its own: 24 -> 15 us per launch
+// over the tensors of two Llama-width layers and the head at 64 rows).
 __global__ __launch_bounds__(256) void patches_batch_kernel(const int32_t* __restrict__ row_off, const int32_t* __restrict__ cols,
                                                             const int16_t* __restrict__ correct, const int16_t* __restrict__ wrong,
                                                             const int32_t* __restrict__ rows, const uint16_t* __restrict__ act,
@@ -330,8 +333,8 @@ __global__ __launch_bounds__(256) void patches_batch_kernel(const int32_t* __res
                                                             int B)
 {
     const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    const int ri = (int)(idx / B), b = (int)(idx % B);
-    if (ri >= n_rows) return;
+    const int b = (int)(idx / n_rows), ri = (int)(idx % n_rows);
+    if (b >= B) return;
     const int row = rows[ri];
     const uint16_t* x = act + (size_t)b * act_stride;
     float c = 0.0f;
