@@ -31,11 +31,29 @@ extern "C" void t12_rope_freqs(int head_dim, float theta, float factor, float lo
 
 namespace {
 
+// Wave-wide maximum, valid in every lane: six DPP row operations fold the wave into lane 63 (lanes a step does not
+// reach keep their own value), one v_readlane hands it to everybody.  (Six exchanges through ds_bpermute take several
+// times as long; the attention kernels do three to five such reductions one after the other per tile.)
 __device__ __forceinline__ float wave_max(float v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, T12_WAVE));
-    return v;
+#define T12_DPP_MAX(ctrl, rmask)                                                                                   \
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v),                 \
+                                                                       __builtin_bit_cast(int, v), (ctrl), (rmask), \
+                                                                       0xF, false)))
+    T12_DPP_MAX(0xB1, 0xF);    // quad_perm [1,0,3,2]
+    T12_DPP_MAX(0x4E, 0xF);    // quad_perm [2,3,0,1]
+    T12_DPP_MAX(0x141, 0xF);   // row_half_mirror
+    T12_DPP_MAX(0x140, 0xF);   // row_mirror: every lane of a 16-lane row holds the row maximum
+    T12_DPP_MAX(0x142, 0xA);   // row_bcast15 into rows 1 and 3
+    T12_DPP_MAX(0x143, 0xC);   // row_bcast31 into rows 2 and 3
+#undef T12_DPP_MAX
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// Wave-wide sum by the same route (the order of the additions differs from t12_wave_sum's butterfly).
+__device__ __forceinline__ float wave_sum_dpp(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, t12_wave_sum_lane63(v)), 63));
 }
 
 // Block-wide sum / max over up to 16 waves; every thread gets the result.
@@ -914,7 +932,7 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
                         wv[i] = pv * vsc[j][i];
                         wmax = fmaxf(wmax, wv[i]);
                     }
-                    psum = t12_wave_sum(psum);
+                    psum = wave_sum_dpp(psum);
                     wmax = wave_max(wmax);
                     const float inv = wmax > 0.0f ? 127.0f / wmax : 0.0f;
 #pragma unroll
@@ -1019,7 +1037,7 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
                         if (t < tl) ph[t] = pv;
                         psum += pv;
                     }
-                    psum = t12_wave_sum(psum);
+                    psum = wave_sum_dpp(psum);
                     l_run[j] = l_run[j] * corr + psum;
                     m_run[j] = m_new;
     #pragma unroll
