@@ -604,10 +604,23 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
     }
 
     constexpr int QSTR = HD + 16;               // row pitch of qlimb, for the same reason as WSTR
+    // QREGC: the fused form rotates head w's 128 values in wave w's registers (two per lane), so the wave derives the
+    // head's limbs there and then, without the round trip through qs and its barrier; the rows it writes are left out
+    // of the clearing below (other threads' zeros and this wave's limbs would race).
+    constexpr bool QREGC = FUSE && WIDE && RATIO * (HD / 2) == 256 && HD == 128;
     __shared__ __attribute__((aligned(16))) int8_t qlimb[WIDE ? 32 * QSTR : 16];
     __shared__ float qscale[RATIO];
-    if constexpr (WIDE)
-        for (int i = tid; i < 32 * QSTR / 16; i += 256) ((uint4*)qlimb)[i] = make_uint4(0, 0, 0, 0);
+    constexpr int WSTR = ATT_TILE + 16;         // row pitch of wq: 32 lanes reading 16 bytes of 32 different rows, no bank shared
+    __shared__ __attribute__((aligned(16))) int8_t wq[WIDE ? 32 * WSTR : 16];
+    if constexpr (WIDE) {
+        // both operand buffers are cleared here, under the latency of the requests above (the rows no head writes must
+        // read as zero); the barrier behind the Q loads covers them
+        for (int i = tid; i < 32 * QSTR / 16; i += 256) {
+            const int row = i / (QSTR / 16);
+            if (!QREGC || (row & 7) >= RATIO || row >= 24) ((uint4*)qlimb)[i] = make_uint4(0, 0, 0, 0);
+        }
+        for (int i = tid; i < 32 * WSTR / 16; i += 256) ((uint4*)wq)[i] = make_uint4(0, 0, 0, 0);
+    }
     if (!FUSE) {
         for (int i = tid; i < RATIO * HD; i += 256) qs[i] = qb[i];
     } else {
@@ -634,7 +647,28 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
         }
         float sn, cs;
         sincosf((float)pos * freq, &sn, &cs);
-        if (qfirst) rope_rotate(qx0, qx1, sn, cs, qs[(tid / HALF) * HD + d], qs[(tid / HALF) * HD + d + HALF]);
+        if constexpr (QREGC) {
+            float q0, q1;
+            rope_rotate(qx0, qx1, sn, cs, q0, q1);
+            const int h = wave;
+            const float amaxq = wave_max(fmaxf(fabsf(q0), fabsf(q1)));
+            const float invq = amaxq > 0.0f ? 127.0f / amaxq : 0.0f;
+            auto limbs = [&](float qv, int dd) {
+                const float s0 = qv * invq;
+                const float a1 = fminf(fmaxf(rintf(s0), -127.0f), 127.0f);
+                const float s1 = (s0 - a1) * 254.0f;
+                const float a2 = fminf(fmaxf(rintf(s1), -127.0f), 127.0f);
+                const float a3 = fminf(fmaxf(rintf((s1 - a2) * 254.0f), -127.0f), 127.0f);
+                qlimb[h * QSTR + dd] = (int8_t)(int)a1;
+                qlimb[(8 + h) * QSTR + dd] = (int8_t)(int)a2;
+                qlimb[(16 + h) * QSTR + dd] = (int8_t)(int)a3;
+            };
+            limbs(q0, lane);
+            limbs(q1, lane + HALF);
+            if (lane == 0) qscale[h] = amaxq / 127.0f;
+        } else if (qfirst) {
+            rope_rotate(qx0, qx1, sn, cs, qs[(tid / HALF) * HD + d], qs[(tid / HALF) * HD + d + HALF]);
+        }
         for (int i = tid + 256; i < RATIO * HALF; i += 256) {        // (more than 256 pairs: GQA ratios above 4 at head_dim 128)
             const int h = i / HALF;
             const float x0 = qb[h * HD + d], x1 = qb[h * HD + d + HALF];
@@ -687,7 +721,7 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
     // 8 * limb + h (the 32 rows of the MFMA are there anyway).
     // INT8 x INT8 products accumulate exactly in int32, so K needs no conversion at all.
     // (qlimb was cleared ahead of the Q loads, under their latency; the barrier above covers it)
-    if constexpr (WIDE) {
+    if constexpr (WIDE && !QREGC) {
     for (int h = wave; h < RATIO; h += 4) {
         float amax = 0.0f;
         for (int d = lane; d < HD; d += 64) amax = fmaxf(amax, fabsf(qs[h * HD + d]));
@@ -732,8 +766,6 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
     constexpr int VSTR = HD + 16;
     constexpr int NBLK = HD / 32;               // dim blocks = waves busy in this phase
     __shared__ __attribute__((aligned(16))) int8_t vth[WIDE ? 128 * VSTR : 16];
-    constexpr int WSTR = ATT_TILE + 16;         // row pitch of wq: 32 lanes reading 16 bytes of 32 different rows, no bank shared
-    __shared__ __attribute__((aligned(16))) int8_t wq[WIDE ? 32 * WSTR : 16];
     __shared__ float wscale_s[RATIO];
     float o_w[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     constexpr int VP = WIDE ? 128 * CH / 256 : 1;   // 16-byte V pieces per thread and half tile
@@ -783,10 +815,6 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
                 dst[j][i] = (wave + 4 * j < RATIO && t < tlx) ? svb[(size_t)(t0x + t) * ssr] : 0.0f;
             }
     };
-    if constexpr (WIDE) {
-        for (int i = tid; i < 32 * WSTR / 16; i += 256) ((uint4*)wq)[i] = make_uint4(0, 0, 0, 0);
-        __syncthreads();
-    }
     const int g = lane / CH, c = lane % CH;     // phase 3: position class, 16-dim chunk
     if constexpr (WIDE) {
         issue_k(c0, tl0, true);
