@@ -604,10 +604,11 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
     }
 
     constexpr int QSTR = HD + 16;               // row pitch of qlimb, for the same reason as WSTR
-    // QREGC: the fused form rotates head w's 128 values in wave w's registers (two per lane), so the wave derives the
-    // head's limbs there and then, without the round trip through qs and its barrier; the rows it writes are left out
-    // of the clearing below (other threads' zeros and this wave's limbs would race).
-    constexpr bool QREGC = FUSE && WIDE && RATIO * (HD / 2) == 256 && HD == 128;
+    // QREG (four query heads of 128 dims): wave w holds head w's 128 values in registers, two per lane -- the fused form
+    // has just rotated them there, the other form loads them that way -- and derives the head's limbs there and then,
+    // without the round trip through qs and its barrier; the rows it writes are left out of the clearing below (other
+    // threads' zeros and this wave's limbs would race).
+    constexpr bool QREG = WIDE && RATIO == 4 && HD == 128;
     __shared__ __attribute__((aligned(16))) int8_t qlimb[WIDE ? 32 * QSTR : 16];
     __shared__ float qscale[RATIO];
     constexpr int WSTR = ATT_TILE + 16;         // row pitch of wq: 32 lanes reading 16 bytes of 32 different rows, no bank shared
@@ -617,12 +618,35 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
         // read as zero); the barrier behind the Q loads covers them
         for (int i = tid; i < 32 * QSTR / 16; i += 256) {
             const int row = i / (QSTR / 16);
-            if (!QREGC || (row & 7) >= RATIO || row >= 24) ((uint4*)qlimb)[i] = make_uint4(0, 0, 0, 0);
+            if (!QREG || (row & 7) >= RATIO || row >= 24) ((uint4*)qlimb)[i] = make_uint4(0, 0, 0, 0);
         }
         for (int i = tid; i < 32 * WSTR / 16; i += 256) ((uint4*)wq)[i] = make_uint4(0, 0, 0, 0);
     }
+    // head `wave`, values q0 = dim lane and q1 = dim lane + 64: s_h = max|q_h| / 127 and the three limbs (see below)
+    auto limbs_from_registers = [&](float q0, float q1) __attribute__((always_inline)) {
+        const int h = wave;
+        const float amaxq = wave_max(fmaxf(fabsf(q0), fabsf(q1)));
+        const float invq = amaxq > 0.0f ? 127.0f / amaxq : 0.0f;
+        auto limbs = [&](float qv, int dd) {
+            const float s0 = qv * invq;
+            const float a1 = fminf(fmaxf(rintf(s0), -127.0f), 127.0f);
+            const float s1 = (s0 - a1) * 254.0f;
+            const float a2 = fminf(fmaxf(rintf(s1), -127.0f), 127.0f);
+            const float a3 = fminf(fmaxf(rintf((s1 - a2) * 254.0f), -127.0f), 127.0f);
+            qlimb[h * QSTR + dd] = (int8_t)(int)a1;
+            qlimb[(8 + h) * QSTR + dd] = (int8_t)(int)a2;
+            qlimb[(16 + h) * QSTR + dd] = (int8_t)(int)a3;
+        };
+        limbs(q0, lane);
+        limbs(q1, lane + 64);
+        if (lane == 0) qscale[h] = amaxq / 127.0f;
+    };
     if (!FUSE) {
-        for (int i = tid; i < RATIO * HD; i += 256) qs[i] = qb[i];
+        if constexpr (QREG) {
+            limbs_from_registers(qb[wave * HD + lane], qb[wave * HD + lane + 64]);
+        } else {
+            for (int i = tid; i < RATIO * HD; i += 256) qs[i] = qb[i];
+        }
     } else {
         constexpr int HALF = HD / 2;
         static_assert(256 % HALF == 0, "a thread keeps one rotation angle");
@@ -647,25 +671,10 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
         }
         float sn, cs;
         sincosf((float)pos * freq, &sn, &cs);
-        if constexpr (QREGC) {
+        if constexpr (QREG) {
             float q0, q1;
             rope_rotate(qx0, qx1, sn, cs, q0, q1);
-            const int h = wave;
-            const float amaxq = wave_max(fmaxf(fabsf(q0), fabsf(q1)));
-            const float invq = amaxq > 0.0f ? 127.0f / amaxq : 0.0f;
-            auto limbs = [&](float qv, int dd) {
-                const float s0 = qv * invq;
-                const float a1 = fminf(fmaxf(rintf(s0), -127.0f), 127.0f);
-                const float s1 = (s0 - a1) * 254.0f;
-                const float a2 = fminf(fmaxf(rintf(s1), -127.0f), 127.0f);
-                const float a3 = fminf(fmaxf(rintf((s1 - a2) * 254.0f), -127.0f), 127.0f);
-                qlimb[h * QSTR + dd] = (int8_t)(int)a1;
-                qlimb[(8 + h) * QSTR + dd] = (int8_t)(int)a2;
-                qlimb[(16 + h) * QSTR + dd] = (int8_t)(int)a3;
-            };
-            limbs(q0, lane);
-            limbs(q1, lane + HALF);
-            if (lane == 0) qscale[h] = amaxq / 127.0f;
+            limbs_from_registers(q0, q1);
         } else if (qfirst) {
             rope_rotate(qx0, qx1, sn, cs, qs[(tid / HALF) * HD + d], qs[(tid / HALF) * HD + d + HALF]);
         }
@@ -721,7 +730,7 @@ __global__ __launch_bounds__(256, FUSE ? 1 : (WIDE ? 3 : 4)) void attn_fast_kern
     // 8 * limb + h (the 32 rows of the MFMA are there anyway).
     // INT8 x INT8 products accumulate exactly in int32, so K needs no conversion at all.
     // (qlimb was cleared ahead of the Q loads, under their latency; the barrier above covers it)
-    if constexpr (WIDE && !QREGC) {
+    if constexpr (WIDE && !QREG) {
     for (int h = wave; h < RATIO; h += 4) {
         float amax = 0.0f;
         for (int d = lane; d < HD; d += 64) amax = fmaxf(amax, fabsf(qs[h * HD + d]));
