@@ -101,8 +101,8 @@ __global__ __launch_bounds__(256) void compat_batch_kernel(const uint8_t* __rest
 {
     __shared__ int wave_tot[4];
     __shared__ float red[4][NB];
-    compat_row_256<NB>(sm, gr, base_exp, bp, esc_row_base, esc_counts, esc_vals, blockIdx.x, K, threadIdx.x, true, wave_tot,
-                       red);
+    compat_row_256<NB>(sm, gr, base_exp, bp, esc_row_base, esc_counts, esc_vals, blockIdx.x, K, threadIdx.x,
+                       (int)blockIdx.x < M, wave_tot, red);
 }
 
 // ---------------------------------------------------------------------------
