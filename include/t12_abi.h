@@ -180,7 +180,9 @@ int t12_gemm_grouped(const T12Group* groups, int ngroups, int K, void* stream);
  * is taken in a fixed order.  The call never waits for the stream: the grouped launches read the rows per expert from
  * the routing kernel's tables on the device (one workgroup per row tile, which walks the expert's batch tiles; with
  * few rows per expert -- a decode step -- the small-batch kernel that sweeps 16 whole weight rows per workgroup, and
- * an expert nobody names costs a workgroup's exit).  An id
+ * an expert nobody names costs a workgroup's exit; with at most eight (token, expert) pairs on at most eight experts
+ * of 2048 columns and more, every pair is one matrix-vector product with its expert's tensors, picked on the device,
+ * gate|up with the SwiGLU in the epilogue).  An id
  * outside 0..E-1 leaves its pair out of the sum and raises a flag that t12_moe_status reads (it waits for the stream).
  * Shapes the tile kernel does not take (n_embd or n_ff not a multiple of 64, base_exp outside 0..240) copy the counts
  * to the host and wait once per call.

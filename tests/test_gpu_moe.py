@@ -278,3 +278,36 @@ def test_moe_few_rows_per_expert_and_one_expert_above_sixteen(t12, oracle, synth
             a = oracle.silu_mul_bf16(oracle.gemm(packs[e][0], X[rows]), oracle.gemm(packs[e][1], X[rows]))
             ref[rows] += w_h[rows, slots][:, None].astype(np.float64) * oracle.gemm(packs[e][2], a)
         assert rel_err(got, ref) < 1e-4, (T, k)
+
+
+def test_moe_handful_of_pairs_runs_matrix_vector_products(t12, oracle, synth, moe):
+    """Up to eight (token, expert) pairs on at most eight experts of 2048 columns and more: each slot is one
+    matrix-vector product with the tensors of its expert, picked on the device (gate|up with the SwiGLU in the
+    epilogue, then down).  One token with top-2 and top-1, four tokens that share experts, a pair list that names one
+    expert in every slot, an id out of range (left out, flagged), rows of 2048 and 2560 columns with escapes."""
+    E, n, n_ff, seed = 8, 2048, 2560, 2400
+    packs = [[oracle.pack(synth.weights_llm(m, kk, seed=seed + 3 * e + j, p_outlier=1e-3))
+              for j, (m, kk) in enumerate([(n_ff, n), (n_ff, n), (n, n_ff)])] for e in range(E)]
+    layer = moe.MoeLayer([moe.Expert(*[t12.DeviceTensor12.from_packed(p, dev()) for p in ps]) for ps in packs])
+    rng = np.random.default_rng(seed)
+    cases = [np.array([[5, 2]], np.int32), np.array([[7]], np.int32),
+             np.array([[0, 3], [3, 1], [6, 0], [3, 7]], np.int32), np.full((8, 1), 4, np.int32),
+             np.array([[1, 9], [2, 1]], np.int32)]
+    for ids_h in cases:
+        T, k = ids_h.shape
+        X = synth.activations(T, n, seed=seed + 11 * T + k)
+        w_h = rng.random((T, k)).astype(np.float32)
+        got = layer(to_dev_bits(X).reshape(T, n), torch.from_numpy(ids_h).to(dev()), torch.from_numpy(w_h).to(dev())).cpu().numpy()
+        if (ids_h >= E).any():
+            with pytest.raises(t12.T12Error):
+                layer.status()
+        else:
+            layer.status()
+        ref = np.zeros((T, n), np.float64)
+        for e in range(E):
+            rows, slots = np.nonzero(ids_h == e)
+            if len(rows) == 0:
+                continue
+            a = oracle.silu_mul_bf16(oracle.gemm(packs[e][0], X[rows]), oracle.gemm(packs[e][1], X[rows]))
+            ref[rows] += w_h[rows, slots][:, None].astype(np.float64) * oracle.gemm(packs[e][2], a)
+        assert rel_err(got, ref) < 1e-4, ids_h.tolist()

@@ -21,8 +21,10 @@
 
 namespace {
 
+constexpr int GEMV_SEGS = 16;              // a mixture-of-experts launch carries (gate, up) of up to eight experts
+
 struct GemvParams {
-    T12Segment seg[T12_MAX_SEGMENTS];
+    T12Segment seg[GEMV_SEGS];
     int blk_start[T12_MAX_SEGMENTS + 1];   // first workgroup of each segment
     int nseg;
     int K;
@@ -35,6 +37,10 @@ struct GemvParams {
     const float* nw;
     float* hidden_out;                     // nx + nres, written by workgroup 0 (may be null)
     float eps;
+    // MOE launches (gridDim.y activation rows, each with the expert the routing gave it):
+    const int* slot_expert;                // [gridDim.y] on the device; a negative entry = no row, the workgroup leaves
+    int act_stride;                        // bf16 elements between activation rows
+    int out_ld;                            // elements between output rows (fp32 outputs and out_bf16)
 };
 
 __device__ __forceinline__ int find_segment(const GemvParams& p, int blk)
@@ -102,10 +108,19 @@ __device__ __forceinline__ float lds_act_at(const uint4* lds_act, int k)
 // workgroup rebuilds them from the fp32 residual stream while its first weight tiles are in
 // flight -- the reference's (add_)rms_norm_bf16_batch kernels (engine/kernels.hip:355-442) as a
 // prologue.  K <= 16 * NW * 64.  Workgroup 0 also stores nx + nres for the residual path.
-template <int NW, int R, int D, int MINB, bool SWIGLU = false, int NORM = 0>
+// MOE: one activation row per blockIdx.y, multiplied with the tensors of the expert slot_expert[blockIdx.y] names --
+// segment e (SWIGLU: segments 2e and 2e + 1); rows of activations and outputs are act_stride / out_ld apart.
+template <int NW, int R, int D, int MINB, bool SWIGLU = false, int NORM = 0, bool MOE = false>
 __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvParams p)
 {
     static_assert(!SWIGLU || R == 2, "the SwiGLU epilogue pairs exactly two rows");
+    static_assert(!MOE || NORM == 0, "expert launches take bf16 activations");
+    int expert = 0;
+    if (MOE) {
+        expert = __builtin_amdgcn_readfirstlane(p.slot_expert[blockIdx.y]);
+        if (expert < 0) return;                // (the whole workgroup: no barrier has been reached)
+    }
+    const uint16_t* const act_row = MOE ? p.act + (size_t)blockIdx.y * p.act_stride : p.act;
     extern __shared__ uint4 lds_act[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K = p.K;
@@ -113,13 +128,13 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
     const int nchunk = (K + 1023) >> 10;
 
     const int blk = blockIdx.x;
-    const int s = SWIGLU ? 0 : find_segment(p, blk);
+    const int s = MOE ? (SWIGLU ? 2 * expert : expert) : (SWIGLU ? 0 : find_segment(p, blk));
     const T12Segment& sg = p.seg[s];
     const int M = sg.M;
     // row r of this wave: tensor SEG(r), matrix row ROW(r)
-#define SEG(r) (SWIGLU ? p.seg[r] : sg)
+#define SEG(r) (SWIGLU ? p.seg[(MOE ? s : 0) + (r)] : sg)
 #define ROW(r) (SWIGLU ? row0 : row0 + (r))
-    const int row0 = SWIGLU ? blk * NW + wave : (blk - p.blk_start[s]) * (NW * R) + wave * R;
+    const int row0 = SWIGLU ? blk * NW + wave : (blk - (MOE ? 0 : p.blk_start[s])) * (NW * R) + wave * R;
     const bool live = row0 < M;                // wave-uniform
     uint32_t be2r[R];
 #pragma unroll
@@ -137,7 +152,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
             const int k = (tid + u * NW * 64) * 8;
             xpre[u] = make_uint4(0, 0, 0, 0);
             if (u == 0 || u * NW * 64 * 8 < K)                       // workgroup-uniform
-                xpre[u] = *(const uint4*)(p.act + min(k, K - 8));    // (clamped: columns >= K are zeroed below)
+                xpre[u] = *(const uint4*)(act_row + min(k, K - 8));  // (clamped: columns >= K are zeroed below)
         }
     }
 
@@ -212,7 +227,7 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
         for (int q = tid + SU * NW * 64; q < nchunk * 128; q += NW * 64) {     // K beyond the pieces requested up front
             const int k = q * 8;
             uint4 v = make_uint4(0, 0, 0, 0);
-            if (k < K) v = *(const uint4*)(p.act + k);
+            if (k < K) v = *(const uint4*)(act_row + k);
             lds_act[(q >> 7) * 128 + (q & 1) * 64 + ((q & 127) >> 1)] = t12_pair_acts(v);
         }
     } else {
@@ -330,12 +345,15 @@ __global__ __launch_bounds__(NW * 64, MINB) void gemv_stream_kernel(const GemvPa
                 v += (t12_bf16_to_f32((uint16_t)SEG(r).correct[q]) - t12_bf16_to_f32((uint16_t)SEG(r).wrong[q])) *
                      lds_act_at(lds_act, SEG(r).cols[q]);
             tot[r] = t12_wave_sum_lane63(v);
-            if (!SWIGLU && lane == 63) sg.out[row0 + r] = p.add ? tot[r] + p.add[row0 + r] : tot[r];
+            if (!SWIGLU && lane == 63) {
+                if (MOE) sg.out[(size_t)blockIdx.y * p.out_ld + row0 + r] = tot[r];
+                else sg.out[row0 + r] = p.add ? tot[r] + p.add[row0 + r] : tot[r];
+            }
         }
     }
     if (SWIGLU && lane == 63) {
         const float g = tot[0];
-        p.out_bf16[row0] = t12_f32_to_bf16(g / (1.0f + expf(-g)) * tot[R - 1]);
+        (MOE ? p.out_bf16 + (size_t)blockIdx.y * p.out_ld : p.out_bf16)[row0] = t12_f32_to_bf16(g / (1.0f + expf(-g)) * tot[R - 1]);
     }
 #undef SEG
 #undef ROW
@@ -617,6 +635,47 @@ int t12_gemv_swiglu_norm(const T12Segment* gate, const T12Segment* up, const flo
     p.hidden_out = hidden_out;
     p.eps = eps;
     return residual ? launch_swiglu<2>(p, (hipStream_t)stream) : launch_swiglu<1>(p, (hipStream_t)stream);
+}
+
+// One activation row per slot, each multiplied with the tensors of the expert the routing gave the slot (a device
+// table): the few-row step of a mixture-of-experts layer, where every named expert is streamed at the rate of the B = 1
+// kernel.  per_expert = 2: segs = (gate, up) per expert, out_bf16[slot, m] = bf16(silu(gate . x) * (up . x));
+// per_expert = 1: segs[e].out[slot * out_ld + m] = W_e[m, :] . x_slot.  Returns 1 when the shape has no such kernel
+// (K not a multiple of 16 or under two tiles, base_exp outside 0..240, more than sixteen segments, misaligned rows).
+__attribute__((visibility("hidden"))) int t12_gemv_experts(const T12Segment* segs, int per_expert, int E, int K,
+                                                           const void* act_bf16, int act_stride, const int* slot_expert,
+                                                           int slots, void* out_bf16, int out_ld, void* stream)
+{
+    if (per_expert < 1 || per_expert > 2 || E < 1 || E * per_expert > GEMV_SEGS || slots < 1) return 1;
+    if (K % 16 != 0 || K < 2048 || (size_t)((K + 1023) / 1024) * 2048 > 160 * 1024) return 1;
+    if (act_stride % 8 != 0 || (uintptr_t)act_bf16 % 16 != 0) return 1;
+    const int M = segs[0].M;
+    GemvParams p;
+    for (int i = 0; i < E * per_expert; i++) {
+        const T12Segment& g = segs[i];
+        if (g.M != M || !g.sm || !g.gr || g.base_exp < 0 || g.base_exp > 240) return 1;
+        if (g.row_off && !(g.cols && g.correct && g.wrong)) return 1;
+        if (per_expert == 1 && !g.out) return 1;
+        p.seg[i] = g;
+    }
+    if (per_expert == 2 && !out_bf16) return 1;
+    p.nseg = E * per_expert;
+    p.K = K;
+    p.act = (const uint16_t*)act_bf16;
+    p.out_bf16 = (uint16_t*)out_bf16;
+    p.add = nullptr;
+    p.slot_expert = slot_expert;
+    p.act_stride = act_stride;
+    p.out_ld = out_ld;
+    const int NW = 8;
+    const size_t lds = (size_t)((K + 1023) / 1024) * 2048;
+    const dim3 grid((M + NW - 1) / NW, slots);
+    if (per_expert == 2)
+        hipLaunchKernelGGL((gemv_stream_kernel<8, 2, 2, 1, true, 0, true>), grid, dim3(NW * 64), lds, (hipStream_t)stream, p);
+    else
+        hipLaunchKernelGGL((gemv_stream_kernel<8, 1, 2, 1, false, 0, true>), grid, dim3(NW * 64), lds, (hipStream_t)stream, p);
+    T12_CHECK_LAUNCH("t12_moe_ffn(gemv)");
+    return T12_OK;
 }
 
 // ---- reference-named launchers ---------------------------------------------

@@ -29,20 +29,27 @@ extern "C" __attribute__((visibility("hidden"))) int t12_gemm_experts(const T12S
                                                                       int first_group, int hint_b, int pairs,
                                                                       void* out_bf16, int out_bf16_ld, void* stream);
 
+extern "C" __attribute__((visibility("hidden"))) int t12_gemv_experts(const T12Segment* segs, int per_expert, int E, int K,
+                                                                      const void* act_bf16, int act_stride,
+                                                                      const int* slot_expert, int slots, void* out_bf16,
+                                                                      int out_ld, void* stream);
+
 namespace {
 
 constexpr int ROUTE_THREADS = 256;
+constexpr int FEW_SLOTS = 8;          // up to this many (token, expert) pairs every slot is its own matrix-vector product
 constexpr int MAX_EXPERTS = 128;      // the sort keeps a 257-entry count row per expert in LDS (132 KB at 128 experts)
 
 // One workgroup.  Thread i owns the pairs [i * chunk, (i + 1) * chunk); pairs of one expert keep their order
 // (pair index ascending), so the grouping is the same on every run.  counts[e] = pairs of expert e, base[e] = its
-// first slot (base[E] = pairs placed); slots past the placed pairs get pair -1.  *bad = 1 if an id lies outside 0..E-1
+// first slot (base[E] = pairs placed), expert_of_slot[slot] = the expert whose range holds the slot; slots past the
+// placed pairs get pair -1 and expert -1.  *bad = 1 if an id lies outside 0..E-1
 // (such a pair gets no slot and contributes nothing).
 template <typename IdT>
 __global__ __launch_bounds__(ROUTE_THREADS) void moe_route_kernel(const IdT* __restrict__ ids, int P, int E,
                                                                   int* __restrict__ counts, int* __restrict__ base,
                                                                   int* __restrict__ pair_of_slot, int* __restrict__ slot_of_pair,
-                                                                  int* __restrict__ bad)
+                                                                  int* __restrict__ expert_of_slot, int* __restrict__ bad)
 {
     extern __shared__ int route_lds[];
     constexpr int LD = ROUTE_THREADS + 1;
@@ -102,11 +109,15 @@ __global__ __launch_bounds__(ROUTE_THREADS) void moe_route_kernel(const IdT* __r
             const int slot = ebase[(int)e] + cnt[(int)e * LD + tid]++;
             pair_of_slot[slot] = q;
             slot_of_pair[q] = slot;
+            expert_of_slot[slot] = (int)e;
         } else {
             slot_of_pair[q] = -1;
         }
     }
-    for (int slot = ebase[E] + tid; slot < P; slot += ROUTE_THREADS) pair_of_slot[slot] = -1;
+    for (int slot = ebase[E] + tid; slot < P; slot += ROUTE_THREADS) {
+        pair_of_slot[slot] = -1;
+        expert_of_slot[slot] = -1;
+    }
 }
 
 // Xg[slot, :] = X[pair_of_slot[slot] / k, :]; one workgroup per slot, 16 bytes per thread and step.
@@ -144,7 +155,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct MoeLayout {
-    size_t bad, counts, base, pair_of_slot, slot_of_pair, xg, gate, up, act, y, total;
+    size_t bad, counts, base, pair_of_slot, slot_of_pair, expert_of_slot, xg, gate, up, act, y, total;
 };
 
 MoeLayout moe_layout(int T, int k, int n_embd, int n_ff, int E)
@@ -157,6 +168,7 @@ MoeLayout moe_layout(int T, int k, int n_embd, int n_ff, int E)
     l.base = o;          o = align256(o + sizeof(int) * (size_t)(E + 1));
     l.pair_of_slot = o;  o = align256(o + sizeof(int) * P);
     l.slot_of_pair = o;  o = align256(o + sizeof(int) * P);
+    l.expert_of_slot = o; o = align256(o + sizeof(int) * P);
     l.xg = o;            o = align256(o + 2 * P * n_embd);
     l.gate = o;          o = align256(o + 4 * P * n_ff);
     l.up = o;            o = align256(o + 4 * P * n_ff);
@@ -260,6 +272,7 @@ int t12_moe_ffn(const T12MoeExpert* experts, int E, const void* x_bf16, int x_st
     int* bad = (int*)(ws + l.bad);
     int* pair_of_slot = (int*)(ws + l.pair_of_slot);
     int* slot_of_pair = (int*)(ws + l.slot_of_pair);
+    int* expert_of_slot = (int*)(ws + l.expert_of_slot);
     uint16_t* xg = (uint16_t*)(ws + l.xg);
     float* gate = (float*)(ws + l.gate);
     float* up = (float*)(ws + l.up);
@@ -275,7 +288,7 @@ int t12_moe_ffn(const T12MoeExpert* experts, int E, const void* x_bf16, int x_st
             return T12_ELAUNCH;
         }
         hipLaunchKernelGGL(fn, dim3(1), dim3(ROUTE_THREADS), route_lds, st, (const int32_t*)expert_ids, P, E, counts, base,
-                           pair_of_slot, slot_of_pair, bad);
+                           pair_of_slot, slot_of_pair, expert_of_slot, bad);
     } else {
         auto fn = moe_route_kernel<long long>;
         if (route_lds > 48 * 1024 && hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)route_lds) != hipSuccess) {
@@ -283,7 +296,7 @@ int t12_moe_ffn(const T12MoeExpert* experts, int E, const void* x_bf16, int x_st
             return T12_ELAUNCH;
         }
         hipLaunchKernelGGL(fn, dim3(1), dim3(ROUTE_THREADS), route_lds, st, (const long long*)expert_ids, P, E, counts, base,
-                           pair_of_slot, slot_of_pair, bad);
+                           pair_of_slot, slot_of_pair, expert_of_slot, bad);
     }
     T12_CHECK_LAUNCH("t12_moe_ffn(route)");
     hipLaunchKernelGGL(moe_gather_kernel, dim3(P), dim3(256), 0, st, (const uint16_t*)x_bf16, x_stride, pair_of_slot, k, n_embd, xg);
@@ -294,6 +307,41 @@ int t12_moe_ffn(const T12MoeExpert* experts, int E, const void* x_bf16, int x_st
     //      above the tile streams its planes once per tile it needs, so a tile below the typical maximum costs more than
     //      a tile above it).  Above 128 rows the SwiGLU goes into the gate|up epilogue; below, the 128-row SwiGLU tile is
     //      slower than two plain groups and the SiLU*mul kernel (Mixtral shape, ~64 rows per expert: 490 against 468 us).
+    // ---- a handful of pairs (a decode step of one or a few sequences): every slot is one matrix-vector product with
+    //      its expert's tensors, picked on the device -- gate|up with the SwiGLU in the epilogue, then down.  Each named
+    //      expert is streamed once per slot that names it, at the rate of the B = 1 kernel (Mixtral shape, one token:
+    //      0.16 -> 0.10 ms against the 16-row sweep below, which also starts a workgroup for every row group of every
+    //      expert nobody named).
+    if (P <= FEW_SLOTS && 2 * E <= 16 && n_embd % 16 == 0 && n_ff % 16 == 0 && n_embd >= 2048 && n_ff >= 2048) {
+        T12Segment sg[16];
+        bool ok = true;
+        for (int e = 0; e < E; e++) {
+            sg[2 * e] = experts[e].w1;
+            sg[2 * e + 1] = experts[e].w3;
+            for (const T12Segment* g : {&experts[e].w1, &experts[e].w3, &experts[e].w2})
+                if (g->base_exp < 0 || g->base_exp > 240 || !g->sm || !g->gr) ok = false;
+        }
+        if (ok) {
+            int rc = t12_gemv_experts(sg, 2, E, n_embd, xg, n_embd, expert_of_slot, P, act, n_ff, stream);
+            if (rc < 0) return rc;
+            if (rc == 0) {
+                for (int e = 0; e < E; e++) {
+                    sg[e] = experts[e].w2;
+                    sg[e].out = y;
+                }
+                rc = t12_gemv_experts(sg, 1, E, n_ff, act, n_ff, expert_of_slot, P, nullptr, n_embd, stream);
+                if (rc < 0) return rc;
+                if (rc == 0) {
+                    hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, st, y, slot_of_pair, weights, k, n_embd, out,
+                                       out_stride);
+                    T12_CHECK_LAUNCH("t12_moe_ffn(combine)");
+                    return T12_OK;
+                }
+                // (the down projection has no such kernel: the grouped path below redoes the layer)
+            }
+        }
+    }
+
     const double mean = (double)P / E;
     const int hint = (int)fmin((double)P, ceil(mean + 4.0 * sqrt(mean * (1.0 - 1.0 / E))));
     const bool fuse_swiglu = hint > 128;
