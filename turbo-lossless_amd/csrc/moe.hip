@@ -13,6 +13,8 @@
 //   5. moe_combine_kernel  out[t] = sum_j weights[t, j] * Y[slot(t, j)]  (j ascending: a fixed order, no atomics)
 // The grouped launches read the rows per expert from the routing kernel's tables on the device: one workgroup per row
 // tile, which walks the expert's batch tiles (one, unless the expert received more rows than the tile holds).
+// A call with at most eight pairs (a decode step of a few sequences) replaces 3 and 4 by two launches of the B = 1
+// kernel over (row groups, slots): every slot multiplies its row with the tensors of its expert, read from the table.
 // Shapes the tile kernel does not take (K not a multiple of 64, base_exp outside 0..240) size their launches on the
 // host instead: one copy of the counts and one wait per call.
 
