@@ -93,6 +93,7 @@ struct GemmParams {
     const int* dev_counts = nullptr;
     const int* dev_base = nullptr;
     int group_of_seg[GMAX];
+    int n_first = 0;                       // mixed small-batch launch: segments [0, n_first) take the larger workgroups
 };
 
 // LDS slot of (unit, row) in a [units][rows] array of 16-byte units.  Rows are rotated
@@ -664,10 +665,9 @@ __global__ __launch_bounds__(256) void gemm_general_kernel(const GemmParams p)
 // the segment's group has dev_counts[g] batch rows starting dev_base[g] rows into the activations and the outputs; a
 // workgroup of a group without rows exits at once, one of a group above 16 rows sweeps its weight rows once per 16.
 // ---------------------------------------------------------------------------
-template <int NW, int D, int RG, bool DEV = false>
-__global__ __launch_bounds__(NW * 64) void gemm_dense16_kernel(const GemmParams p)
+template <int NW, int D, int RG, bool DEV>
+__device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4 (*red)[NW][64])
 {
-    __shared__ t12_f32x4 red[RG][NW][64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, g = lane >> 4;
 
@@ -815,6 +815,27 @@ __global__ __launch_bounds__(NW * 64) void gemm_dense16_kernel(const GemmParams 
     }
     if (DEV && b_first + 16 < b_all) __syncthreads();        // the next 16 batch rows reuse the reduction buffer
     }
+}
+
+template <int NW, int D, int RG, bool DEV = false>
+__global__ __launch_bounds__(NW * 64) void gemm_dense16_kernel(const GemmParams p)
+{
+    __shared__ t12_f32x4 red[RG][NW][64];
+    gemm_dense16_body<NW, D, RG, DEV>(p, red);
+}
+
+// The same sweep with two sizes of workgroup in one launch.  With RGA row groups per workgroup (its registers allow one
+// workgroup per CU) a launch is a sequence of rounds of one workgroup per CU, each as long as a workgroup lives, and a
+// last round that fills a fraction of the chip costs as much as a full one (gate|up at B = 16: 448 workgroups = 256 +
+// 192, two rounds of 23 us).  The host therefore cuts every tensor in two: the first n_first segments of the launch
+// are the heads of the tensors, swept RGA groups per workgroup in whole rounds, the others their tails, swept RGB < RGA
+// groups per workgroup so that the last round covers the chip once with shorter workgroups.
+template <int NW, int D, int RGA, int RGB>
+__global__ __launch_bounds__(NW * 64) void gemm_dense16_mixed_kernel(const GemmParams p)
+{
+    __shared__ t12_f32x4 red[RGA][NW][64];
+    if (find_segment(p, blockIdx.x) < p.n_first) gemm_dense16_body<NW, D, RGA, false>(p, red);
+    else gemm_dense16_body<NW, D, RGB, false>(p, red);
 }
 
 // ---------------------------------------------------------------------------
@@ -1107,6 +1128,90 @@ int t12_gemm_swiglu(const T12Segment* gate, const T12Segment* up, const void* ac
 
 namespace {
 
+// CUs of the current device (a launch of one workgroup per CU is one round of the small-batch kernel).
+int device_cus()
+{
+    static std::mutex mu;
+    static int cus[16] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return 256;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!cus[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
+        cus[dev] = n;
+    }
+    return cus[dev];
+}
+
+// The small-batch launch with rg row groups per workgroup whose last round would fill only part of the chip: every
+// tensor is cut into a head, swept rg groups per workgroup in whole rounds, and a tail swept in fewer groups per
+// workgroup, chosen so that the tails of all tensors together are one round.  p holds the launch as gemm_impl set it up
+// (segments, K, B, activations); returns false, with nothing launched, when the plain launch is as good.
+bool launch_dense16_mixed(GemmParams p, int nseg, int rg, int groups16, hipStream_t st)
+{
+    const int C = device_cus();
+    int sets = 0;
+    for (int i = 0; i < nseg; i++) sets += (p.seg[i].M + 16 * rg - 1) / (16 * rg);
+    // one round or less, whole rounds, or a last round that is nearly full: nothing to gain
+    if (2 * nseg > GMAX || sets <= C || sets % C == 0 || (sets % C) * 8 >= C * 7) return false;
+    const int full = (sets / C) * C;                       // workgroups of the whole rounds
+    int a[GMAX], rem[GMAX], rem_total = 0;
+    for (int i = 0; i < nseg; i++) {
+        const int gi = (p.seg[i].M + 15) / 16;
+        a[i] = (int)((long long)full * gi / groups16);     // this tensor's share of the whole rounds
+        if (a[i] * rg > gi) a[i] = gi / rg;
+        rem[i] = gi - a[i] * rg;
+        rem_total += rem[i];
+    }
+    int rgb = (rem_total + C - 1) / C;
+    for (; rgb >= 1 && rgb < rg; rgb++) {
+        int b = 0;
+        for (int i = 0; i < nseg; i++) b += (rem[i] + rgb - 1) / rgb;
+        if (b <= C) break;
+    }
+    if (rgb < 1 || rgb >= rg) return false;
+    // heads first, then tails.  A tail is the same tensor from row 16 rg a on: the row pointers of the escape list hold
+    // absolute entry numbers, so only the pointer to them moves; 16 rg a rows of K columns are a whole number of bytes of
+    // the nibble plane.
+    T12Segment src[GMAX];
+    for (int i = 0; i < nseg; i++) src[i] = p.seg[i];
+    int n = 0, total = 0;
+    p.n_first = 0;
+    for (int pass = 0; pass < 2; pass++)
+        for (int i = 0; i < nseg; i++) {
+            const int rows_a = min(16 * rg * a[i], src[i].M);
+            const int m = pass == 0 ? rows_a : src[i].M - rows_a;
+            if (m <= 0) continue;
+            T12Segment g = src[i];
+            if (pass == 1) {
+                const size_t e = (size_t)rows_a * p.K;
+                g.sm += e;
+                g.gr += e / 2;
+                if (g.row_off) g.row_off += rows_a;
+                g.out += rows_a;
+            }
+            g.M = m;
+            const int per = 16 * (pass == 0 ? rg : rgb);
+            p.seg[n] = g;
+            p.blk_start[n] = total;
+            total += (m + per - 1) / per;
+            n++;
+            if (pass == 0) p.n_first = n;
+        }
+    p.blk_start[n] = total;
+    p.nseg = n;
+    p.ksplit = 1;
+    p.kslice = p.K;
+    const dim3 grid(total), block(512);
+    if (rg == 4 && rgb == 3) hipLaunchKernelGGL((gemm_dense16_mixed_kernel<8, 2, 4, 3>), grid, block, 0, st, p);
+    else if (rg == 4 && rgb == 2) hipLaunchKernelGGL((gemm_dense16_mixed_kernel<8, 2, 4, 2>), grid, block, 0, st, p);
+    else if (rg == 4 && rgb == 1) hipLaunchKernelGGL((gemm_dense16_mixed_kernel<8, 2, 4, 1>), grid, block, 0, st, p);
+    else if (rg == 2 && rgb == 1) hipLaunchKernelGGL((gemm_dense16_mixed_kernel<8, 2, 2, 1>), grid, block, 0, st, p);
+    else return false;
+    return true;
+}
+
 // The body of t12_gemm / t12_gemm_deferred / t12_gemm_noalloc.  static_ws: the K-split partial sums go to the
 // library's fixed device array instead of a grown hipMalloc buffer, and a launch that needs more is refused.
 int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_stride, int out_stride, int K,
@@ -1202,6 +1307,10 @@ int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_st
         // rows of a padded batch cost no activation traffic, more rows per wave cost registers)
         const int want = B > 8 ? 4 : (B > 4 ? 2 : 1);
         const int rg = groups16 >= 4 * 448 && want >= 4 ? 4 : (groups16 >= 2 * 448 && want >= 2 ? 2 : 1);
+        if (rg > 1 && launch_dense16_mixed(p, nseg, rg, groups16, st)) {
+            T12_CHECK_LAUNCH("t12_gemm(dense16, two workgroup sizes)");
+            return T12_OK;
+        }
         int groups = 0;
         for (int i = 0; i < nseg; i++) {
             p.blk_start[i] = groups;
