@@ -340,6 +340,32 @@ def test_gemm_small_batch_segments_and_strides(t12, oracle, synth):
         off += p.M
 
 
+@pytest.mark.parametrize("B,K", [(7, 256), (16, 128), (11, 384)])
+def test_gemm_small_batch_ragged_segments_head_and_tail_workgroups(t12, oracle, synth, B, K):
+    """Six tensors of unlike, ragged row counts (one of a single row group, one that is no multiple of 16) in one
+    small-batch launch of ~29 000 rows: more workgroups than one round of the chip and a last round that would be
+    partly empty, so the launch cuts every tensor into a head and a tail with fewer row groups per workgroup (the
+    16-row tensor has no head at all).  Every output row must be written once and equal the oracle's."""
+    Ms = [9001, 16, 5000, 1234, 7777, 6000]
+    ps = [oracle.pack(synth.weights_llm(M, K, seed=50 + i, sigma=0.02 * (i + 1), p_outlier=2e-3)) for i, M in enumerate(Ms)]
+    X = synth.activations(B, K, seed=B + K)
+    dts = [t12.DeviceTensor12.from_packed(p, dev()) for p in ps]
+    total = sum(Ms)
+    big = torch.full((B, total + 8), float("nan"), device=dev())
+    outs, off = [], 0
+    for M in Ms:
+        outs.append(big[:, off:off + M])
+        off += M
+    t12.gemm(dts, to_dev_bits(X).reshape(B, K), outs=outs)
+    torch.cuda.synchronize()
+    h = big.cpu().numpy()
+    assert np.isnan(h[:, total:]).all()                      # nothing written past the last tensor
+    off = 0
+    for p, M in zip(ps, Ms):
+        assert rel_err(h[:, off:off + M], oracle.gemm(p, X)) < TOL
+        off += M
+
+
 @pytest.mark.parametrize("B", [2, 3, 4])
 @pytest.mark.parametrize("M,K,law", [(4096, 4096, "llm"), (101, 2048, "diffusion"), (8, 1024, "llm"), (300, 8192, "diffusion")])
 def test_gemm_two_to_four_rows_whole_row_kernel(t12, oracle, synth, M, K, law, B):
