@@ -366,6 +366,49 @@ def test_gemm_small_batch_ragged_segments_head_and_tail_workgroups(t12, oracle, 
         off += M
 
 
+@pytest.mark.parametrize("B", [17, 24, 31, 32])
+@pytest.mark.parametrize("M,K,law", [(4096, 4096, "llm"), (37, 128, "llm"), (1280, 5120, "diffusion"), (8000, 1280, "diffusion"),
+                                     (5000, 4096, "llm"), (2048, 8192, "llm")])
+def test_gemm_17_to_32_rows_two_batch_tiles(t12, oracle, synth, M, K, law, B):
+    """17 .. 32 batch rows on tensors of at most one round of workgroups take the whole-row sweep with two batch tiles
+    per weight load (16 or 32 weight rows per workgroup by row count; long rows fall back to the tile kernel by
+    K x B, so both sides of that rule are among the cases): ragged row counts, a second batch tile with a single row
+    (B = 17), rows with many escapes (the diffusion law), patched and unpatched."""
+    w = synth.weights_diffusion(M, K, seed=M + K) if law == "diffusion" else synth.weights_llm(M, K, seed=M + K, p_outlier=1e-3)
+    p = oracle.pack(w)
+    X = synth.activations(B, K, seed=B)
+    (got,) = run_gemm(t12, [p], X)
+    assert rel_err(got, oracle.gemm(p, X)) < TOL
+    (un,) = run_gemm(t12, [p], X, patched=False)
+    assert rel_err(un, oracle.gemm(p, X, patched=False)) < TOL
+
+
+def test_gemm_17_to_32_rows_segments_and_strides(t12, oracle, synth):
+    """q|k|v-like: three tensors (4096 + 1000 + 1024 rows, three base_exp) in one launch at B = 20, padded activation
+    stride, outputs in column slices of one buffer whose other columns must stay untouched."""
+    K, B = 2048, 20
+    ps = [oracle.pack(synth.weights_llm(4096, K, seed=1, sigma=0.02)), oracle.pack(synth.weights_llm(1000, K, seed=2, sigma=0.3)),
+          oracle.pack(synth.weights_llm(1024, K, seed=3, sigma=0.002, p_outlier=5e-3))]
+    X = synth.activations(B, K, seed=4)
+    Xpad = torch.zeros((B, K + 64), dtype=torch.int16, device=dev())
+    Xpad[:, :K] = to_dev_bits(X).reshape(B, K)
+    dts = [t12.DeviceTensor12.from_packed(p, dev()) for p in ps]
+    total = sum(p.M for p in ps)
+    big = torch.full((B, total + 8), float("nan"), device=dev())
+    outs, off = [], 0
+    for p in ps:
+        outs.append(big[:, off:off + p.M])
+        off += p.M
+    t12.gemm(dts, Xpad[:, :K], outs=outs)
+    torch.cuda.synchronize()
+    h = big.cpu().numpy()
+    assert np.isnan(h[:, total:]).all()
+    off = 0
+    for p in ps:
+        assert rel_err(h[:, off:off + p.M], oracle.gemm(p, X)) < TOL
+        off += p.M
+
+
 @pytest.mark.parametrize("B", [2, 3, 4])
 @pytest.mark.parametrize("M,K,law", [(4096, 4096, "llm"), (101, 2048, "diffusion"), (8, 1024, "llm"), (300, 8192, "diffusion")])
 def test_gemm_two_to_four_rows_whole_row_kernel(t12, oracle, synth, M, K, law, B):

@@ -660,12 +660,14 @@ __global__ __launch_bounds__(256) void gemm_general_kernel(const GemmParams p)
 //   * no barrier until the end, where the waves' partial 16 x 16 tiles are added through LDS in wave order;
 //   * escapes: the streamed value of a group-0 weight is its "wrong" value; wave w adds (correct - wrong) * x[b, col]
 //     for the entries w, w + NW, ... of each row (the four lanes of a row each for their four batch rows).
-// Requires K % 128 == 0, 0 <= base_exp <= 240, B <= 16.  blk_start counts 16-row groups per segment.
+// Requires K % 128 == 0, 0 <= base_exp <= 240, B <= 16 NBT (NBT batch tiles of 16 rows share every weight load and
+// decode; accumulators, activation registers and the reduction buffer grow with NBT).  blk_start counts the workgroups
+// (16 RG rows each) per segment.
 // Rows per group known on the device only (dev_counts, the experts of a mixture-of-experts layer at a few tokens):
 // the segment's group has dev_counts[g] batch rows starting dev_base[g] rows into the activations and the outputs; a
 // workgroup of a group without rows exits at once, one of a group above 16 rows sweeps its weight rows once per 16.
 // ---------------------------------------------------------------------------
-template <int NW, int D, int RG, bool DEV>
+template <int NW, int D, int RG, bool DEV, int NBT = 1>
 __device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4 (*red)[NW][64])
 {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -678,8 +680,8 @@ __device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4
     // DEV: the group's rows from the device tables; otherwise one pass over the launch's B <= 16 rows
     const int b_all = DEV ? p.dev_counts[p.group_of_seg[s]] : 1;
     const int row_base = DEV ? p.dev_base[p.group_of_seg[s]] : 0;
-    for (int b_first = 0; b_first < b_all; b_first += 16) {
-    const int B = DEV ? min(16, b_all - b_first) : p.B;
+    for (int b_first = 0; b_first < b_all; b_first += 16 * NBT) {
+    const int B = DEV ? min(16 * NBT, b_all - b_first) : p.B;
     const uint16_t* const act = DEV ? p.act + (size_t)(row_base + b_first) * p.act_stride : p.act;
     float* const outp = DEV ? sg.out + (size_t)(row_base + b_first) * sg.out_stride : sg.out;
     const int m0 = (blk - p.blk_start[s]) * (16 * RG);               // RG groups of 16 rows share every activation load
@@ -707,12 +709,15 @@ __device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4
         smp[rg] = sg.sm + e0 + 32 * g + (size_t)wblk * 128;
         grp[rg] = sg.gr + (e0 >> 1) + 16 * g + (size_t)wblk * 64;
     }
-    const uint16_t* xp = act + (size_t)min(n, B - 1) * p.act_stride + 32 * g + (size_t)wblk * 128;
-    uint4 rS[D][RG][2], rG[D][RG], rX[D][4];
+    const uint16_t* xp[NBT];                          // NBT tiles of 16 batch rows share every weight load and decode
+#pragma unroll
+    for (int t = 0; t < NBT; t++) xp[t] = act + (size_t)min(16 * t + n, B - 1) * p.act_stride + 32 * g + (size_t)wblk * 128;
+    uint4 rS[D][RG][2], rG[D][RG], rX[D][NBT][4];
 #define T12_DS_FETCH(slot, j)                                                              \
     {                                                                                      \
-        _Pragma("unroll") for (int q = 0; q < 4; q++)                                      \
-            rX[slot][q] = *(const uint4*)(xp + (size_t)(j) * (NW * 128) + 8 * q);          \
+        _Pragma("unroll") for (int t = 0; t < NBT; t++)                                    \
+            _Pragma("unroll") for (int q = 0; q < 4; q++)                                  \
+                rX[slot][t][q] = *(const uint4*)(xp[t] + (size_t)(j) * (NW * 128) + 8 * q); \
         _Pragma("unroll") for (int rg = 0; rg < RG; rg++) {                                \
             rS[slot][rg][0] = *(const uint4*)(smp[rg] + (size_t)(j) * (NW * 128));         \
             rS[slot][rg][1] = *(const uint4*)(smp[rg] + (size_t)(j) * (NW * 128) + 16);    \
@@ -738,12 +743,15 @@ __device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4
         }
     }
 
-    t12_f32x4 acc[RG];
+    t12_f32x4 acc[NBT][RG];
 #pragma unroll
-    for (int rg = 0; rg < RG; rg++) acc[rg] = t12_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int t = 0; t < NBT; t++)
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) acc[t][rg] = t12_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #define T12_DS_CONSUME(slot)                                                                                 \
     _Pragma("unroll") for (int q = 0; q < 4; q++) {                                                          \
-        const uint4 xa = t12_pair_acts(rX[slot][q]);                                                         \
+        uint4 xa[NBT];                                                                                       \
+        _Pragma("unroll") for (int t = 0; t < NBT; t++) xa[t] = t12_pair_acts(rX[slot][t][q]);               \
         _Pragma("unroll") for (int rg = 0; rg < RG; rg++) {                                                  \
             const uint4 sv = rS[slot][rg][q >> 1];                                                           \
             const uint32_t gq = q == 0 ? rG[slot][rg].x : (q == 1 ? rG[slot][rg].y : (q == 2 ? rG[slot][rg].z : rG[slot][rg].w)); \
@@ -751,8 +759,9 @@ __device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4
             if (q & 1) t12_decode8(sv.z, sv.w, gq, be2, w_);                                                 \
             else t12_decode8(sv.x, sv.y, gq, be2, w_);                                                       \
             const uint4 wv = make_uint4(w_[0], w_[1], w_[2], w_[3]);                                         \
-            acc[rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(t12_bf16x8, xa),            \
-                                                              __builtin_bit_cast(t12_bf16x8, wv), acc[rg], 0, 0, 0); \
+            _Pragma("unroll") for (int t = 0; t < NBT; t++)                                                  \
+                acc[t][rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(t12_bf16x8, xa[t]),  \
+                                                                     __builtin_bit_cast(t12_bf16x8, wv), acc[t][rg], 0, 0, 0); \
         }                                                                                                    \
     }
     int j = 0;
@@ -776,52 +785,62 @@ __device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4
 #undef T12_DS_FETCH
 #undef T12_DS_CONSUME
 
-    // ---- escapes.  Accumulator register r of lane (n, g) is D[batch 4g + r][row n].
+    // ---- escapes.  Accumulator register r of lane (n, g) in batch tile t is D[batch 16t + 4g + r][row n].
     {
-        const uint16_t* xrow[4];
+        const uint16_t* xrow[NBT][4];
 #pragma unroll
-        for (int r = 0; r < 4; r++) xrow[r] = act + (size_t)min(4 * g + r, B - 1) * p.act_stride;
+        for (int t = 0; t < NBT; t++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) xrow[t][r] = act + (size_t)min(16 * t + 4 * g + r, B - 1) * p.act_stride;
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
             if (pcol[rg] >= 0) {
                 const float delta = t12_bf16_to_f32((uint16_t)pcorrect[rg]) - t12_bf16_to_f32((uint16_t)pwrong[rg]);
 #pragma unroll
-                for (int r = 0; r < 4; r++) acc[rg][r] += delta * t12_bf16_to_f32(xrow[r][pcol[rg]]);
+                for (int t = 0; t < NBT; t++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc[t][rg][r] += delta * t12_bf16_to_f32(xrow[t][r][pcol[rg]]);
             }
             for (int e = e_beg[rg] + wave + NW; e < e_end[rg]; e += NW) {        // rows with more than NW escapes
                 const int col = sg.cols[e];
                 const float delta = t12_bf16_to_f32((uint16_t)sg.correct[e]) - t12_bf16_to_f32((uint16_t)sg.wrong[e]);
 #pragma unroll
-                for (int r = 0; r < 4; r++) acc[rg][r] += delta * t12_bf16_to_f32(xrow[r][col]);
+                for (int t = 0; t < NBT; t++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc[t][rg][r] += delta * t12_bf16_to_f32(xrow[t][r][col]);
             }
         }
     }
 
     // ---- the waves' partial tiles, added in wave order; thread (r, l) = (tid / 64, tid % 64) of the first four waves
-    //      finishes element D[batch 4 (l / 16) + r][row l % 16] of every row group
+    //      finishes element D[batch 16 t + 4 (l / 16) + r][row l % 16] of every batch tile and row group
 #pragma unroll
-    for (int rg = 0; rg < RG; rg++) red[rg][wave][lane] = acc[rg];
+    for (int t = 0; t < NBT; t++)
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) red[t * RG + rg][wave][lane] = acc[t][rg];
     __syncthreads();
     if (tid < 256) {
         const int r = tid >> 6, l = tid & 63;
 #pragma unroll
-        for (int rg = 0; rg < RG; rg++) {
-            float v = 0.0f;
+        for (int t = 0; t < NBT; t++)
 #pragma unroll
-            for (int w = 0; w < NW; w++) v += red[rg][w][l][r];
-            const int b = 4 * (l >> 4) + r, row = m0 + 16 * rg + (l & 15);
-            if (b < B && row < M) outp[(size_t)b * sg.out_stride + row] = v;
-        }
+            for (int rg = 0; rg < RG; rg++) {
+                float v = 0.0f;
+#pragma unroll
+                for (int w = 0; w < NW; w++) v += red[t * RG + rg][w][l][r];
+                const int b = 16 * t + 4 * (l >> 4) + r, row = m0 + 16 * rg + (l & 15);
+                if (b < B && row < M) outp[(size_t)b * sg.out_stride + row] = v;
+            }
     }
-    if (DEV && b_first + 16 < b_all) __syncthreads();        // the next 16 batch rows reuse the reduction buffer
+    if (DEV && b_first + 16 * NBT < b_all) __syncthreads();  // the next batch rows reuse the reduction buffer
     }
 }
 
-template <int NW, int D, int RG, bool DEV = false>
+template <int NW, int D, int RG, bool DEV = false, int NBT = 1>
 __global__ __launch_bounds__(NW * 64) void gemm_dense16_kernel(const GemmParams p)
 {
-    __shared__ t12_f32x4 red[RG][NW][64];
-    gemm_dense16_body<NW, D, RG, DEV>(p, red);
+    __shared__ t12_f32x4 red[NBT * RG][NW][64];
+    gemm_dense16_body<NW, D, RG, DEV, NBT>(p, red);
 }
 
 // The same sweep with two sizes of workgroup in one launch.  With RGA row groups per workgroup (its registers allow one
@@ -1298,6 +1317,37 @@ int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_st
         hipLaunchKernelGGL((gemm_rows_kernel<2, 2>), dim3(groups), dim3(512), (size_t)2 * K * 2, st, p);
         T12_CHECK_LAUNCH("t12_gemm(rows)");
         return T12_OK;
+    }
+    if (B > 16 && B <= 32 && K % 128 == 0) {
+        // 17 .. 32 batch rows on tensors of few rows: the same sweep with two batch tiles per weight load and decode.
+        // One round of workgroups takes ~4.5 us + (K / 4096) (3.7 + 0.2 B) us whatever the row count, because every
+        // workgroup reads all B activation rows for its 16 (32) weight rows; the tile kernel below needs a K split and a
+        // reduction launch on such tensors and takes 15-22 us.  Measured at B = 17 / 24 / 32 (tile kernel in brackets):
+        // 4096 x 4096 11.7 / 12.7 / 14.6 us (17.6-18.0), 4096 x 2048 7.6 / 8.5 / 9.1 (15.5), 1024|1024|4096 x 4096 as three
+        // segments 16.7 / 17.8 / 19.1 (20.3-21.1), 8192 x 4096 16.3 / 17.6 / 18.8 (20.6), 4096 x 8192 18.8 / 21.6 / 25.2
+        // (22.5).  Past one round, or with long rows, the tile kernel wins (4096 x 14336: 32 against 42 us at B = 32).
+        const int C = device_cus();
+        int groups16 = 0, sets2 = 0;
+        for (int i = 0; i < nseg; i++) {
+            groups16 += (segs[i].M + 15) / 16;
+            sets2 += (segs[i].M + 31) / 32;
+        }
+        const long long kb = (long long)K * B;
+        const int rg = groups16 <= C && kb <= 4096 * 48 ? 1 : (sets2 <= C && kb <= 5120 * 32 ? 2 : 0);
+        if (rg) {
+            int groups = 0;
+            for (int i = 0; i < nseg; i++) {
+                p.blk_start[i] = groups;
+                groups += (segs[i].M + 16 * rg - 1) / (16 * rg);
+            }
+            p.blk_start[nseg] = groups;
+            p.ksplit = 1;
+            p.kslice = K;
+            if (rg == 2) hipLaunchKernelGGL((gemm_dense16_kernel<8, 2, 2, false, 2>), dim3(groups), dim3(512), 0, st, p);
+            else hipLaunchKernelGGL((gemm_dense16_kernel<8, 2, 1, false, 2>), dim3(groups), dim3(512), 0, st, p);
+            T12_CHECK_LAUNCH("t12_gemm(dense16, two batch tiles)");
+            return T12_OK;
+        }
     }
     if (B <= 16 && K % 128 == 0) {
         // row groups that share an activation load: as many as leave the launch >= 448 workgroups
