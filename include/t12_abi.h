@@ -126,7 +126,8 @@ int t12_gemv_batch(const T12Segment* segs, int nseg, const void* act_bf16, int a
  * out_s[b*out_stride + m] = sum_k dec(W_s[m,k]) * X[b*act_stride + k], bf16 MFMA with
  * fp32 accumulation, escapes exact.  B <= 16 (K a multiple of 128): kernels bound by the
  * weight stream, no K split (B = 2: whole-row waves with two accumulators, v_dot2; else
- * 16-row groups swept whole by eight waves, 16x16x32 MFMA); larger B: 128-row tiles staged
+ * 16-row groups swept whole by eight waves, 16x16x32 MFMA; the same sweep up to B = 32 on
+ * tensors of few, short rows); larger B: 128-row tiles staged
  * through LDS, K split across workgroups when the tiles alone do not fill the chip.  Replaces
  * nv_launch_split12_fused_gemm_async (nvidia_kernels.cu:444) +
  * nv_launch_patches_batch_async (:426) + nv_launch_split12_cublas_batch_async (:550). */
