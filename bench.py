@@ -303,6 +303,16 @@ def run_decode(args, t12, torch, dev):
                     "through the batched prefill; not a mode of the reference" % args.prompt}
         es.close()
 
+    # ---- the batch sizes between 1 and 256 that the reference publishes (docs/TECHNICAL.md:121-126), same lock-step mode
+    batch_sweep = None
+    if args.batch256:
+        batch_sweep = {}
+        for B in (4, 8, 16, 32, 64, 128):
+            eb = eng.new_state(B)
+            msb, _ = decode_loop(eb, B)
+            batch_sweep["b%d" % B] = {"tok_s": round(B * 1e3 / msb, 1), "ms_per_step": round(msb, 4)}
+            eb.close()
+
     result = {
         "metric": "tok/s at B=1 (Llama-3.1-8B shape), greedy decode of a split-12 model; B=256 and decode-GEMV GB/s alongside",
         "value": 1e3 / ms1, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -316,6 +326,7 @@ def run_decode(args, t12, torch, dev):
                    "escape_fraction": n_esc / max(n_weights, 1),
                    "baseline": "57.0 tok/s, Llama 3.1 8B B=1 on RTX 5070 Ti (reference README.md:46)"},
         "b256": b256,
+        "batch_sweep": batch_sweep,
         "gemv_compressed_GBps": plane_bytes / (ms_gemv * 1e-3) / 1e9,
         "gemv_only_ms_per_step": ms_gemv,
         "gemm_layers": gemm_layers,
