@@ -43,6 +43,8 @@ void launch_rope_store_attention(float*, float*, const float*, int8_t*, int8_t*,
                                  int, int, int, int, float, float, int, int, hipStream_t);
 void launch_rope_store_attention_regions(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int16_t*,
                                          const int*, int, int, int, int, float, float, int, int, int, hipStream_t);
+void t12_rope_store_attention_copies(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int16_t*, const int*,
+                                     int, int, int, int, float, float, int, int, hipStream_t);
 void launch_rope_store_attention_partials_regions(float*, float*, const float*, int8_t*, int8_t*, float*, float*, int16_t*,
                                                   const int*, int, int, int, int, float, float, int, const float*, int,
                                                   size_t, int, int, int, hipStream_t);
@@ -97,9 +99,12 @@ struct KvView {
 // RoPE + KV store + attention on either layout
 void rope_store_attention(const KvView& kv, float* q, float* k, const float* v, int8_t* ck, int8_t* cv, float* sk, float* sv,
                           int16_t* out, const int* positions, int position, int n_head, int n_head_kv, int head_dim,
-                          float theta, float scale, int B, hipStream_t st)
+                          float theta, float scale, int B, hipStream_t st, bool copies = false)
 {
-    if (kv.head_major)
+    if (copies && kv.kv_stride == 0)
+        t12_rope_store_attention_copies(q, k, v, ck, cv, sk, sv, out, positions, position, n_head, n_head_kv, head_dim, theta,
+                                        scale, B, kv.head_major, st);
+    else if (kv.head_major)
         launch_rope_store_attention_regions(q, k, v, ck, cv, sk, sv, out, positions, position, n_head, n_head_kv, head_dim,
                                             theta, scale, B, kv.kv_stride, kv.head_major, st);
     else
@@ -397,7 +402,9 @@ KvView kv_view(const InferenceState* state)
 // R > 1, whose positions are in state->d_positions; pos0 = position of the row when R == 1, else the largest
 // position of the rows (a length hint for the attention launch).  Logits: for every row into
 // state->logits (LOGITS_ALL), for the last row only into logits_last (LOGITS_LAST_ROW), or not at all.
-void forward_rows(InferenceState* state, int R, const KvView& kv, int pos0, LogitsMode lm, float* logits_last)
+// copies: the rows are copies of one sequence at one position on a shared cache (the lock-step batch of forward()).
+void forward_rows(InferenceState* state, int R, const KvView& kv, int pos0, LogitsMode lm, float* logits_last,
+                  bool copies = false)
 {
     Model* m = state->model;
     const ModelConfig& c = m->config;
@@ -450,7 +457,7 @@ void forward_rows(InferenceState* state, int R, const KvView& kv, int pos0, Logi
         else
             rope_store_attention(kv, state->q_buf, state->k_buf, state->v_buf, kv.k + kv_off, kv.v + kv_off, kv.sk + sc_off,
                                  kv.sv + sc_off, bf16_a, B == 1 ? nullptr : state->d_positions, pos0, c.n_head, c.n_head_kv,
-                                 head_dim, c.rope_theta, scale, B, st);
+                                 head_dim, c.rope_theta, scale, B, st, copies);
 
         S.o[0] = seg_of(L.wo, res, n);
         if (B > 1) {
@@ -532,7 +539,11 @@ void forward(InferenceState* state, const int* token_ids)
     if (token_ids) (void)hipMemcpyAsync(state->d_tokens, token_ids, B * sizeof(int), hipMemcpyHostToDevice, st);
     if (B > 1) (void)hipMemcpyAsync(state->d_positions, state->positions, B * sizeof(int), hipMemcpyHostToDevice, st);
     // with a position array the scalar position is only the attention launch's length hint: the longest row
-    forward_rows(state, B, kv, B > 1 ? max_pos : state->positions[0], LOGITS_ALL, nullptr);
+    // A batch on one shared cache whose rows stand at one position is the reference's batched mode: copies of one
+    // sequence (inference.cpp:430-435; rows with unlike tokens would overwrite each other's cache slot there too).
+    bool copies = B > 1 && !impl->per_seq;
+    for (int b = 1; b < B && copies; b++) copies = state->positions[b] == state->positions[0];
+    forward_rows(state, B, kv, B > 1 ? max_pos : state->positions[0], LOGITS_ALL, nullptr, copies);
     for (int b = 0; b < B; b++) state->positions[b]++;
 }
 

@@ -1729,14 +1729,18 @@ void launch_rope_store_kv_batch(float* q, float* k, const float* v, int8_t* kv_k
 static void rope_store_attention(float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v, float* scale_k,
                                  float* scale_v, int16_t* output, const int* positions, int position, int n_head,
                                  int n_head_kv, int head_dim, float theta, float scale, int batch_size, int kv_stride,
-                                 int hm, hipStream_t stream)
+                                 int hm, hipStream_t stream, bool copies = false)
 {
     // Fusing pays when every workgroup stores its own cache slot (one sequence, or per-sequence caches) and
     // the launch is small enough to be a chain of latencies: the fused kernel holds prefetched rows in more
     // registers, so only two of its workgroups fit a CU (measured at B = 256 on per-sequence caches: 35 us
     // fused against 26 + 7 us for the two launches at 150 positions, 256 against 248 + 7 us at 2000).  Lock-step
-    // copies on a shared cache (kv_stride = 0, batch > 1) would store the same slot from every workgroup.
-    if (attn_has_fast(n_head, n_head_kv, head_dim) && (batch_size == 1 || (kv_stride != 0 && batch_size * n_head_kv <= 256))) {
+    // copies on a shared cache (kv_stride = 0, batch > 1) store the same slot from every workgroup: the same bytes when
+    // the caller vouches that the rows are copies of one sequence at one position (`copies`), and every workgroup
+    // attends to its own new row either way; without that promise the rows may be the positions of one prompt, which
+    // need each other's stores, and take the two launches.
+    if (attn_has_fast(n_head, n_head_kv, head_dim) &&
+        (batch_size == 1 || ((kv_stride != 0 || copies) && batch_size * n_head_kv <= 256))) {
         AttnFuse fz;
         fz.k_new = k;
         fz.v_new = v;
@@ -1764,6 +1768,18 @@ void launch_rope_store_attention(float* q, float* k, const float* v, int8_t* kv_
 {
     rope_store_attention(q, k, v, kv_k, kv_v, scale_k, scale_v, output, positions, position, n_head, n_head_kv, head_dim,
                          theta, scale, batch_size, kv_stride, 0, stream);
+}
+
+// Library-internal (the engine's lock-step batches): launch_rope_store_attention on ONE shared cache region for rows
+// that are copies of one sequence, all at `position` -- the reference's batched mode (inference.cpp:430-435: every
+// row stores the slot of the shared cache, kernels.hip:785-788).  Small batches then take the fused kernel.
+extern "C" __attribute__((visibility("hidden"))) void t12_rope_store_attention_copies(
+    float* q, float* k, const float* v, int8_t* kv_k, int8_t* kv_v, float* scale_k, float* scale_v, int16_t* output,
+    const int* positions, int position, int n_head, int n_head_kv, int head_dim, float theta, float scale, int batch_size,
+    int region_positions, hipStream_t stream)
+{
+    rope_store_attention(q, k, v, kv_k, kv_v, scale_k, scale_v, output, positions, position, n_head, n_head_kv, head_dim,
+                         theta, scale, batch_size, 0, region_positions, stream, true);
 }
 
 // The same on head-major cache regions: region_positions > 0 rows per (region, KV head), a region laid out
