@@ -31,3 +31,27 @@ def test_one_json_line_with_the_contract_fields():
         assert key in d, key
     assert d["n_gpus"] == 1 and d["steps"] == 3 and d["value"] > 0 and "workload" in d["config"]
     assert "Tokenizer:" in r.stderr                         # the library's report went to standard error
+
+
+def test_traffic_figures_belong_to_the_committed_kernel_sources(tmp_path, monkeypatch):
+    """roofline.traffic comes from profiles/measured_traffic.txt, keyed by the hash of the kernel's source file at the
+    time of the counter runs: the committed lines must name the sources as they are (so the bench prints the figures,
+    not null), and a line whose source has changed since must read as None."""
+    sys.path.insert(0, ROOT)
+    import bench
+    for key in ("gemv_stack_b1", "gemm_gate_up_b256"):
+        v = bench.measured_traffic(key)
+        assert v is not None and 5e7 < v < 5e8, (key, v)
+    assert bench.measured_traffic("no_such_kernel") is None
+    # the same file with one source's hash changed
+    fake = tmp_path / "repo"
+    (fake / "profiles").mkdir(parents=True)
+    (fake / "src").mkdir()
+    (fake / "src" / "k.hip").write_text("kernel v2\n")
+    (fake / "profiles" / "measured_traffic.txt").write_text("# comment\nk 1.0e8 src/k.hip 0123456789abcdef\n")
+    monkeypatch.setattr(bench, "ROOT", str(fake))
+    assert bench.measured_traffic("k") is None
+    import hashlib
+    h = hashlib.sha256(b"kernel v2\n").hexdigest()[:16]
+    (fake / "profiles" / "measured_traffic.txt").write_text("k 1.0e8 src/k.hip %s\n" % h)
+    assert bench.measured_traffic("k") == 1.0e8
