@@ -42,6 +42,7 @@
 
 #include "t12_device.h"
 #include "t12_host.h"
+#include "dense16_plan.h"
 
 // library-internal (hidden: not part of the ABI)
 extern "C" __attribute__((visibility("hidden"))) void t12_glue_release_stream(hipStream_t st);      // glue.hip
@@ -1167,29 +1168,12 @@ int device_cus()
 // tensor is cut into a head, swept rg groups per workgroup in whole rounds, and a tail swept in fewer groups per
 // workgroup, chosen so that the tails of all tensors together are one round.  p holds the launch as gemm_impl set it up
 // (segments, K, B, activations); returns false, with nothing launched, when the plain launch is as good.
-bool launch_dense16_mixed(GemmParams p, int nseg, int rg, int groups16, hipStream_t st)
+bool launch_dense16_mixed(GemmParams p, int nseg, int rg, hipStream_t st)
 {
-    const int C = device_cus();
-    int sets = 0;
-    for (int i = 0; i < nseg; i++) sets += (p.seg[i].M + 16 * rg - 1) / (16 * rg);
-    // one round or less, whole rounds, or a last round that is nearly full: nothing to gain
-    if (2 * nseg > GMAX || sets <= C || sets % C == 0 || (sets % C) * 8 >= C * 7) return false;
-    const int full = (sets / C) * C;                       // workgroups of the whole rounds
-    int a[GMAX], rem[GMAX], rem_total = 0;
-    for (int i = 0; i < nseg; i++) {
-        const int gi = (p.seg[i].M + 15) / 16;
-        a[i] = (int)((long long)full * gi / groups16);     // this tensor's share of the whole rounds
-        if (a[i] * rg > gi) a[i] = gi / rg;
-        rem[i] = gi - a[i] * rg;
-        rem_total += rem[i];
-    }
-    int rgb = (rem_total + C - 1) / C;
-    for (; rgb >= 1 && rgb < rg; rgb++) {
-        int b = 0;
-        for (int i = 0; i < nseg; i++) b += (rem[i] + rgb - 1) / rgb;
-        if (b <= C) break;
-    }
-    if (rgb < 1 || rgb >= rg) return false;
+    int rows[GMAX], head_rows[GMAX];
+    for (int i = 0; i < nseg; i++) rows[i] = p.seg[i].M;
+    const int rgb = t12_plan_dense16_heads(rows, nseg, rg, device_cus(), GMAX, head_rows);
+    if (!rgb) return false;
     // heads first, then tails.  A tail is the same tensor from row 16 rg a on: the row pointers of the escape list hold
     // absolute entry numbers, so only the pointer to them moves; 16 rg a rows of K columns are a whole number of bytes of
     // the nibble plane.
@@ -1199,7 +1183,7 @@ bool launch_dense16_mixed(GemmParams p, int nseg, int rg, int groups16, hipStrea
     p.n_first = 0;
     for (int pass = 0; pass < 2; pass++)
         for (int i = 0; i < nseg; i++) {
-            const int rows_a = min(16 * rg * a[i], src[i].M);
+            const int rows_a = head_rows[i];
             const int m = pass == 0 ? rows_a : src[i].M - rows_a;
             if (m <= 0) continue;
             T12Segment g = src[i];
@@ -1357,7 +1341,7 @@ int gemm_impl(const T12Segment* segs, int nseg, const void* act_bf16, int act_st
         // rows of a padded batch cost no activation traffic, more rows per wave cost registers)
         const int want = B > 8 ? 4 : (B > 4 ? 2 : 1);
         const int rg = groups16 >= 4 * 448 && want >= 4 ? 4 : (groups16 >= 2 * 448 && want >= 2 ? 2 : 1);
-        if (rg > 1 && launch_dense16_mixed(p, nseg, rg, groups16, st)) {
+        if (rg > 1 && launch_dense16_mixed(p, nseg, rg, st)) {
             T12_CHECK_LAUNCH("t12_gemm(dense16, two workgroup sizes)");
             return T12_OK;
         }
