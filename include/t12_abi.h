@@ -151,7 +151,7 @@ int t12_gemm_deferred(const T12Segment* segs, int nseg, const void* act_bf16, in
                       int out_stride, int K, int B, T12GemmPartials* part, void* stream);
 /* out_bf16[b*out_stride + m] = bf16( silu(gate[m,:] . X[b,:]) * (up[m,:] . X[b,:]) ): the gate|up projection with
  * silu_mul_bf16 (engine/kernels.hip:447-459, inference.cpp:327) in the GEMM's epilogue -- no fp32 round trip of
- * the two projections.  Returns 0 when launched, 1 when the shape has no fused kernel (B <= 64, few rows, K not
+ * the two projections.  Returns 0 when launched, 1 when the shape has no fused kernel (B <= 64 other than 5 .. 8, few rows, K not
  * a multiple of 64, base_exp outside 0..240): run t12_gemm on the two segments and launch_silu_mul_bf16_batch
  * then; negative on bad operands. */
 int t12_gemm_swiglu(const T12Segment* gate, const T12Segment* up, const void* act_bf16, int act_stride,

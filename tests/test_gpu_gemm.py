@@ -242,6 +242,41 @@ def test_gemm_swiglu_epilogue_is_bit_identical_to_unfused(t12, synth, M, K, B, p
     assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("M,K,B,p_out", [(14336, 4096, 8, 3e-4), (14336, 4096, 5, 3e-4), (1000, 512, 5, 2e-3), (37, 128, 7, 5e-2),
+                                          (4096, 1280, 6, 2e-2), (2001, 256, 8, 0.0), (520, 2048, 7, 0.2)])
+def test_gemm_swiglu_small_batches_bit_identical_to_unfused(t12, synth, M, K, B, p_out):
+    """5 .. 8 batch rows: t12_gemm_swiglu runs the whole-row sweep with gate rows and the same rows of up in one
+    workgroup and must give t12_gemm on (gate, up) + launch_silu_mul_bf16_batch bit for bit: ragged row counts, one
+    128-column block per row, rows with more escapes than waves, unlike base_exp of gate and up (unlike sigma)."""
+    g = torch.Generator(device=dev())
+
+    def mk(seed, sigma):
+        g.manual_seed(seed)
+        w = torch.randn((M, K), generator=g, device=dev()) * sigma
+        if p_out > 0:
+            m = torch.rand((M, K), generator=g, device=dev()) < p_out
+            w = torch.where(m, torch.randn((M, K), generator=g, device=dev()) * 8, w)
+        return t12.pack_device(w.to(torch.bfloat16))
+
+    gate, up = mk(1, 0.02), mk(2, 0.3)
+    if p_out < 1e-2:                                          # (many outliers pull both windows to the same place)
+        assert gate.segment(None).base_exp != up.segment(None).base_exp
+    g.manual_seed(3)
+    X = torch.randn((B, K), generator=g, device=dev()).to(torch.bfloat16).view(torch.int16)
+    st = t12.current_stream()
+    og, ou = t12.gemm([gate, up], X)
+    want = torch.empty((B, M), dtype=torch.int16, device=dev())
+    t12.lib.launch_silu_mul_bf16_batch(og.data_ptr(), ou.data_ptr(), want.data_ptr(), M, B, st)
+    got = torch.full((B, M + 8), -1, dtype=torch.int16, device=dev())
+    sg = t12._seg_array([gate.segment(None)])
+    su = t12._seg_array([up.segment(None)])
+    rc = t12.lib.t12_gemm_swiglu(sg, su, X.data_ptr(), K, K, B, got.data_ptr(), M + 8, st)
+    torch.cuda.synchronize()
+    assert rc == 0, t12.lib.t12_last_error()
+    assert torch.equal(got[:, :M], want)
+    assert bool((got[:, M:] == -1).all())                     # nothing written past the last row
+
+
 def test_gemm_swiglu_declines_shapes_without_a_fused_kernel(t12, oracle, synth):
     p = oracle.pack(synth.weights_llm(512, 256, seed=1))
     dt = t12.DeviceTensor12.from_packed(p, dev())
@@ -250,7 +285,9 @@ def test_gemm_swiglu_declines_shapes_without_a_fused_kernel(t12, oracle, synth):
     s1 = t12._seg_array([dt.segment(None)])
     st = t12.current_stream()
     assert t12.lib.t12_gemm_swiglu(s1, s1, X.data_ptr(), 256, 256, 256, out.data_ptr(), 512, st) == 1      # few rows
-    assert t12.lib.t12_gemm_swiglu(s1, s1, X.data_ptr(), 256, 256, 64, out.data_ptr(), 512, st) == 1       # small batch
+    assert t12.lib.t12_gemm_swiglu(s1, s1, X.data_ptr(), 256, 256, 64, out.data_ptr(), 512, st) == 1       # 9 .. 64 rows
+    assert t12.lib.t12_gemm_swiglu(s1, s1, X.data_ptr(), 256, 256, 16, out.data_ptr(), 512, st) == 1
+    assert t12.lib.t12_gemm_swiglu(s1, s1, X.data_ptr(), 256, 256, 4, out.data_ptr(), 512, st) == 1        # up to 4 rows
     assert t12.lib.t12_gemm_swiglu(s1, s1, X.data_ptr(), 256, 256, 256, out.data_ptr(), 100, st) == -1     # out_stride < M
 
 

@@ -668,14 +668,20 @@ __global__ __launch_bounds__(256) void gemm_general_kernel(const GemmParams p)
 // the segment's group has dev_counts[g] batch rows starting dev_base[g] rows into the activations and the outputs; a
 // workgroup of a group without rows exits at once, one of a group above 16 rows sweeps its weight rows once per 16.
 // ---------------------------------------------------------------------------
-template <int NW, int D, int RG, bool DEV, int NBT = 1>
+// SWI (a launch of ONE gate / up pair, segments 0 and 1 of equal row count): the first RG / 2 row groups of a workgroup
+// are 16 RG / 2 rows of gate, the others the same rows of up, and the thread that finishes an element of both stores
+// bf16( silu(gate) * up ) to out_bf16 instead of the two sums (the arithmetic of silu_mul_kernel, so the result is
+// what t12_gemm + launch_silu_mul_bf16_batch give, bit for bit).
+template <int NW, int D, int RG, bool DEV, int NBT = 1, bool SWI = false>
 __device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4 (*red)[NW][64])
 {
+    static_assert(!SWI || (RG % 2 == 0 && !DEV && NBT == 1), "the SwiGLU form pairs row groups");
+    constexpr int RH = SWI ? RG / 2 : RG;             // row groups of one tensor
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, g = lane >> 4;
 
     const int blk = blockIdx.x;
-    const int s = find_segment(p, blk);
+    const int s = SWI ? 0 : find_segment(p, blk);
     const T12Segment& sg = p.seg[s];
     const int M = sg.M, K = p.K;
     // DEV: the group's rows from the device tables; otherwise one pass over the launch's B <= 16 rows
@@ -685,14 +691,19 @@ __device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4
     const int B = DEV ? min(16 * NBT, b_all - b_first) : p.B;
     const uint16_t* const act = DEV ? p.act + (size_t)(row_base + b_first) * p.act_stride : p.act;
     float* const outp = DEV ? sg.out + (size_t)(row_base + b_first) * sg.out_stride : sg.out;
-    const int m0 = (blk - p.blk_start[s]) * (16 * RG);               // RG groups of 16 rows share every activation load
+    const int m0 = (blk - p.blk_start[s]) * (16 * RH);               // RG groups of 16 rows share every activation load
     const int nblk = K >> 7;                          // 128-column blocks per row
     const int mine = nblk > wave ? (nblk - wave + NW - 1) / NW : 0;      // blocks of this wave
     // A wave without a block (K < NW * 128) still issues the first D fetches below and drops them: it aims them at
     // block 0, because its own first block would lie past the end of the row -- and, in the last rows of a plane or
     // of the activations, past the end of the allocation.
     const int wblk = mine > 0 ? wave : 0;
-    const uint32_t be2 = t12_opaque(((uint32_t)sg.base_exp << 7) | ((uint32_t)sg.base_exp << 23));
+    uint32_t be2r[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+        const int be = p.seg[SWI && rg >= RH ? 1 : s].base_exp;
+        be2r[rg] = t12_opaque(((uint32_t)be << 7) | ((uint32_t)be << 23));
+    }
 
     // CSR pointers of this lane's rows (used after the stream)
     int e_beg[RG], e_end[RG];
@@ -700,15 +711,16 @@ __device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4
     const uint8_t* grp[RG];
 #pragma unroll
     for (int rg = 0; rg < RG; rg++) {
-        const int row = m0 + 16 * rg + n;
+        const T12Segment& sr = p.seg[SWI && rg >= RH ? 1 : s];      // (SWI: gate for the first half, up for the second)
+        const int row = m0 + 16 * (rg % RH) + n;
         e_beg[rg] = e_end[rg] = 0;
-        if (sg.row_off && row < M) {
-            e_beg[rg] = sg.row_off[row];
-            e_end[rg] = sg.row_off[row + 1];
+        if (sr.row_off && row < M) {
+            e_beg[rg] = sr.row_off[row];
+            e_end[rg] = sr.row_off[row + 1];
         }
         const size_t e0 = (size_t)min(row, M - 1) * K;              // rows past the end are clamped, never stored
-        smp[rg] = sg.sm + e0 + 32 * g + (size_t)wblk * 128;
-        grp[rg] = sg.gr + (e0 >> 1) + 16 * g + (size_t)wblk * 64;
+        smp[rg] = sr.sm + e0 + 32 * g + (size_t)wblk * 128;
+        grp[rg] = sr.gr + (e0 >> 1) + 16 * g + (size_t)wblk * 64;
     }
     const uint16_t* xp[NBT];                          // NBT tiles of 16 batch rows share every weight load and decode
 #pragma unroll
@@ -738,9 +750,10 @@ __device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4
         pcol[rg] = -1;
         pcorrect[rg] = pwrong[rg] = 0;
         if (e_beg[rg] + wave < e_end[rg]) {
-            pcol[rg] = sg.cols[e_beg[rg] + wave];
-            pcorrect[rg] = sg.correct[e_beg[rg] + wave];
-            pwrong[rg] = sg.wrong[e_beg[rg] + wave];
+            const T12Segment& sr = p.seg[SWI && rg >= RH ? 1 : s];
+            pcol[rg] = sr.cols[e_beg[rg] + wave];
+            pcorrect[rg] = sr.correct[e_beg[rg] + wave];
+            pwrong[rg] = sr.wrong[e_beg[rg] + wave];
         }
     }
 
@@ -757,8 +770,8 @@ __device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4
             const uint4 sv = rS[slot][rg][q >> 1];                                                           \
             const uint32_t gq = q == 0 ? rG[slot][rg].x : (q == 1 ? rG[slot][rg].y : (q == 2 ? rG[slot][rg].z : rG[slot][rg].w)); \
             uint32_t w_[4];                                                                                  \
-            if (q & 1) t12_decode8(sv.z, sv.w, gq, be2, w_);                                                 \
-            else t12_decode8(sv.x, sv.y, gq, be2, w_);                                                       \
+            if (q & 1) t12_decode8(sv.z, sv.w, gq, be2r[rg], w_);                                            \
+            else t12_decode8(sv.x, sv.y, gq, be2r[rg], w_);                                                  \
             const uint4 wv = make_uint4(w_[0], w_[1], w_[2], w_[3]);                                         \
             _Pragma("unroll") for (int t = 0; t < NBT; t++)                                                  \
                 acc[t][rg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(t12_bf16x8, xa[t]),  \
@@ -802,9 +815,10 @@ __device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4
 #pragma unroll
                     for (int r = 0; r < 4; r++) acc[t][rg][r] += delta * t12_bf16_to_f32(xrow[t][r][pcol[rg]]);
             }
+            const T12Segment& sr = p.seg[SWI && rg >= RH ? 1 : s];
             for (int e = e_beg[rg] + wave + NW; e < e_end[rg]; e += NW) {        // rows with more than NW escapes
-                const int col = sg.cols[e];
-                const float delta = t12_bf16_to_f32((uint16_t)sg.correct[e]) - t12_bf16_to_f32((uint16_t)sg.wrong[e]);
+                const int col = sr.cols[e];
+                const float delta = t12_bf16_to_f32((uint16_t)sr.correct[e]) - t12_bf16_to_f32((uint16_t)sr.wrong[e]);
 #pragma unroll
                 for (int t = 0; t < NBT; t++)
 #pragma unroll
@@ -825,12 +839,19 @@ __device__ __forceinline__ void gemm_dense16_body(const GemmParams& p, t12_f32x4
 #pragma unroll
         for (int t = 0; t < NBT; t++)
 #pragma unroll
-            for (int rg = 0; rg < RG; rg++) {
-                float v = 0.0f;
+            for (int rg = 0; rg < RH; rg++) {
+                float v = 0.0f, u = 0.0f;
 #pragma unroll
                 for (int w = 0; w < NW; w++) v += red[t * RG + rg][w][l][r];
+                if (SWI) {
+#pragma unroll
+                    for (int w = 0; w < NW; w++) u += red[RH + rg][w][l][r];
+                }
                 const int b = 16 * t + 4 * (l >> 4) + r, row = m0 + 16 * rg + (l & 15);
-                if (b < B && row < M) outp[(size_t)b * sg.out_stride + row] = v;
+                if (SWI) {
+                    if (b < B && row < M)
+                        p.out_bf16[(size_t)b * p.out_bf16_ld + row] = t12_f32_to_bf16(v / (1.0f + expf(-v)) * u);
+                } else if (b < B && row < M) outp[(size_t)b * sg.out_stride + row] = v;
             }
     }
     if (DEV && b_first + 16 * NBT < b_all) __syncthreads();  // the next batch rows reuse the reduction buffer
@@ -842,6 +863,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_dense16_kernel(const GemmParams 
 {
     __shared__ t12_f32x4 red[NBT * RG][NW][64];
     gemm_dense16_body<NW, D, RG, DEV, NBT>(p, red);
+}
+
+// The sweep over one gate / up pair with the SiLU * mul in its last step (blockIdx.x counts sets of 16 RG / 2 rows).
+template <int NW, int D, int RG>
+__global__ __launch_bounds__(NW * 64) void gemm_dense16_swiglu_kernel(const GemmParams p)
+{
+    __shared__ t12_f32x4 red[RG][NW][64];
+    gemm_dense16_body<NW, D, RG, false, 1, true>(p, red);
 }
 
 // The same sweep with two sizes of workgroup in one launch.  With RGA row groups per workgroup (its registers allow one
@@ -1115,6 +1144,37 @@ int t12_gemm_swiglu(const T12Segment* gate, const T12Segment* up, const void* ac
         T12_REQUIRE(!g->row_off || (g->cols && g->correct && g->wrong), "t12_gemm_swiglu: row_off without lists");
         T12_REQUIRE(g->base_exp >= -1 && g->base_exp <= 254, "t12_gemm_swiglu: base_exp %d out of range", g->base_exp);
         if (g->base_exp < 0 || g->base_exp > 240) fast = false;
+    }
+    // 5 .. 8 batch rows: the whole-row sweep over 32 rows of gate and the same rows of up per workgroup.  Measured on
+    // 2 x 14336 x 4096 against t12_gemm + launch_silu_mul_bf16_batch: 43.6 / 44.7 us at B = 5 / 8 against 44.3 / 47.1; no
+    // gain at B <= 4 (43.9 against 44.2; B = 2: 44.5 against 39) nor above 8, where the unfused launch balances its
+    // last round (B = 9 / 12 / 16: 45.3 / 46.7 / 49.0 against 45.5 / 46.6 / 48.4).
+    bool sweep = K % 128 == 0 && act_stride % 8 == 0 && (uintptr_t)act_bf16 % 16 == 0 && B >= 5 && B <= 8;
+    for (const T12Segment* g : two)
+        if (g->base_exp < 0 || g->base_exp > 240) sweep = false;
+    if (sweep) {
+        const int rg = 4;
+        GemmParams p;
+        p.seg[0] = *gate;
+        p.seg[1] = *up;
+        p.nseg = 2;
+        p.K = K;
+        p.B = B;
+        p.act_stride = act_stride;
+        p.act = (const uint16_t*)act_bf16;
+        p.ws = nullptr;
+        p.ksplit = 1;
+        p.kslice = K;
+        p.m_total = gate->M;
+        const int sets = (gate->M + 8 * rg - 1) / (8 * rg);
+        p.blk_start[0] = 0;
+        p.blk_start[1] = p.blk_start[2] = sets;
+        p.out_bf16 = (uint16_t*)out_bf16;
+        p.out_bf16_ld = out_stride;
+        hipStream_t st = (hipStream_t)stream;
+        hipLaunchKernelGGL((gemm_dense16_swiglu_kernel<8, 2, 4>), dim3(sets), dim3(512), 0, st, p);
+        T12_CHECK_LAUNCH("t12_gemm_swiglu(dense16)");
+        return T12_OK;
     }
     const int tiles = (gate->M + TM / 2 - 1) / (TM / 2);
     const int btiles = B > 128 ? (B + 255) / 256 : 1;
